@@ -1,0 +1,265 @@
+"""Pins the CPU oracle (oracle/nsa_oracle.py) WITHOUT using its own formulas: closed forms, library routines,
+brute-force loops on tiny inputs, and the committed golden vectors of the upstream torch_topk."""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import nsa_oracle as O
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden", "topk_golden.npz")
+
+
+def rand(*shape, seed=0, dtype=torch.float64):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g, dtype=torch.float32).to(dtype)
+
+
+# ------------------------------------------------------------------ lengths
+@pytest.mark.parametrize("L,y", [(0, 0), (31, 0), (32, 1), (47, 1), (48, 2), (63, 2), (64, 3), (4096, 255),
+                                 (65536, 4095)])
+def test_lengths_hand_cases(L, y):
+    m = O.seq_lengths([0, L])
+    assert m["y_seqlens"] == [y]
+    assert m["k_seqlens"] == [(L + 63) // 64]
+
+
+# ------------------------------------------------------------------ pooling / im2col
+@pytest.mark.parametrize("lens", [[200], [31, 32, 47, 48, 100], [0, 64, 5]])
+def test_pooling_closed_forms(lens):
+    cu = np.concatenate([[0], np.cumsum(lens)])
+    T = int(cu[-1])
+    x = rand(T, 2, 8, seed=1)
+    y = O.mean_pooling(x, cu)
+    blk = O.construct_block(x, cu)
+    assert torch.equal(blk.mean(-2), y)
+    outs = []
+    for b, L in enumerate(lens):
+        xs = x[cu[b]:cu[b + 1]]
+        if L < 32:
+            continue
+        # library routine: avg_pool1d over the token axis
+        p = F.avg_pool1d(xs.permute(1, 2, 0).reshape(1, -1, L), kernel_size=32, stride=16)
+        outs.append(p.reshape(2, 8, -1).permute(2, 0, 1))
+        # unfold closed form for im2col
+        u = xs.unfold(0, 32, 16)  # [y,H,D,32]
+        assert torch.equal(u.permute(0, 1, 3, 2), blk[sum(max((l - 32) // 16 + 1, 0) for l in lens[:b]):][:u.shape[0]])
+    ref = torch.cat(outs, 0) if outs else x.new_zeros(0, 2, 8)
+    assert y.shape == ref.shape
+    assert torch.allclose(y, ref, atol=1e-12)
+
+
+def test_learned_compression_closed_form():
+    x = rand(80, 2, 4, seed=2)
+    w = rand(8, 32 * 4, seed=3)
+    out = O.compress(x, [0, 80], "sigmoid-mul", w)
+    # brute force, window by window
+    for i in range(out.shape[0]):
+        for h in range(2):
+            flat = x[16 * i:16 * i + 32, h].reshape(-1)
+            hid = w @ flat
+            ref = torch.sigmoid(hid[:4]) * hid[4:]
+            assert torch.allclose(out[i, h], ref, atol=1e-12)
+    lin = O.compress(x, [0, 80], "linear", w[:4])
+    assert torch.allclose(lin[1, 1], w[:4] @ x[16:48, 1].reshape(-1), atol=1e-12)
+    sw = O.compress(x, [0, 80], "swiglu", w)
+    hid = w @ x[0:32, 0].reshape(-1)
+    assert torch.allclose(sw[0, 0], F.silu(hid[:4]) * hid[4:], atol=1e-12)
+
+
+# ------------------------------------------------------------------ attention branches vs SDPA
+def sdpa(q, k, v, mask, scale):
+    """q [L,QH,D] k,v [M,KH,*] mask [L,M] or [KH,L,M] -> o via torch's library attention."""
+    QH, KH = q.shape[1], k.shape[1]
+    G = QH // KH
+    qq = q.permute(1, 0, 2)[None]
+    kk = k.repeat_interleave(G, 1).permute(1, 0, 2)[None]
+    vv = v.repeat_interleave(G, 1).permute(1, 0, 2)[None]
+    if mask.dim() == 3:
+        mask = mask.repeat_interleave(G, 0)[None]
+    o = F.scaled_dot_product_attention(qq, kk, vv, attn_mask=mask, scale=scale)
+    return o[0].permute(1, 0, 2)
+
+
+def test_cmp_attn_vs_sdpa_and_lse():
+    L, QH, KH, D = 150, 4, 2, 16
+    q, k, v = rand(L, QH, D, seed=4), rand(L, KH, D, seed=5), rand(L, KH, D, seed=6)
+    cu = [0, L]
+    ck, cv = O.mean_pooling(k, cu), O.mean_pooling(v, cu)
+    o, lse2 = O.cmp_attn(q, ck, cv, cu)
+    y = ck.shape[0]
+    mask = torch.arange(L)[:, None] >= (torch.arange(y) * 16 + 31)[None, :]
+    ref = sdpa(q[31:], ck, cv, mask[31:], D ** -0.5)
+    assert torch.allclose(o[31:], ref, atol=1e-10)
+    assert torch.all(o[:31] == 0) and torch.all(lse2[:, :31] == 0)
+    assert lse2.shape == (QH, L)
+    # brute force lse (log2 units) for one entry
+    t, h = 100, 3
+    s = torch.stack([(q[t, h] * ck[i, h // 2]).sum() * D ** -0.5 for i in range(y) if t >= 16 * i + 31])
+    assert abs(float(lse2[h, t]) - float(torch.log2(torch.exp(s).sum()))) < 1e-10
+
+
+def test_swa_vs_sdpa_band_mask():
+    lens = [700, 90]
+    cu = [0, 700, 790]
+    QH, KH, D = 4, 2, 8
+    q, k, v = rand(790, QH, D, seed=7), rand(790, KH, D, seed=8), rand(790, KH, D, seed=9)
+    o, lse2 = O.swa(q, k, v, cu, 512)
+    for b in range(2):
+        a, e = cu[b], cu[b + 1]
+        L = e - a
+        t = torch.arange(L)
+        d = t[:, None] - t[None, :]
+        ref = sdpa(q[a:e], k[a:e], v[a:e], (d >= 0) & (d <= 512), D ** -0.5)
+        assert torch.allclose(o[a:e], ref, atol=1e-10)
+    # brute-force count: row 600 of seq 0 sees exactly 513 keys, row 10 sees 11
+    t, h = 600, 1
+    s = torch.stack([(q[t, h] * k[j, 0]).sum() * D ** -0.5 for j in range(t - 512, t + 1)])
+    assert abs(float(lse2[t, h]) - float(torch.log2(torch.exp(s).sum()))) < 1e-10
+
+
+def test_slc_attn_brute_force():
+    L, QH, KH, D = 300, 4, 2, 8
+    q, k, v = rand(L, QH, D, seed=10), rand(L, KH, D, seed=11), rand(L, KH, D, seed=12)
+    cu = [0, L]
+    cfg = O.OracleConfig(top_n=3, num_init_blocks=1, num_local_blocks=1)
+    ck = O.mean_pooling(k, cu)
+    _, lse = O.cmp_attn(q, ck, ck, cu)
+    topk = O.slc_topk(q, ck, lse, cu, cfg)
+    o, lse2 = O.slc_attn(q, k, v, topk, cu, 64)
+    for t in [0, 5, 63, 64, 130, 299]:
+        for h in range(QH):
+            kh = h // 2
+            nv = min(3, t // 64 + 1)
+            keys = sorted({j * 64 + r for j in topk[kh, t, :nv].tolist() for r in range(64) if j * 64 + r <= t})
+            s = torch.stack([(q[t, h] * k[j, kh]).sum() * D ** -0.5 for j in keys])
+            p = torch.softmax(s, 0)
+            ref = sum(p[i] * v[j, kh] for i, j in enumerate(keys))
+            assert torch.allclose(o[t, h], ref, atol=1e-10)
+            assert abs(float(lse2[t, h]) - float(torch.log2(torch.exp(s).sum()))) < 1e-10
+
+
+# ------------------------------------------------------------------ selection: golden vectors + brute force
+def _golden_cases():
+    z = np.load(GOLD)
+    for ci in range(int(z["n_cases"])):
+        yield ci, z[f"c{ci}_params"], z[f"c{ci}_q"], z[f"c{ci}_ck"], z[f"c{ci}_topk"]
+
+
+def test_topk_matches_upstream_golden_vectors():
+    n_checked = 0
+    for ci, prm, q, ck, gold in _golden_cases():
+        T, QH, KH, D, K, S, Bs, N, I, Lc, seed = [int(v) for v in prm]
+        cfg = O.OracleConfig(kernel_size=K, stride=S, block_size=Bs, top_n=N, num_init_blocks=I, num_local_blocks=Lc)
+        q, ck = torch.from_numpy(q), torch.from_numpy(ck)
+        topk, imps = O.slc_topk(q, ck, None, [0, T], cfg, return_importance=True)
+        gold = torch.from_numpy(gold)
+        assert topk.shape == gold.shape == (KH, T, N)
+        for kh in range(KH):
+            for t in range(T):
+                nv = min(N, t // Bs + 1)
+                a = sorted(topk[kh, t, :nv].tolist())
+                b = sorted(gold[kh, t, :nv].tolist())
+                forced = set(range(I)) | {t // Bs - i for i in range(Lc) if t // Bs - i >= 0}
+                if a != b and nv < len(forced):
+                    # fewer slots than forced blocks: upstream marks all of them 99999 and torch.topk picks an
+                    # arbitrary subset; the device rule (init slots first, then local) is checked separately
+                    assert set(b) <= forced and set(a) <= forced, (ci, kh, t, a, b)
+                elif a != b:  # only exact-score ties may differ (upstream uses torch.topk, unordered on ties)
+                    diff = set(a) ^ set(b)
+                    vals = [float(imps[0][kh, t, j]) for j in diff]
+                    assert max(vals) - min(vals) < 1e-6, (ci, kh, t, a, b)
+                assert all(int(v) == 99999999 for v in gold[kh, t, nv:].tolist())
+                n_checked += 1
+    assert n_checked > 3000
+
+
+def test_select_slot_order_and_invariants():
+    # brute force restatement of the device selector's slot order on a tiny case
+    T, KH, nbk = 400, 1, 7
+    g = torch.Generator().manual_seed(0)
+    imp = torch.rand(KH, T, nbk, generator=g, dtype=torch.float64)
+    t_abs = torch.arange(T)
+    imp = torch.where((torch.arange(nbk)[None, :] <= (t_abs // 64)[:, None])[None], imp, torch.zeros_like(imp))
+    out = O.select_blocks(imp, t_abs, 64, 5, 1, 2, ignore_index=-7)
+    for t in range(T):
+        nk = t // 64
+        row = imp[0, t].clone()
+        exp = [-7] * 5
+        if 0 <= nk:
+            exp[0] = 0
+        row[0] = -1
+        for i in range(2):
+            if 1 + i <= nk:
+                exp[1 + i] = nk - i
+            if nk - i >= 0:
+                row[nk - i] = -1
+        for s in range(3, min(5, nk + 1)):
+            j = int(torch.argmax(row))
+            exp[s] = j
+            row[j] = -1
+        assert out[0, t].tolist() == exp, (t, out[0, t].tolist(), exp)
+        valid = [v for v in exp if v != -7]
+        assert len(valid) == min(5, nk + 1) and len(set(valid)) == len(valid) and all(0 <= v <= nk for v in valid)
+
+
+def test_overlap_weights():
+    assert O.overlap_weights(32, 16, 64) == [1, 2, 2, 2, 1]
+    # sum of weights * stride = tokens of the block counted with multiplicity kernel/stride
+    for K, S, Bs in [(32, 16, 64), (64, 32, 128), (32, 8, 32), (32, 32, 64)]:
+        assert sum(O.overlap_weights(K, S, Bs)) * S == Bs * (K // S)
+
+
+# ------------------------------------------------------------------ combine + gradients
+def test_combine_closed_form():
+    a, b, c, w = rand(5, 2, 4, seed=1), rand(5, 2, 4, seed=2), rand(5, 2, 4, seed=3), rand(5, 2, 3, seed=4)
+    o = O.combine(a, b, c, w)
+    t, h = 3, 1
+    ref = a[t, h] / (1 + math.exp(-w[t, h, 0])) + b[t, h] / (1 + math.exp(-w[t, h, 1])) + c[t, h] / (
+        1 + math.exp(-w[t, h, 2]))
+    assert torch.allclose(o[t, h], ref, atol=1e-12)
+
+
+def test_nsa_forward_gradcheck_fp64():
+    L, QH, KH, D = 100, 2, 1, 4
+    cfg = O.OracleConfig(top_n=2, num_init_blocks=1, num_local_blocks=1, window_size=20)
+    q, k, v, w = [rand(*s, seed=i).requires_grad_() for i, s in
+                  enumerate([(L, QH, D), (L, KH, D), (L, KH, D), (L, QH, 3)])]
+    cu = [0, 60, 100]
+    with torch.no_grad():
+        topk = O.nsa_forward(q, k, v, w, cu, cfg, return_parts=True)[1]["topk"]
+    fn = lambda q_, k_, v_, w_: O.nsa_forward(q_, k_, v_, w_, cu, cfg, topk=topk)
+    assert torch.autograd.gradcheck(fn, (q, k, v, w), eps=1e-6, atol=1e-5, rtol=1e-4, nondet_tol=0)
+
+
+def test_paged_oracle_equals_contiguous():
+    # decode == last row of the contiguous forward; chunked prefill rows == contiguous rows
+    L, QH, KH, D, page = 700, 4, 2, 8, 128
+    cfg = O.OracleConfig(top_n=4, window_size=100)
+    q, k, v, w = rand(L, QH, D, seed=1), rand(L, KH, D, seed=2), rand(L, KH, D, seed=3), rand(L, QH, 3, seed=4)
+    o_ref, parts = O.nsa_forward(q, k, v, w, [0, L], cfg, return_parts=True)
+    P = 16
+    perm = torch.randperm(P, generator=torch.Generator().manual_seed(0))
+    kc, vc = torch.zeros(P, page, KH, D, dtype=torch.float64), torch.zeros(P, page, KH, D, dtype=torch.float64)
+    npg = (L + page - 1) // page
+    bt = perm[:npg][None].to(torch.int32)
+    cbt = perm[npg:npg + 1][None].to(torch.int32)
+    kf, vf = kc.view(-1, KH, D), vc.view(-1, KH, D)
+    for n in range(L):
+        kf[int(bt[0, n // page]) * page + n % page] = k[n]
+        vf[int(bt[0, n // page]) * page + n % page] = v[n]
+    y = (L - 32) // 16 + 1
+    slots = torch.tensor([int(cbt[0, i // page]) * page + i % page for i in range(y)], dtype=torch.int32)
+    ctx = torch.tensor([L], dtype=torch.int32)
+    ycu = torch.tensor([0, y], dtype=torch.int32)
+    O.paged_pool_prefill(kc, ycu, ctx, bt, slots)
+    O.paged_pool_prefill(vc, ycu, ctx, bt, slots)
+    assert torch.allclose(O.gather_rows(kc, cbt[0], y), parts["cmp_k"], atol=1e-12)
+    xcu = torch.tensor([0, 200], dtype=torch.int32)
+    o_chunk = O.nsa_paged_forward(q[500:], kc, vc, w[500:], xcu, ctx, bt, cbt, cfg)
+    assert torch.allclose(o_chunk, o_ref[500:], atol=1e-10)
+    o_dec = O.nsa_paged_forward(q[-1:], kc, vc, w[-1:], torch.tensor([0, 1]), ctx, bt, cbt, cfg)
+    assert torch.allclose(o_dec, o_ref[-1:], atol=1e-10)
