@@ -1,0 +1,95 @@
+/* C ABI of libnsa_hip.so: MI355X (gfx950) kernels for the Native-Sparse-Attention hot path.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless stated otherwise; tensors are bf16 unless stated otherwise;
+ *   - strides are in ELEMENTS; "_st" = token/row stride, "_sh" = head stride; the channel dim is contiguous;
+ *   - packed variable-length batches: x_cu [B+1] int32 token offsets, y_cu [B+1] int32 compressed-row offsets
+ *     (y_len = max((L-kernel)/stride+1, 0) per sequence);
+ *   - `stream` is a hipStream_t passed as void*; kernels are enqueued, never synchronised;
+ *   - return value: 0 = ok, otherwise an error code; nsa_last_error() gives the message (thread local);
+ *   - log-sum-exp outputs are in log2 units (m + log2(l)), as upstream stores them.
+ * Citations name the upstream (mdy666/Scalable-Flash-Native-Sparse-Attention) interface each entry replaces.
+ */
+#ifndef NSA_HIP_H
+#define NSA_HIP_H
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* nsa_last_error(void);
+int nsa_abi_version(void);
+
+/* flash_nsa/ops/compress_kv.py:335-366 mean_pooling_fwd */
+int nsa_mean_pool_fwd(const void* x, int64_t x_st, int64_t x_sh, void* y, int64_t y_st, int64_t y_sh,
+                      const int32_t* x_cu, const int32_t* y_cu, int B, int y_maxlen, int H, int D, int kernel_size,
+                      int stride, void* stream);
+/* flash_nsa/ops/compress_kv.py:368-399 mean_pooling_bwd; dx fp32 (optionally accumulated into) or bf16 */
+int nsa_mean_pool_bwd(const void* dy, int64_t dy_st, int64_t dy_sh, void* dx, int64_t dx_st, int64_t dx_sh,
+                      int dx_is_f32, int accumulate, const int32_t* x_cu, const int32_t* y_cu, int B, int x_maxlen,
+                      int H, int D, int kernel_size, int stride, void* stream);
+/* flash_nsa/ops/compress_kv.py:126-170 construct_block_fwd; y contiguous [y_len,H,kernel,D] */
+int nsa_construct_block_fwd(const void* x, int64_t x_st, int64_t x_sh, void* y, const int32_t* x_cu,
+                            const int32_t* y_cu, int B, int y_maxlen, int H, int D, int kernel_size, int stride,
+                            void* stream);
+/* flash_nsa/ops/compress_kv.py:172-218 construct_block_bwd */
+int nsa_construct_block_bwd(const void* dblock, void* dx, int64_t dx_st, int64_t dx_sh, int dx_is_f32,
+                            int accumulate, const int32_t* x_cu, const int32_t* y_cu, int B, int x_maxlen, int H,
+                            int D, int kernel_size, int stride, void* stream);
+/* flash_nsa/ops/act.py:175-208 sigmoid_mul_fwd/bwd (act 0) and :60-100 swiglu_fwd/bwd (act 1);
+ * x [N,2d] = gate|up, y [N,d], dx [N,2d] = dgate|dup (dx may alias x) */
+int nsa_glu_fwd(const void* x, void* y, int64_t N, int d, int act, void* stream);
+int nsa_glu_bwd(const void* x, const void* dy, void* dx, int64_t N, int d, int act, void* stream);
+
+/* flash_nsa/ops/combine.py:114-144 combine_fwd */
+int nsa_combine_fwd(const void* a, const void* b, const void* c, int64_t i_st, int64_t i_sh, const void* w,
+                    int64_t w_st, int64_t w_sh, void* o, int64_t o_st, int64_t o_sh, int64_t T, int H, int D,
+                    void* stream);
+/* flash_nsa/ops/combine.py:146-177 combine_bwd; da/db/dc contiguous [T,H,D], dw [T,H,3];
+ * delta3 (optional, fp32 [3,T,H]) receives rowsum(x_k * dx_k) for the three branches */
+int nsa_combine_bwd(const void* a, const void* b, const void* c, int64_t i_st, int64_t i_sh, const void* w,
+                    int64_t w_st, int64_t w_sh, const void* dy, int64_t dy_st, int64_t dy_sh, void* da, void* db,
+                    void* dc, void* dw, float* delta3, int64_t T, int H, int D, void* stream);
+/* flash_nsa/ops/compress_attn.py:160-184 _bwd_preprocess: delta[T,H] fp32 = rowsum(o*do) */
+int nsa_delta(const void* o, int64_t o_st, int64_t o_sh, const void* dO, int64_t d_st, int64_t d_sh, float* delta,
+              int64_t T, int H, int D, void* stream);
+
+/* flash_nsa/ops/compress_attn.py:531-592 cmp_attn_fwd; lse addressed tok*lse_st + head*lse_sh */
+int nsa_cmp_attn_fwd(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr, int64_t ck_sh,
+                     const void* cv, int64_t cv_sr, int64_t cv_sh, void* o, int64_t o_st, int64_t o_sh, float* lse,
+                     int64_t lse_st, int64_t lse_sh, const int32_t* x_cu, const int32_t* y_cu, int B, int x_maxlen,
+                     int QH, int KH, int D, int VD, int kernel_size, int stride, float sm_scale, void* stream);
+/* flash_nsa/ops/sliding_window_attention.py:42-95 swa_fwd (FlashAttention varlen, window=(W,-1), causal) */
+int nsa_swa_fwd(const void* q, int64_t q_st, int64_t q_sh, const void* k, int64_t k_sr, int64_t k_sh,
+                const void* v, int64_t v_sr, int64_t v_sh, void* o, int64_t o_st, int64_t o_sh, float* lse,
+                int64_t lse_st, int64_t lse_sh, const int32_t* x_cu, int B, int x_maxlen, int QH, int KH, int D,
+                int VD, int window, float sm_scale, void* stream);
+/* flash_nsa/ops/topk.py:630-775 slc_topk_indices; topk int32 addressed kh*tk_sh + tok*tk_st + slot;
+ * imp_out optional fp32 block scores [KH, T, imp_cols] */
+int nsa_topk_select(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr, int64_t ck_sh,
+                    const float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk, int64_t tk_sh, int64_t tk_st,
+                    float* imp_out, int64_t imp_sh, int64_t imp_st, int imp_cols, const int32_t* x_cu,
+                    const int32_t* y_cu, int B, int x_maxlen, int QH, int KH, int D, int kernel_size, int stride,
+                    int block_size, int top_n, int num_init, int num_local, int ignore_index, float sm_scale,
+                    void* stream);
+/* flash_nsa/ops/select_attn.py:439-507 slc_attn_fwd */
+int nsa_slc_attn_fwd(const void* q, int64_t q_st, int64_t q_sh, const void* k, int64_t k_sr, int64_t k_sh,
+                     const void* v, int64_t v_sr, int64_t v_sh, const int32_t* topk, int64_t tk_sh, int64_t tk_st,
+                     void* o, int64_t o_st, int64_t o_sh, float* lse, int64_t lse_st, int64_t lse_sh,
+                     const int32_t* x_cu, int B, int x_maxlen, int QH, int KH, int D, int VD, int block_size,
+                     int top_n, float sm_scale, void* stream);
+
+/* flash_nsa/inference/compress_kv.py:191-220 mean_pooling_prefill (in-pool write at flat row slot) */
+int nsa_paged_pool_prefill(void* cache, int64_t c_sr, int64_t c_sh, const int32_t* y_cu, const int32_t* block_tables,
+                           int table_stride, const int32_t* cmp_slot_mapping, int B, int y_maxlen, int page_size,
+                           int H, int D, int kernel_size, int stride, void* stream);
+/* flash_nsa/inference/compress_kv.py:253-287 kv_mean_pooling_decode */
+int nsa_paged_pool_decode(void* k_cache, int64_t k_sr, int64_t k_sh, int Dk, void* v_cache, int64_t v_sr,
+                          int64_t v_sh, int Dv, const int32_t* context_lens, const int32_t* block_tables,
+                          int table_stride, const int32_t* cmp_slot_mapping, int B, int page_size, int H,
+                          int kernel_size, int stride, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

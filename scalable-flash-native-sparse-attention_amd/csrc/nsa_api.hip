@@ -1,0 +1,144 @@
+// C entry points for the attention stages plus the library's error plumbing.  Argument checks live here so
+// that a kernel is never launched on shapes its tiling does not cover.
+#include <stdarg.h>
+#include <stdio.h>
+#include <math.h>
+#include "nsa_common.h"
+#include "nsa_api_internal.h"
+
+static thread_local char g_err[512] = "";
+
+void nsa_set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+int nsa_check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    nsa_set_error("%s: launch failed: %s", what, hipGetErrorString(e));
+    return NSA_ERR_LAUNCH;
+  }
+  return NSA_OK;
+}
+
+static int check_heads(const char* who, int QH, int KH, int D, int VD) {
+  NSA_REQUIRE(QH > 0 && KH > 0 && QH % KH == 0, NSA_ERR_BAD_ARG, "%s: q heads %d must be a multiple of kv heads %d",
+              who, QH, KH);
+  NSA_REQUIRE(D % 32 == 0 && VD % 32 == 0, NSA_ERR_BAD_ARG, "%s: head dims %d/%d must be multiples of 32", who, D, VD);
+  return NSA_OK;
+}
+static int check_nsa_sizes(const char* who, int kernel_size, int stride, int block_size) {
+  NSA_REQUIRE(stride > 0 && (stride & (stride - 1)) == 0, NSA_ERR_BAD_ARG, "%s: stride %d must be a power of 2", who,
+              stride);
+  NSA_REQUIRE(kernel_size % stride == 0 && kernel_size >= stride, NSA_ERR_BAD_ARG,
+              "%s: kernel_size %d must be a multiple of stride %d", who, kernel_size, stride);
+  if (block_size > 0) {
+    NSA_REQUIRE(block_size >= kernel_size && block_size % stride == 0, NSA_ERR_BAD_ARG,
+                "%s: block_size %d must be >= kernel_size %d and a multiple of stride %d", who, block_size,
+                kernel_size, stride);
+  }
+  return NSA_OK;
+}
+
+extern "C" {
+
+const char* nsa_last_error(void) { return g_err; }
+int nsa_abi_version(void) { return 1; }
+
+int nsa_cmp_attn_fwd(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr, int64_t ck_sh,
+                     const void* cv, int64_t cv_sr, int64_t cv_sh, void* o, int64_t o_st, int64_t o_sh, float* lse,
+                     int64_t lse_st, int64_t lse_sh, const int32_t* x_cu, const int32_t* y_cu, int B, int x_maxlen,
+                     int QH, int KH, int D, int VD, int kernel_size, int stride, float sm_scale, void* stream) {
+  int rc = check_heads("cmp_attn_fwd", QH, KH, D, VD);
+  if (rc) return rc;
+  rc = check_nsa_sizes("cmp_attn_fwd", kernel_size, stride, 0);
+  if (rc) return rc;
+  NsaFwdTileParams p{};
+  p.q = (const bf16_t*)q; p.q_st = q_st; p.q_sh = q_sh;
+  p.k = (const bf16_t*)ck; p.k_sr = ck_sr; p.k_sh = ck_sh;
+  p.v = (const bf16_t*)cv; p.v_sr = cv_sr; p.v_sh = cv_sh;
+  p.o = (bf16_t*)o; p.o_st = o_st; p.o_sh = o_sh;
+  p.lse = lse; p.lse_st = lse_st; p.lse_sh = lse_sh;
+  p.x_cu = x_cu; p.k_cu = y_cu;
+  p.G = QH / KH; p.KH = KH;
+  p.scale_log2 = sm_scale * NSA_LOG2E;
+  p.kernel_size = kernel_size; p.stride = stride; p.window = 0;
+  return nsa_fwd_tile_launch(p, 0, false, B, x_maxlen, D, VD, (hipStream_t)stream);
+}
+
+int nsa_swa_fwd(const void* q, int64_t q_st, int64_t q_sh, const void* k, int64_t k_sr, int64_t k_sh,
+                const void* v, int64_t v_sr, int64_t v_sh, void* o, int64_t o_st, int64_t o_sh, float* lse,
+                int64_t lse_st, int64_t lse_sh, const int32_t* x_cu, int B, int x_maxlen, int QH, int KH, int D,
+                int VD, int window, float sm_scale, void* stream) {
+  int rc = check_heads("swa_fwd", QH, KH, D, VD);
+  if (rc) return rc;
+  NSA_REQUIRE(window >= 0, NSA_ERR_BAD_ARG, "swa_fwd: window %d must be >= 0", window);
+  NsaFwdTileParams p{};
+  p.q = (const bf16_t*)q; p.q_st = q_st; p.q_sh = q_sh;
+  p.k = (const bf16_t*)k; p.k_sr = k_sr; p.k_sh = k_sh;
+  p.v = (const bf16_t*)v; p.v_sr = v_sr; p.v_sh = v_sh;
+  p.o = (bf16_t*)o; p.o_st = o_st; p.o_sh = o_sh;
+  p.lse = lse; p.lse_st = lse_st; p.lse_sh = lse_sh;
+  p.x_cu = x_cu; p.k_cu = x_cu;
+  p.G = QH / KH; p.KH = KH;
+  p.scale_log2 = sm_scale * NSA_LOG2E;
+  p.kernel_size = 1; p.stride = 1; p.window = window;
+  return nsa_fwd_tile_launch(p, 1, false, B, x_maxlen, D, VD, (hipStream_t)stream);
+}
+
+int nsa_topk_select(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr, int64_t ck_sh,
+                    const float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk, int64_t tk_sh, int64_t tk_st,
+                    float* imp_out, int64_t imp_sh, int64_t imp_st, int imp_cols, const int32_t* x_cu,
+                    const int32_t* y_cu, int B, int x_maxlen, int QH, int KH, int D, int kernel_size, int stride,
+                    int block_size, int top_n, int num_init, int num_local, int ignore_index, float sm_scale,
+                    void* stream) {
+  int rc = check_heads("topk_select", QH, KH, D, 32);
+  if (rc) return rc;
+  rc = check_nsa_sizes("topk_select", kernel_size, stride, block_size);
+  if (rc) return rc;
+  NSA_REQUIRE(top_n >= 1 && top_n <= 64, NSA_ERR_BAD_ARG, "topk_select: top_n %d must be in [1,64]", top_n);
+  NSA_REQUIRE(num_init >= 0 && num_local >= 0 && num_init + num_local <= top_n, NSA_ERR_BAD_ARG,
+              "topk_select: num_init %d + num_local %d must be <= top_n %d", num_init, num_local, top_n);
+  NsaTopkParams p{};
+  p.q = (const bf16_t*)q; p.q_st = q_st; p.q_sh = q_sh;
+  p.ck = (const bf16_t*)ck; p.ck_sr = ck_sr; p.ck_sh = ck_sh;
+  p.lse = lse; p.lse_st = lse_st; p.lse_sh = lse_sh;
+  p.topk = topk; p.tk_sh = tk_sh; p.tk_st = tk_st;
+  p.imp_out = imp_out; p.imp_sh = imp_sh; p.imp_st = imp_st; p.imp_cols = imp_cols;
+  p.x_cu = x_cu; p.y_cu = y_cu;
+  p.G = QH / KH; p.KH = KH;
+  p.scale_log2 = sm_scale * NSA_LOG2E;
+  p.kernel_size = kernel_size; p.stride = stride; p.block_size = block_size;
+  p.top_n = top_n; p.num_init = num_init; p.num_local = num_local; p.ignore_index = ignore_index;
+  p.nb_max = (x_maxlen + block_size - 1) / block_size;
+  if (p.nb_max < 1) p.nb_max = 1;
+  return nsa_topk_launch(p, false, B, x_maxlen, D, (hipStream_t)stream);
+}
+
+int nsa_slc_attn_fwd(const void* q, int64_t q_st, int64_t q_sh, const void* k, int64_t k_sr, int64_t k_sh,
+                     const void* v, int64_t v_sr, int64_t v_sh, const int32_t* topk, int64_t tk_sh, int64_t tk_st,
+                     void* o, int64_t o_st, int64_t o_sh, float* lse, int64_t lse_st, int64_t lse_sh,
+                     const int32_t* x_cu, int B, int x_maxlen, int QH, int KH, int D, int VD, int block_size,
+                     int top_n, float sm_scale, void* stream) {
+  int rc = check_heads("slc_attn_fwd", QH, KH, D, VD);
+  if (rc) return rc;
+  NSA_REQUIRE(block_size % 64 == 0 && block_size > 0, NSA_ERR_UNSUPPORTED,
+              "slc_attn_fwd: block_size %d must be a multiple of 64", block_size);
+  NSA_REQUIRE(top_n >= 1 && top_n <= 64, NSA_ERR_BAD_ARG, "slc_attn_fwd: top_n %d must be in [1,64]", top_n);
+  NsaSlcParams p{};
+  p.q = (const bf16_t*)q; p.q_st = q_st; p.q_sh = q_sh;
+  p.k = (const bf16_t*)k; p.k_sr = k_sr; p.k_sh = k_sh;
+  p.v = (const bf16_t*)v; p.v_sr = v_sr; p.v_sh = v_sh;
+  p.o = (bf16_t*)o; p.o_st = o_st; p.o_sh = o_sh;
+  p.lse = lse; p.lse_st = lse_st; p.lse_sh = lse_sh;
+  p.topk = topk; p.tk_sh = tk_sh; p.tk_st = tk_st;
+  p.x_cu = x_cu;
+  p.G = QH / KH; p.KH = KH; p.top_n = top_n; p.block_size = block_size;
+  p.scale_log2 = sm_scale * NSA_LOG2E;
+  return nsa_slc_fwd_launch(p, false, B, x_maxlen, D, VD, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,111 @@
+// Shared device helpers for the gfx950 (CDNA4) Native-Sparse-Attention kernels.
+//
+// MFMA operand layouts used throughout (wave64, verified on hardware):
+//   v_mfma_f32_32x32x16_bf16:  A[m][k]: lane l holds m = l%32, k = (l/32)*8 .. +7
+//                              B[k][n]: lane l holds n = l%32, k = (l/32)*8 .. +7
+//                              C[m][n]: lane l holds n = l%32, m = (i/4)*8 + (l/32)*4 + i%4, i = 0..15
+//   v_mfma_f32_16x16x32_bf16:  A[m][k]: lane l holds m = l%16, k = (l/16)*8 .. +7
+//                              B[k][n]: lane l holds n = l%16, k = (l/16)*8 .. +7
+//                              C[m][n]: lane l holds n = l%16, m = (l/16)*4 + i, i = 0..3
+// A C-tile can be fed back as the B operand of a following MFMA whose contraction runs over the C-tile's
+// m index: the lane's accumulator values i = 8c .. 8c+7 are the k-slice of "virtual" k-chunk c, as long as the
+// A operand of that MFMA is gathered with the same m -> k permutation (see frag_tr_* below).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+#define NSA_DEVICE __device__ __forceinline__
+#define LDS_PTR(T) __attribute__((address_space(3))) T*
+
+constexpr float NSA_LOG2E = 1.4426950408889634f;
+constexpr float NSA_LN2 = 0.6931471805599453f;
+constexpr float NSA_NEG_INF = -__builtin_huge_valf();
+
+NSA_DEVICE f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+NSA_DEVICE f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+NSA_DEVICE float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+NSA_DEVICE float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+NSA_DEVICE float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+NSA_DEVICE float bf16_bits_to_f32(uint32_t hi16) { return __builtin_bit_cast(float, hi16 << 16); }
+
+// 16-byte global load of 8 bf16
+NSA_DEVICE bf16x8 ld_global_b128(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
+NSA_DEVICE bf16x8 zero_bf16x8() {
+  u32x4 z = {0, 0, 0, 0};
+  return __builtin_bit_cast(bf16x8, z);
+}
+
+// pack 8 floats to bf16x8 (round to nearest even via the hardware convert)
+NSA_DEVICE bf16x8 pack8(float a0, float a1, float a2, float a3, float a4, float a5, float a6, float a7) {
+  bf16x8 r;
+  r[0] = (bf16_t)a0; r[1] = (bf16_t)a1; r[2] = (bf16_t)a2; r[3] = (bf16_t)a3;
+  r[4] = (bf16_t)a4; r[5] = (bf16_t)a5; r[6] = (bf16_t)a6; r[7] = (bf16_t)a7;
+  return r;
+}
+NSA_DEVICE bf16x4 pack4(float a0, float a1, float a2, float a3) {
+  bf16x4 r;
+  r[0] = (bf16_t)a0; r[1] = (bf16_t)a1; r[2] = (bf16_t)a2; r[3] = (bf16_t)a3;
+  return r;
+}
+
+// LDS transpose read (gfx950 ds_read_b64_tr_b16).  Within each group of 16 lanes, lane i receives
+// element (i%4) of the 4-element rows addressed by lanes (i/4), (i/4)+4, (i/4)+8, (i/4)+12 of the group.
+// With lane s of a group pointing at &M[row0 + s/4][col0 + 4*(s%4)] of a row-major bf16 matrix in LDS, lane i
+// gets M[row0+0..3][col0 + i]: four consecutive rows of one column, i.e. a k-slice for an operand whose
+// contraction index is the LDS row.
+NSA_DEVICE bf16x4 lds_read_tr(const bf16_t* p) {
+  s16x4 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))p);
+  return __builtin_bit_cast(bf16x4, r);
+}
+NSA_DEVICE bf16x8 cat4(bf16x4 a, bf16x4 b) {
+  return __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+NSA_DEVICE float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+NSA_DEVICE float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+__host__ __device__ inline int cdiv_i(int a, int b) { return (a + b - 1) / b; }
+
+// error codes returned by the C entry points
+enum {
+  NSA_OK = 0,
+  NSA_ERR_BAD_ARG = 1,
+  NSA_ERR_UNSUPPORTED = 2,
+  NSA_ERR_LAUNCH = 3,
+  NSA_ERR_WORKSPACE = 4,
+};
+
+void nsa_set_error(const char* fmt, ...);
+int nsa_check_launch(const char* what);
+
+#define NSA_REQUIRE(cond, code, ...)        \
+  do {                                      \
+    if (!(cond)) {                          \
+      nsa_set_error(__VA_ARGS__);           \
+      return (code);                        \
+    }                                       \
+  } while (0)

@@ -1,0 +1,477 @@
+// Bandwidth-bound kernels of the path: KV mean pooling (contiguous and paged), im2col of compression
+// windows, the sigmoid-mul / swiglu activations, the sigmoid-gated combine and the delta pre-pass.
+// Every thread moves 16-byte vectors; reductions over a head's channels run across the D/8 lanes that share
+// a (token, head) pair.
+// Upstream: flash_nsa/ops/compress_kv.py:17-426, flash_nsa/ops/act.py:13-208, flash_nsa/ops/combine.py:15-177,
+//           flash_nsa/ops/compress_attn.py:160-184, flash_nsa/inference/compress_kv.py:13-287,
+//           flash_nsa/inference/combine.py:16-127.
+#include "nsa_common.h"
+#include "nsa_api_internal.h"
+
+namespace {
+
+NSA_DEVICE void acc8(float* a, bf16x8 v) {
+#pragma unroll
+  for (int e = 0; e < 8; e++) a[e] += (float)v[e];
+}
+NSA_DEVICE float sigmoidf_(float x) { return 1.f / (1.f + __expf(-x)); }
+
+// ------------------------------------------------------------------------------------------ mean pooling fwd
+// grid (cdiv(y_maxlen*H*D/8, 256), B)
+__global__ void mean_pool_fwd_kernel(const bf16_t* x, int64_t x_st, int64_t x_sh, bf16_t* y, int64_t y_st,
+                                     int64_t y_sh, const int32_t* x_cu, const int32_t* y_cu, int H, int D, int K,
+                                     int S) {
+  const int b = blockIdx.y;
+  const int x0 = x_cu[b], y0 = y_cu[b];
+  const int yl = y_cu[b + 1] - y0;
+  const int C = D / 8;
+  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (int64_t)yl * H * C) return;
+  int c = idx % C;
+  int h = (idx / C) % H;
+  int i = idx / ((int64_t)C * H);
+  float a[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  const bf16_t* xp = x + (int64_t)(x0 + (int64_t)S * i) * x_st + (int64_t)h * x_sh + c * 8;
+  for (int r = 0; r < K; r++) acc8(a, ld_global_b128(xp + r * x_st));
+  float inv = 1.f / (float)K;
+  *reinterpret_cast<bf16x8*>(y + (int64_t)(y0 + i) * y_st + (int64_t)h * y_sh + c * 8) =
+      pack8(a[0] * inv, a[1] * inv, a[2] * inv, a[3] * inv, a[4] * inv, a[5] * inv, a[6] * inv, a[7] * inv);
+}
+
+// ------------------------------------------------------------------------------------------ mean pooling bwd
+// dx[n] (+)= sum over windows containing n of dy[i]/K.  grid (cdiv(x_maxlen*H*D/8, 256), B)
+template <bool DX_F32, bool ACCUM>
+__global__ void mean_pool_bwd_kernel(const bf16_t* dy, int64_t dy_st, int64_t dy_sh, void* dxv, int64_t dx_st,
+                                     int64_t dx_sh, const int32_t* x_cu, const int32_t* y_cu, int H, int D, int K,
+                                     int S) {
+  const int b = blockIdx.y;
+  const int x0 = x_cu[b], y0 = y_cu[b];
+  const int xl = x_cu[b + 1] - x0, yl = y_cu[b + 1] - y0;
+  const int C = D / 8;
+  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (int64_t)xl * H * C) return;
+  int c = idx % C;
+  int h = (idx / C) % H;
+  int n = idx / ((int64_t)C * H);
+  int i_lo = n - K + 1 <= 0 ? 0 : (n - K + 1 + S - 1) / S;
+  int i_hi = min(n / S, yl - 1);
+  float a[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int i = i_lo; i <= i_hi; i++)
+    acc8(a, ld_global_b128(dy + (int64_t)(y0 + i) * dy_st + (int64_t)h * dy_sh + c * 8));
+  float inv = 1.f / (float)K;
+  int64_t off = (int64_t)(x0 + n) * dx_st + (int64_t)h * dx_sh + c * 8;
+  if (DX_F32) {
+    float* dx = (float*)dxv + off;
+    f32x4 lo = {a[0] * inv, a[1] * inv, a[2] * inv, a[3] * inv};
+    f32x4 hi = {a[4] * inv, a[5] * inv, a[6] * inv, a[7] * inv};
+    if (ACCUM) {
+      if (i_lo > i_hi) return;
+      lo += *reinterpret_cast<f32x4*>(dx);
+      hi += *reinterpret_cast<f32x4*>(dx + 4);
+    }
+    *reinterpret_cast<f32x4*>(dx) = lo;
+    *reinterpret_cast<f32x4*>(dx + 4) = hi;
+  } else {
+    bf16_t* dx = (bf16_t*)dxv + off;
+    *reinterpret_cast<bf16x8*>(dx) =
+        pack8(a[0] * inv, a[1] * inv, a[2] * inv, a[3] * inv, a[4] * inv, a[5] * inv, a[6] * inv, a[7] * inv);
+  }
+}
+
+// ------------------------------------------------------------------------------------------ im2col fwd / bwd
+// y[i,h,r,:] = x[S*i+r,h,:]   grid (cdiv(y_maxlen*H*K*D/8,256), B); y contiguous [y_len,H,K,D]
+__global__ void construct_block_fwd_kernel(const bf16_t* x, int64_t x_st, int64_t x_sh, bf16_t* y,
+                                           const int32_t* x_cu, const int32_t* y_cu, int H, int D, int K, int S) {
+  const int b = blockIdx.y;
+  const int x0 = x_cu[b], y0 = y_cu[b];
+  const int yl = y_cu[b + 1] - y0;
+  const int C = D / 8;
+  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (int64_t)yl * H * K * C) return;
+  int c = idx % C;
+  int r = (idx / C) % K;
+  int h = (idx / ((int64_t)C * K)) % H;
+  int i = idx / ((int64_t)C * K * H);
+  bf16x8 v = ld_global_b128(x + (int64_t)(x0 + (int64_t)S * i + r) * x_st + (int64_t)h * x_sh + c * 8);
+  *reinterpret_cast<bf16x8*>(y + (((int64_t)(y0 + i) * H + h) * K + r) * D + c * 8) = v;
+}
+
+// dx[n,h,:] (+)= sum_i dblock[i,h,n-S*i,:]
+template <bool DX_F32, bool ACCUM>
+__global__ void construct_block_bwd_kernel(const bf16_t* dyb, void* dxv, int64_t dx_st, int64_t dx_sh,
+                                           const int32_t* x_cu, const int32_t* y_cu, int H, int D, int K, int S) {
+  const int b = blockIdx.y;
+  const int x0 = x_cu[b], y0 = y_cu[b];
+  const int xl = x_cu[b + 1] - x0, yl = y_cu[b + 1] - y0;
+  const int C = D / 8;
+  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (int64_t)xl * H * C) return;
+  int c = idx % C;
+  int h = (idx / C) % H;
+  int n = idx / ((int64_t)C * H);
+  int i_lo = n - K + 1 <= 0 ? 0 : (n - K + 1 + S - 1) / S;
+  int i_hi = min(n / S, yl - 1);
+  float a[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int i = i_lo; i <= i_hi; i++)
+    acc8(a, ld_global_b128(dyb + (((int64_t)(y0 + i) * H + h) * K + (n - S * i)) * D + c * 8));
+  int64_t off = (int64_t)(x0 + n) * dx_st + (int64_t)h * dx_sh + c * 8;
+  if (DX_F32) {
+    float* dx = (float*)dxv + off;
+    f32x4 lo = {a[0], a[1], a[2], a[3]};
+    f32x4 hi = {a[4], a[5], a[6], a[7]};
+    if (ACCUM) {
+      if (i_lo > i_hi) return;
+      lo += *reinterpret_cast<f32x4*>(dx);
+      hi += *reinterpret_cast<f32x4*>(dx + 4);
+    }
+    *reinterpret_cast<f32x4*>(dx) = lo;
+    *reinterpret_cast<f32x4*>(dx + 4) = hi;
+  } else {
+    *reinterpret_cast<bf16x8*>((bf16_t*)dxv + off) = pack8(a[0], a[1], a[2], a[3], a[4], a[5], a[6], a[7]);
+  }
+}
+
+// ------------------------------------------------------------------------------------------ gated activations
+// x [N, 2*d] (gate | up) -> y [N, d];  ACT 0: sigmoid(gate)*up, 1: silu(gate)*up
+template <int ACT>
+__global__ void glu_fwd_kernel(const bf16_t* x, bf16_t* y, int64_t N, int d) {
+  const int C = d / 8;
+  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= N * C) return;
+  int c = idx % C;
+  int64_t n = idx / C;
+  bf16x8 g = ld_global_b128(x + n * 2 * d + c * 8);
+  bf16x8 u = ld_global_b128(x + n * 2 * d + d + c * 8);
+  float o[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++) {
+    float gf = (float)g[e], uf = (float)u[e];
+    float s = sigmoidf_(gf);
+    o[e] = (ACT == 0 ? s : s * gf) * uf;
+  }
+  *reinterpret_cast<bf16x8*>(y + n * d + c * 8) = pack8(o[0], o[1], o[2], o[3], o[4], o[5], o[6], o[7]);
+}
+// dx [N, 2*d] = [dgate | dup]; may alias x (each thread reads its inputs before writing)
+template <int ACT>
+__global__ void glu_bwd_kernel(const bf16_t* x, const bf16_t* dy, bf16_t* dx, int64_t N, int d) {
+  const int C = d / 8;
+  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= N * C) return;
+  int c = idx % C;
+  int64_t n = idx / C;
+  bf16x8 g = ld_global_b128(x + n * 2 * d + c * 8);
+  bf16x8 u = ld_global_b128(x + n * 2 * d + d + c * 8);
+  bf16x8 go = ld_global_b128(dy + n * d + c * 8);
+  float dg[8], du[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++) {
+    float gf = (float)g[e], uf = (float)u[e], d0 = (float)go[e];
+    float s = sigmoidf_(gf);
+    if (ACT == 0) {
+      du[e] = d0 * s;
+      dg[e] = d0 * uf * s * (1.f - s);
+    } else {
+      du[e] = d0 * s * gf;
+      dg[e] = d0 * uf * (s + gf * s * (1.f - s));
+    }
+  }
+  *reinterpret_cast<bf16x8*>(dx + n * 2 * d + c * 8) = pack8(dg[0], dg[1], dg[2], dg[3], dg[4], dg[5], dg[6], dg[7]);
+  *reinterpret_cast<bf16x8*>(dx + n * 2 * d + d + c * 8) =
+      pack8(du[0], du[1], du[2], du[3], du[4], du[5], du[6], du[7]);
+}
+
+// ------------------------------------------------------------------------------------------ combine
+// o = a*sig(w0) + b*sig(w1) + c*sig(w2).  One thread per 8 channels; grid cdiv(T*H*D/8, 256)
+__global__ void combine_fwd_kernel(const bf16_t* a, const bf16_t* bb, const bf16_t* c, int64_t i_st, int64_t i_sh,
+                                   const bf16_t* w, int64_t w_st, int64_t w_sh, bf16_t* o, int64_t o_st,
+                                   int64_t o_sh, int64_t T, int H, int D) {
+  const int C = D / 8;
+  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= T * H * C) return;
+  int cc = idx % C;
+  int h = (idx / C) % H;
+  int64_t t = idx / ((int64_t)C * H);
+  const bf16_t* wp = w + t * w_st + (int64_t)h * w_sh;
+  float s0 = sigmoidf_((float)wp[0]), s1 = sigmoidf_((float)wp[1]), s2 = sigmoidf_((float)wp[2]);
+  int64_t off = t * i_st + (int64_t)h * i_sh + cc * 8;
+  bf16x8 va = ld_global_b128(a + off), vb = ld_global_b128(bb + off), vc = ld_global_b128(c + off);
+  float r[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++) r[e] = (float)va[e] * s0 + (float)vb[e] * s1 + (float)vc[e] * s2;
+  *reinterpret_cast<bf16x8*>(o + t * o_st + (int64_t)h * o_sh + cc * 8) =
+      pack8(r[0], r[1], r[2], r[3], r[4], r[5], r[6], r[7]);
+}
+
+// backward: da,db,dc = dy*sig(w_k); dw_k = sig_k(1-sig_k) * sum_d dy*x_k; optional delta_k = sig_k * sum_d dy*x_k
+// (= rowsum(x_k * d x_k), the softmax-backward correction term of branch k), written as delta[k][T][H] fp32.
+// D/8 consecutive lanes share one (t,h); D/8 must be a power of two <= 64.
+__global__ void combine_bwd_kernel(const bf16_t* a, const bf16_t* bb, const bf16_t* c, int64_t i_st, int64_t i_sh,
+                                   const bf16_t* w, int64_t w_st, int64_t w_sh, const bf16_t* dy, int64_t dy_st,
+                                   int64_t dy_sh, bf16_t* da, bf16_t* db, bf16_t* dc, bf16_t* dw, float* delta,
+                                   int64_t T, int H, int D) {
+  const int C = D / 8;
+  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  bool ok = idx < T * H * C;
+  if (!ok) idx = T * H * C - 1;
+  int cc = idx % C;
+  int h = (idx / C) % H;
+  int64_t t = idx / ((int64_t)C * H);
+  const bf16_t* wp = w + t * w_st + (int64_t)h * w_sh;
+  float s0 = sigmoidf_((float)wp[0]), s1 = sigmoidf_((float)wp[1]), s2 = sigmoidf_((float)wp[2]);
+  int64_t off = t * i_st + (int64_t)h * i_sh + cc * 8;
+  bf16x8 va = ld_global_b128(a + off), vb = ld_global_b128(bb + off), vc = ld_global_b128(c + off);
+  bf16x8 g = ld_global_b128(dy + t * dy_st + (int64_t)h * dy_sh + cc * 8);
+  float ra[8], rb[8], rc[8], p0 = 0.f, p1 = 0.f, p2 = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; e++) {
+    float gf = (float)g[e];
+    ra[e] = gf * s0; rb[e] = gf * s1; rc[e] = gf * s2;
+    p0 += gf * (float)va[e]; p1 += gf * (float)vb[e]; p2 += gf * (float)vc[e];
+  }
+  for (int o = C >> 1; o > 0; o >>= 1) {
+    p0 += __shfl_xor(p0, o, 64); p1 += __shfl_xor(p1, o, 64); p2 += __shfl_xor(p2, o, 64);
+  }
+  if (!ok) return;
+  int64_t ooff = (t * H + h) * (int64_t)D + cc * 8;  // grads are contiguous [T,H,D]
+  *reinterpret_cast<bf16x8*>(da + ooff) = pack8(ra[0], ra[1], ra[2], ra[3], ra[4], ra[5], ra[6], ra[7]);
+  *reinterpret_cast<bf16x8*>(db + ooff) = pack8(rb[0], rb[1], rb[2], rb[3], rb[4], rb[5], rb[6], rb[7]);
+  *reinterpret_cast<bf16x8*>(dc + ooff) = pack8(rc[0], rc[1], rc[2], rc[3], rc[4], rc[5], rc[6], rc[7]);
+  if (cc == 0) {
+    bf16_t* dwp = dw + (t * H + h) * 3;
+    dwp[0] = (bf16_t)(s0 * (1.f - s0) * p0);
+    dwp[1] = (bf16_t)(s1 * (1.f - s1) * p1);
+    dwp[2] = (bf16_t)(s2 * (1.f - s2) * p2);
+    if (delta != nullptr) {
+      int64_t TH = T * H;
+      delta[0 * TH + t * H + h] = s0 * p0;
+      delta[1 * TH + t * H + h] = s1 * p1;
+      delta[2 * TH + t * H + h] = s2 * p2;
+    }
+  }
+}
+
+// delta[t,h] = sum_d o*do   (fp32, contiguous [T,H])
+__global__ void delta_kernel(const bf16_t* o, int64_t o_st, int64_t o_sh, const bf16_t* dO, int64_t d_st,
+                             int64_t d_sh, float* delta, int64_t T, int H, int D) {
+  const int C = D / 8;
+  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  bool ok = idx < T * H * C;
+  if (!ok) idx = T * H * C - 1;
+  int cc = idx % C;
+  int h = (idx / C) % H;
+  int64_t t = idx / ((int64_t)C * H);
+  bf16x8 vo = ld_global_b128(o + t * o_st + (int64_t)h * o_sh + cc * 8);
+  bf16x8 vd = ld_global_b128(dO + t * d_st + (int64_t)h * d_sh + cc * 8);
+  float s = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; e++) s += (float)vo[e] * (float)vd[e];
+  for (int o2 = C >> 1; o2 > 0; o2 >>= 1) s += __shfl_xor(s, o2, 64);
+  if (ok && cc == 0) delta[t * H + h] = s;
+}
+
+// ------------------------------------------------------------------------------------------ paged pooling
+// prefill: one compressed row per (entry e, head, chunk); rows read through the raw block table, written to flat
+// pool row slot[e] unless slot[e] < 0.   grid (cdiv(y_maxlen*H*C,256), B)
+__global__ void paged_pool_prefill_kernel(bf16_t* cache, int64_t c_sr, int64_t c_sh, const int32_t* y_cu,
+                                          const int32_t* table, int table_stride, const int32_t* slots,
+                                          int page, int H, int D, int K, int S) {
+  const int b = blockIdx.y;
+  const int y0 = y_cu[b];
+  const int yl = y_cu[b + 1] - y0;
+  const int C = D / 8;
+  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (int64_t)yl * H * C) return;
+  int c = idx % C;
+  int h = (idx / C) % H;
+  int i = idx / ((int64_t)C * H);
+  int slot = slots[y0 + i];
+  if (slot < 0) return;
+  const int32_t* tb = table + (int64_t)b * table_stride;
+  float a[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int r = 0; r < K; r++) {
+    int n = S * i + r;
+    int64_t row = (int64_t)tb[n / page] * page + (n % page);
+    acc8(a, ld_global_b128(cache + row * c_sr + (int64_t)h * c_sh + c * 8));
+  }
+  float inv = 1.f / (float)K;
+  *reinterpret_cast<bf16x8*>(cache + (int64_t)slot * c_sr + (int64_t)h * c_sh + c * 8) =
+      pack8(a[0] * inv, a[1] * inv, a[2] * inv, a[3] * inv, a[4] * inv, a[5] * inv, a[6] * inv, a[7] * inv);
+}
+
+// decode: per request, pool the last complete window of K (blockIdx.z = 0) and V (= 1) if slot >= 0 and len >= K.
+// grid (cdiv(H*C, 64), B, 2), block 64
+__global__ void paged_pool_decode_kernel(bf16_t* kc, int64_t k_sr, int64_t k_sh, int Dk, bf16_t* vc, int64_t v_sr,
+                                         int64_t v_sh, int Dv, const int32_t* ctx_lens, const int32_t* table,
+                                         int table_stride, const int32_t* slots, int page, int H, int K, int S) {
+  const int b = blockIdx.y;
+  const int slot = slots[b];
+  const int L = ctx_lens[b];
+  if (slot < 0 || L < K) return;
+  bf16_t* cache = blockIdx.z == 0 ? kc : vc;
+  const int64_t c_sr = blockIdx.z == 0 ? k_sr : v_sr, c_sh = blockIdx.z == 0 ? k_sh : v_sh;
+  const int D = blockIdx.z == 0 ? Dk : Dv;
+  const int C = D / 8;
+  int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= H * C) return;
+  int c = idx % C, h = idx / C;
+  const int st = ((L - K) / S) * S;
+  const int32_t* tb = table + (int64_t)b * table_stride;
+  float a[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int r = 0; r < K; r++) {
+    int n = st + r;
+    int64_t row = (int64_t)tb[n / page] * page + (n % page);
+    acc8(a, ld_global_b128(cache + row * c_sr + (int64_t)h * c_sh + c * 8));
+  }
+  float inv = 1.f / (float)K;
+  *reinterpret_cast<bf16x8*>(cache + (int64_t)slot * c_sr + (int64_t)h * c_sh + c * 8) =
+      pack8(a[0] * inv, a[1] * inv, a[2] * inv, a[3] * inv, a[4] * inv, a[5] * inv, a[6] * inv, a[7] * inv);
+}
+
+inline unsigned blocks_for(int64_t n, int bs) { return (unsigned)((n + bs - 1) / bs); }
+
+}  // namespace
+
+// ============================================================================================== C entry points
+extern "C" {
+
+int nsa_mean_pool_fwd(const void* x, int64_t x_st, int64_t x_sh, void* y, int64_t y_st, int64_t y_sh,
+                      const int32_t* x_cu, const int32_t* y_cu, int B, int y_maxlen, int H, int D, int kernel_size,
+                      int stride, void* stream) {
+  NSA_REQUIRE(D % 8 == 0 && D > 0, NSA_ERR_BAD_ARG, "mean_pool_fwd: head dim %d must be a multiple of 8", D);
+  if (B <= 0 || y_maxlen <= 0) return NSA_OK;
+  dim3 grid(blocks_for((int64_t)y_maxlen * H * (D / 8), 256), B);
+  mean_pool_fwd_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const bf16_t*)x, x_st, x_sh, (bf16_t*)y, y_st, y_sh,
+                                                              x_cu, y_cu, H, D, kernel_size, stride);
+  return nsa_check_launch("mean_pool_fwd");
+}
+
+int nsa_mean_pool_bwd(const void* dy, int64_t dy_st, int64_t dy_sh, void* dx, int64_t dx_st, int64_t dx_sh,
+                      int dx_is_f32, int accumulate, const int32_t* x_cu, const int32_t* y_cu, int B, int x_maxlen,
+                      int H, int D, int kernel_size, int stride, void* stream) {
+  NSA_REQUIRE(D % 8 == 0 && D > 0, NSA_ERR_BAD_ARG, "mean_pool_bwd: head dim %d must be a multiple of 8", D);
+  NSA_REQUIRE(dx_is_f32 || !accumulate, NSA_ERR_BAD_ARG, "mean_pool_bwd: accumulation needs an fp32 dx");
+  if (B <= 0 || x_maxlen <= 0) return NSA_OK;
+  dim3 grid(blocks_for((int64_t)x_maxlen * H * (D / 8), 256), B);
+  hipStream_t s = (hipStream_t)stream;
+  const bf16_t* g = (const bf16_t*)dy;
+  if (dx_is_f32 && accumulate)
+    mean_pool_bwd_kernel<true, true><<<grid, 256, 0, s>>>(g, dy_st, dy_sh, dx, dx_st, dx_sh, x_cu, y_cu, H, D, kernel_size, stride);
+  else if (dx_is_f32)
+    mean_pool_bwd_kernel<true, false><<<grid, 256, 0, s>>>(g, dy_st, dy_sh, dx, dx_st, dx_sh, x_cu, y_cu, H, D, kernel_size, stride);
+  else
+    mean_pool_bwd_kernel<false, false><<<grid, 256, 0, s>>>(g, dy_st, dy_sh, dx, dx_st, dx_sh, x_cu, y_cu, H, D, kernel_size, stride);
+  return nsa_check_launch("mean_pool_bwd");
+}
+
+int nsa_construct_block_fwd(const void* x, int64_t x_st, int64_t x_sh, void* y, const int32_t* x_cu,
+                            const int32_t* y_cu, int B, int y_maxlen, int H, int D, int kernel_size, int stride,
+                            void* stream) {
+  NSA_REQUIRE(D % 8 == 0 && D > 0, NSA_ERR_BAD_ARG, "construct_block_fwd: head dim %d must be a multiple of 8", D);
+  if (B <= 0 || y_maxlen <= 0) return NSA_OK;
+  dim3 grid(blocks_for((int64_t)y_maxlen * H * kernel_size * (D / 8), 256), B);
+  construct_block_fwd_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const bf16_t*)x, x_st, x_sh, (bf16_t*)y, x_cu,
+                                                                    y_cu, H, D, kernel_size, stride);
+  return nsa_check_launch("construct_block_fwd");
+}
+
+int nsa_construct_block_bwd(const void* dblock, void* dx, int64_t dx_st, int64_t dx_sh, int dx_is_f32,
+                            int accumulate, const int32_t* x_cu, const int32_t* y_cu, int B, int x_maxlen, int H,
+                            int D, int kernel_size, int stride, void* stream) {
+  NSA_REQUIRE(D % 8 == 0 && D > 0, NSA_ERR_BAD_ARG, "construct_block_bwd: head dim %d must be a multiple of 8", D);
+  NSA_REQUIRE(dx_is_f32 || !accumulate, NSA_ERR_BAD_ARG, "construct_block_bwd: accumulation needs an fp32 dx");
+  if (B <= 0 || x_maxlen <= 0) return NSA_OK;
+  dim3 grid(blocks_for((int64_t)x_maxlen * H * (D / 8), 256), B);
+  hipStream_t s = (hipStream_t)stream;
+  const bf16_t* g = (const bf16_t*)dblock;
+  if (dx_is_f32 && accumulate)
+    construct_block_bwd_kernel<true, true><<<grid, 256, 0, s>>>(g, dx, dx_st, dx_sh, x_cu, y_cu, H, D, kernel_size, stride);
+  else if (dx_is_f32)
+    construct_block_bwd_kernel<true, false><<<grid, 256, 0, s>>>(g, dx, dx_st, dx_sh, x_cu, y_cu, H, D, kernel_size, stride);
+  else
+    construct_block_bwd_kernel<false, false><<<grid, 256, 0, s>>>(g, dx, dx_st, dx_sh, x_cu, y_cu, H, D, kernel_size, stride);
+  return nsa_check_launch("construct_block_bwd");
+}
+
+int nsa_glu_fwd(const void* x, void* y, int64_t N, int d, int act, void* stream) {
+  NSA_REQUIRE(d % 8 == 0 && d > 0, NSA_ERR_BAD_ARG, "glu_fwd: width %d must be a multiple of 8", d);
+  NSA_REQUIRE(act == 0 || act == 1, NSA_ERR_BAD_ARG, "glu_fwd: act must be 0 (sigmoid-mul) or 1 (swiglu)");
+  if (N <= 0) return NSA_OK;
+  unsigned g = blocks_for(N * (d / 8), 256);
+  if (act == 0) glu_fwd_kernel<0><<<g, 256, 0, (hipStream_t)stream>>>((const bf16_t*)x, (bf16_t*)y, N, d);
+  else glu_fwd_kernel<1><<<g, 256, 0, (hipStream_t)stream>>>((const bf16_t*)x, (bf16_t*)y, N, d);
+  return nsa_check_launch("glu_fwd");
+}
+
+int nsa_glu_bwd(const void* x, const void* dy, void* dx, int64_t N, int d, int act, void* stream) {
+  NSA_REQUIRE(d % 8 == 0 && d > 0, NSA_ERR_BAD_ARG, "glu_bwd: width %d must be a multiple of 8", d);
+  NSA_REQUIRE(act == 0 || act == 1, NSA_ERR_BAD_ARG, "glu_bwd: act must be 0 (sigmoid-mul) or 1 (swiglu)");
+  if (N <= 0) return NSA_OK;
+  unsigned g = blocks_for(N * (d / 8), 256);
+  if (act == 0) glu_bwd_kernel<0><<<g, 256, 0, (hipStream_t)stream>>>((const bf16_t*)x, (const bf16_t*)dy, (bf16_t*)dx, N, d);
+  else glu_bwd_kernel<1><<<g, 256, 0, (hipStream_t)stream>>>((const bf16_t*)x, (const bf16_t*)dy, (bf16_t*)dx, N, d);
+  return nsa_check_launch("glu_bwd");
+}
+
+int nsa_combine_fwd(const void* a, const void* b, const void* c, int64_t i_st, int64_t i_sh, const void* w,
+                    int64_t w_st, int64_t w_sh, void* o, int64_t o_st, int64_t o_sh, int64_t T, int H, int D,
+                    void* stream) {
+  NSA_REQUIRE(D % 8 == 0 && D > 0, NSA_ERR_BAD_ARG, "combine_fwd: head dim %d must be a multiple of 8", D);
+  if (T <= 0) return NSA_OK;
+  combine_fwd_kernel<<<blocks_for(T * H * (D / 8), 256), 256, 0, (hipStream_t)stream>>>(
+      (const bf16_t*)a, (const bf16_t*)b, (const bf16_t*)c, i_st, i_sh, (const bf16_t*)w, w_st, w_sh, (bf16_t*)o, o_st,
+      o_sh, T, H, D);
+  return nsa_check_launch("combine_fwd");
+}
+
+int nsa_combine_bwd(const void* a, const void* b, const void* c, int64_t i_st, int64_t i_sh, const void* w,
+                    int64_t w_st, int64_t w_sh, const void* dy, int64_t dy_st, int64_t dy_sh, void* da, void* db,
+                    void* dc, void* dw, float* delta3, int64_t T, int H, int D, void* stream) {
+  int C = D / 8;
+  NSA_REQUIRE(D % 8 == 0 && C > 0 && C <= 64 && (C & (C - 1)) == 0, NSA_ERR_BAD_ARG,
+              "combine_bwd: head dim %d must be 8 * a power of two <= 512", D);
+  if (T <= 0) return NSA_OK;
+  combine_bwd_kernel<<<blocks_for(T * H * C, 256), 256, 0, (hipStream_t)stream>>>(
+      (const bf16_t*)a, (const bf16_t*)b, (const bf16_t*)c, i_st, i_sh, (const bf16_t*)w, w_st, w_sh, (const bf16_t*)dy,
+      dy_st, dy_sh, (bf16_t*)da, (bf16_t*)db, (bf16_t*)dc, (bf16_t*)dw, delta3, T, H, D);
+  return nsa_check_launch("combine_bwd");
+}
+
+int nsa_delta(const void* o, int64_t o_st, int64_t o_sh, const void* dO, int64_t d_st, int64_t d_sh, float* delta,
+              int64_t T, int H, int D, void* stream) {
+  int C = D / 8;
+  NSA_REQUIRE(D % 8 == 0 && C > 0 && C <= 64 && (C & (C - 1)) == 0, NSA_ERR_BAD_ARG,
+              "delta: head dim %d must be 8 * a power of two <= 512", D);
+  if (T <= 0) return NSA_OK;
+  delta_kernel<<<blocks_for(T * H * C, 256), 256, 0, (hipStream_t)stream>>>((const bf16_t*)o, o_st, o_sh,
+                                                                            (const bf16_t*)dO, d_st, d_sh, delta, T, H, D);
+  return nsa_check_launch("delta");
+}
+
+int nsa_paged_pool_prefill(void* cache, int64_t c_sr, int64_t c_sh, const int32_t* y_cu, const int32_t* block_tables,
+                           int table_stride, const int32_t* cmp_slot_mapping, int B, int y_maxlen, int page_size,
+                           int H, int D, int kernel_size, int stride, void* stream) {
+  NSA_REQUIRE(D % 8 == 0 && D > 0, NSA_ERR_BAD_ARG, "paged_pool_prefill: head dim %d must be a multiple of 8", D);
+  if (B <= 0 || y_maxlen <= 0) return NSA_OK;
+  dim3 grid(blocks_for((int64_t)y_maxlen * H * (D / 8), 256), B);
+  paged_pool_prefill_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((bf16_t*)cache, c_sr, c_sh, y_cu, block_tables,
+                                                                   table_stride, cmp_slot_mapping, page_size, H, D,
+                                                                   kernel_size, stride);
+  return nsa_check_launch("paged_pool_prefill");
+}
+
+int nsa_paged_pool_decode(void* k_cache, int64_t k_sr, int64_t k_sh, int Dk, void* v_cache, int64_t v_sr,
+                          int64_t v_sh, int Dv, const int32_t* context_lens, const int32_t* block_tables,
+                          int table_stride, const int32_t* cmp_slot_mapping, int B, int page_size, int H,
+                          int kernel_size, int stride, void* stream) {
+  NSA_REQUIRE(Dk % 8 == 0 && Dv % 8 == 0, NSA_ERR_BAD_ARG, "paged_pool_decode: head dims must be multiples of 8");
+  if (B <= 0) return NSA_OK;
+  int mx = Dk > Dv ? Dk : Dv;
+  dim3 grid(blocks_for((int64_t)H * (mx / 8), 64), B, 2);
+  paged_pool_decode_kernel<<<grid, 64, 0, (hipStream_t)stream>>>((bf16_t*)k_cache, k_sr, k_sh, Dk, (bf16_t*)v_cache,
+                                                                 v_sr, v_sh, Dv, context_lens, block_tables,
+                                                                 table_stride, cmp_slot_mapping, page_size, H,
+                                                                 kernel_size, stride);
+  return nsa_check_launch("paged_pool_decode");
+}
+
+}  // extern "C"

@@ -1,0 +1,284 @@
+// Dense-tile flash forward for the two branches whose key set is a contiguous range per query:
+//   MODE_CMP: compressed attention, key i visible to absolute query position t iff t >= stride*i + kernel-1
+//             (upstream flash_nsa/ops/compress_attn.py:17-153; paged: flash_nsa/inference/compress_attn.py:19-149)
+//   MODE_SWA: causal sliding window, keys max(0,t-W) <= j <= t
+//             (upstream flash_nsa/ops/sliding_window_attention.py:26-95, which calls FlashAttention)
+//
+// Work decomposition: a "row" is one (query token, q-head) pair of one kv-head group, rows ordered
+// token-major / head-minor so that the G heads sharing K/V sit next to each other.  A workgroup of 4 waves
+// owns 4*32*RS consecutive rows; every lane owns RS rows (lane l and l+32 share a row and split its keys), so
+// the online-softmax statistics are per-lane scalars.  Key tiles of 64 rows are staged in LDS (row-major) and
+// shared by the 4 waves.  S^T = K Q^T and O^T = V^T P^T are computed with v_mfma_f32_32x32x16_bf16; the V^T
+// operand comes from ds_read_b64_tr_b16 so V never needs an explicit transpose.
+#include "nsa_common.h"
+#include "nsa_api_internal.h"
+
+namespace {
+
+constexpr int MODE_CMP = 0;
+constexpr int MODE_SWA = 1;
+
+template <int D, int VD, int MODE, bool PAGED, int RS>
+__global__ __launch_bounds__(256) void fwd_tile_kernel(NsaFwdTileParams p) {
+  constexpr int ROWS_W = 32 * RS;
+  constexpr int ROWS_WG = 4 * ROWS_W;
+  constexpr int KT = 64;
+  constexpr int KLD = D + 8;
+  constexpr int VLD = VD + 8;
+  __shared__ __attribute__((aligned(16))) bf16_t Ks[KT * KLD];
+  __shared__ __attribute__((aligned(16))) bf16_t Vs[KT * VLD];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int l32 = lane & 31;
+  const int hl = lane >> 5;
+  const int b = blockIdx.y;
+  const int kh = blockIdx.z;
+  const int G = p.G;
+
+  const int x0 = p.x_cu[b];
+  const int xl = p.x_cu[b + 1] - x0;
+  const int rows_total = xl * G;
+  const int r0 = blockIdx.x * ROWS_WG;
+  if (r0 >= rows_total) return;
+  const int ctx = PAGED ? p.ctx_lens[b] : xl;
+  const int qoff = ctx - xl;
+  int nkeys, kbase = 0;
+  if (MODE == MODE_CMP) {
+    nkeys = ctx >= p.kernel_size ? (ctx - p.kernel_size) / p.stride + 1 : 0;
+    if (!PAGED) kbase = p.k_cu[b];
+  } else {
+    nkeys = ctx;
+    if (!PAGED) kbase = x0;
+  }
+  const int32_t* table = PAGED ? p.table + (int64_t)b * p.table_stride : nullptr;
+
+  // ---- per-lane rows ----
+  int t_row[RS];
+  bool valid[RS];
+  int64_t tok[RS];
+  int head[RS];
+  bf16x8 qf[RS][D / 16];
+#pragma unroll
+  for (int rs = 0; rs < RS; rs++) {
+    int r = r0 + wave * ROWS_W + rs * 32 + l32;
+    valid[rs] = r < rows_total;
+    int rr = valid[rs] ? r : rows_total - 1;
+    int n = rr / G;
+    int g = rr - n * G;
+    t_row[rs] = n + qoff;
+    tok[rs] = x0 + n;
+    head[rs] = kh * G + g;
+    const bf16_t* qp = p.q + tok[rs] * p.q_st + (int64_t)head[rs] * p.q_sh + hl * 8;
+#pragma unroll
+    for (int kc = 0; kc < D / 16; kc++) qf[rs][kc] = ld_global_b128(qp + kc * 16);
+  }
+  // wave-uniform position range
+  const int rw_lo = r0 + wave * ROWS_W;
+  const int rw_hi = min(rw_lo + ROWS_W - 1, rows_total - 1);
+  const bool wave_active = rw_lo < rows_total;
+  const int tw_lo = (wave_active ? rw_lo / G : 0) + qoff;
+  const int tw_hi = (wave_active ? rw_hi / G : 0) + qoff;
+  // workgroup position range
+  const int t_lo = r0 / G + qoff;
+  const int t_hi = min(r0 + ROWS_WG - 1, rows_total - 1) / G + qoff;
+
+  int key_begin, key_end;
+  if (MODE == MODE_CMP) {
+    key_begin = 0;
+    key_end = t_hi >= p.kernel_size - 1 ? min((t_hi - p.kernel_size + 1) / p.stride + 1, nkeys) : 0;
+  } else {
+    key_begin = (max(0, t_lo - p.window) / KT) * KT;
+    key_end = min(t_hi + 1, nkeys);
+  }
+
+  f32x16 oacc[RS][VD / 32];
+  float m_run[RS], l_run[RS];
+#pragma unroll
+  for (int rs = 0; rs < RS; rs++) {
+    m_run[rs] = NSA_NEG_INF;
+    l_run[rs] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < VD / 32; dt++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) oacc[rs][dt][i] = 0.f;
+  }
+
+  const float sc = p.scale_log2;
+
+  for (int kt = key_begin; kt < key_end; kt += KT) {
+    __syncthreads();
+    // ---- stage K and V tiles ----
+    {
+      int64_t page_row0 = 0;
+      if (PAGED) {
+        int pg = table[kt / p.page_size];
+        page_row0 = (int64_t)pg * p.page_size + (kt % p.page_size);
+      }
+      constexpr int KP = D / 8;
+#pragma unroll
+      for (int j = 0; j < (KT * KP) / 256; j++) {
+        int pc = tid + j * 256;
+        int kr = pc / KP, dp = pc - kr * KP;
+        bf16x8 val = zero_bf16x8();
+        if (kt + kr < key_end) {
+          int64_t row = PAGED ? page_row0 + kr : (int64_t)kbase + kt + kr;
+          val = ld_global_b128(p.k + row * p.k_sr + (int64_t)kh * p.k_sh + dp * 8);
+        }
+        *reinterpret_cast<bf16x8*>(&Ks[kr * KLD + dp * 8]) = val;
+      }
+      constexpr int VP = VD / 8;
+#pragma unroll
+      for (int j = 0; j < (KT * VP) / 256; j++) {
+        int pc = tid + j * 256;
+        int kr = pc / VP, dp = pc - kr * VP;
+        bf16x8 val = zero_bf16x8();
+        if (kt + kr < key_end) {
+          int64_t row = PAGED ? page_row0 + kr : (int64_t)kbase + kt + kr;
+          val = ld_global_b128(p.v + row * p.v_sr + (int64_t)kh * p.v_sh + dp * 8);
+        }
+        *reinterpret_cast<bf16x8*>(&Vs[kr * VLD + dp * 8]) = val;
+      }
+    }
+    __syncthreads();
+    if (!wave_active) continue;
+
+    // wave-uniform visibility classification of this tile
+    bool any_vis, full_vis;
+    if (MODE == MODE_CMP) {
+      any_vis = tw_hi >= p.stride * kt + p.kernel_size - 1;
+      full_vis = (tw_lo >= p.stride * (kt + KT - 1) + p.kernel_size - 1) && (kt + KT <= nkeys);
+    } else {
+      any_vis = (kt <= tw_hi) && (kt + KT - 1 >= tw_lo - p.window);
+      full_vis = (kt + KT - 1 <= tw_lo) && (kt >= tw_hi - p.window);
+    }
+    if (!any_vis) continue;
+
+#pragma unroll
+    for (int rs = 0; rs < RS; rs++) {
+      // ---- S^T = K Q^T : two 32-key sub tiles ----
+      f32x16 sacc[2];
+#pragma unroll
+      for (int nt = 0; nt < 2; nt++) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) sacc[nt][i] = 0.f;
+        const bf16_t* kp = &Ks[(nt * 32 + l32) * KLD + hl * 8];
+#pragma unroll
+        for (int kc = 0; kc < D / 16; kc++) {
+          bf16x8 kf = *reinterpret_cast<const bf16x8*>(kp + kc * 16);
+          sacc[nt] = mfma32(kf, qf[rs][kc], sacc[nt]);
+        }
+      }
+      // ---- scale, mask, online softmax ----
+      const int t = t_row[rs];
+      float tmax = NSA_NEG_INF;
+#pragma unroll
+      for (int nt = 0; nt < 2; nt++) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          float s = sacc[nt][i] * sc;
+          if (!full_vis) {
+            int key = kt + nt * 32 + (i >> 2) * 8 + hl * 4 + (i & 3);
+            bool vis;
+            if (MODE == MODE_CMP) vis = (key < nkeys) && (t >= p.stride * key + p.kernel_size - 1);
+            else vis = (key <= t) && (key >= t - p.window);
+            s = vis ? s : NSA_NEG_INF;
+          }
+          sacc[nt][i] = s;
+          tmax = fmaxf(tmax, s);
+        }
+      }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      float m_new = fmaxf(m_run[rs], tmax);
+      float m_safe = (m_new == NSA_NEG_INF) ? 0.f : m_new;
+      float alpha = fast_exp2(m_run[rs] - m_safe);
+      m_run[rs] = m_new;
+      float psum = 0.f;
+#pragma unroll
+      for (int nt = 0; nt < 2; nt++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          float pv = fast_exp2(sacc[nt][i] - m_safe);
+          sacc[nt][i] = pv;
+          psum += pv;
+        }
+      l_run[rs] = l_run[rs] * alpha + psum;
+#pragma unroll
+      for (int dt = 0; dt < VD / 32; dt++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) oacc[rs][dt][i] *= alpha;
+
+      // ---- O^T += V^T P^T ----
+      const int g16 = lane >> 4, i16 = lane & 15;
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const int nt = c >> 1, ch = c & 1;
+        bf16x8 pf = pack8(sacc[nt][ch * 8 + 0], sacc[nt][ch * 8 + 1], sacc[nt][ch * 8 + 2], sacc[nt][ch * 8 + 3],
+                          sacc[nt][ch * 8 + 4], sacc[nt][ch * 8 + 5], sacc[nt][ch * 8 + 6], sacc[nt][ch * 8 + 7]);
+        const int kb0 = nt * 32 + (2 * ch) * 8 + hl * 4;
+        const int kb1 = kb0 + 8;
+#pragma unroll
+        for (int dt = 0; dt < VD / 32; dt++) {
+          const int col = dt * 32 + (g16 & 1) * 16 + 4 * (i16 & 3);
+          bf16x4 v0 = lds_read_tr(&Vs[(kb0 + (i16 >> 2)) * VLD + col]);
+          bf16x4 v1 = lds_read_tr(&Vs[(kb1 + (i16 >> 2)) * VLD + col]);
+          oacc[rs][dt] = mfma32(cat4(v0, v1), pf, oacc[rs][dt]);
+        }
+      }
+    }
+  }
+
+  // ---- epilogue ----
+#pragma unroll
+  for (int rs = 0; rs < RS; rs++) {
+    float l_tot = l_run[rs] + __shfl_xor(l_run[rs], 32, 64);
+    if (!valid[rs]) continue;
+    float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    bf16_t* op = p.o + tok[rs] * p.o_st + (int64_t)head[rs] * p.o_sh;
+#pragma unroll
+    for (int dt = 0; dt < VD / 32; dt++)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; i4++) {
+        int d = dt * 32 + i4 * 8 + hl * 4;
+        bf16x4 w = pack4(oacc[rs][dt][i4 * 4 + 0] * inv, oacc[rs][dt][i4 * 4 + 1] * inv,
+                         oacc[rs][dt][i4 * 4 + 2] * inv, oacc[rs][dt][i4 * 4 + 3] * inv);
+        *reinterpret_cast<bf16x4*>(op + d) = w;
+      }
+    if (hl == 0 && p.lse != nullptr) {
+      float lse2 = l_tot > 0.f ? m_run[rs] + fast_log2(l_tot) : 0.f;
+      p.lse[tok[rs] * p.lse_st + (int64_t)head[rs] * p.lse_sh] = lse2;
+    }
+  }
+}
+
+template <int D, int VD, int MODE, bool PAGED>
+int launch_fwd_tile(const NsaFwdTileParams& p, int B, int max_q_len, hipStream_t stream) {
+  constexpr int RS = 1;
+  constexpr int ROWS_WG = 128 * RS;
+  if (B <= 0 || max_q_len <= 0) return NSA_OK;
+  dim3 grid(cdiv_i(max_q_len * p.G, ROWS_WG), B, p.KH);
+  fwd_tile_kernel<D, VD, MODE, PAGED, RS><<<grid, 256, 0, stream>>>(p);
+  return nsa_check_launch("fwd_tile_kernel");
+}
+
+template <int MODE, bool PAGED>
+int dispatch_fwd_tile(const NsaFwdTileParams& p, int B, int max_q_len, int D, int VD, hipStream_t stream) {
+  if (D == 128 && VD == 128) return launch_fwd_tile<128, 128, MODE, PAGED>(p, B, max_q_len, stream);
+  if (D == 64 && VD == 64) return launch_fwd_tile<64, 64, MODE, PAGED>(p, B, max_q_len, stream);
+  if (D == 192 && VD == 128) return launch_fwd_tile<192, 128, MODE, PAGED>(p, B, max_q_len, stream);
+  nsa_set_error("attention forward: unsupported head dims D=%d VD=%d (built: 128/128, 64/64, 192/128)", D, VD);
+  return NSA_ERR_UNSUPPORTED;
+}
+
+}  // namespace
+
+int nsa_fwd_tile_launch(const NsaFwdTileParams& p, int mode, bool paged, int B, int max_q_len, int D, int VD,
+                        hipStream_t stream) {
+  if (mode == MODE_CMP) {
+    return paged ? dispatch_fwd_tile<MODE_CMP, true>(p, B, max_q_len, D, VD, stream)
+                 : dispatch_fwd_tile<MODE_CMP, false>(p, B, max_q_len, D, VD, stream);
+  }
+  return paged ? dispatch_fwd_tile<MODE_SWA, true>(p, B, max_q_len, D, VD, stream)
+               : dispatch_fwd_tile<MODE_SWA, false>(p, B, max_q_len, D, VD, stream);
+}

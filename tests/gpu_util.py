@@ -1,0 +1,39 @@
+"""Helpers shared by the GPU parity tests: seeded inputs generated on the CPU (so that oracle and device see the
+same bf16 values) and the tolerance of the parity bar."""
+import numpy as np
+import torch
+
+# parity bar for bf16 outputs and gradients against the fp32 oracle
+ATOL = 2e-2
+RTOL = 1e-2
+
+
+def make_cu(lens):
+    return torch.tensor(np.concatenate([[0], np.cumsum(lens)]), dtype=torch.int32)
+
+
+def randn_bf16(*shape, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g, dtype=torch.float32).to(torch.bfloat16)
+
+
+def make_qkvw(T, QH, KH, D, VD=None, seed=0):
+    VD = D if VD is None else VD
+    q = randn_bf16(T, QH, D, seed=seed)
+    k = randn_bf16(T, KH, D, seed=seed + 1)
+    v = randn_bf16(T, KH, VD, seed=seed + 2)
+    w = randn_bf16(T, QH, 3, seed=seed + 3)
+    return q, k, v, w
+
+
+def assert_close(dev, ref, name, atol=ATOL, rtol=RTOL):
+    dev = dev.detach().float().cpu()
+    ref = ref.detach().float().cpu()
+    assert dev.shape == ref.shape, (name, dev.shape, ref.shape)
+    assert torch.isfinite(dev).all(), f"{name}: non-finite values on device"
+    err = (dev - ref).abs()
+    bound = atol + rtol * ref.abs()
+    bad = err > bound
+    assert not bad.any(), (f"{name}: {int(bad.sum())}/{bad.numel()} outside atol={atol} rtol={rtol}; "
+                           f"max abs err {float(err.max()):.4g} at {np.unravel_index(int(err.argmax()), err.shape)}")
+    return float(err.max())

@@ -1,0 +1,120 @@
+"""GPU parity of the forward operators against the CPU oracle (same seeded bf16 inputs).
+Mirrors upstream test.py --func mean/construct/cmp/topk/slc/combine (test.py:74-318), with asserted tolerances."""
+import pytest
+import torch
+
+from oracle import nsa_oracle as O
+from gpu_util import make_cu, make_qkvw, randn_bf16, assert_close
+
+pytestmark = pytest.mark.gpu
+
+LENS_CASES = [
+    [1000],
+    [5, 31, 32, 47, 48, 100, 333, 700],
+    [64, 0, 129, 513],
+]
+HEAD_CASES = [(16, 1, 128), (8, 2, 128), (4, 4, 64)]
+
+
+def setup_helper(cu_dev, **kw):
+    from flash_nsa import NSAHelper
+    NSAHelper.set_hyperparameters(**kw)
+    NSAHelper.init_cu_seqlens(cu_dev)
+    return NSAHelper
+
+
+@pytest.mark.parametrize("lens", LENS_CASES)
+def test_mean_pooling_and_construct_block(device, lens):
+    from flash_nsa.ops.compress_kv import mean_pooling_fwd, construct_block_fwd
+    cu = make_cu(lens)
+    T = int(cu[-1])
+    x = randn_bf16(T, 4, 128, seed=1)
+    setup_helper(cu.to(device))
+    y = mean_pooling_fwd(x.to(device))
+    ref = O.mean_pooling(x.float(), cu)
+    assert y.shape == ref.shape
+    # fp32 mean rounded to bf16: allow one bf16 ulp of slack for summation order
+    assert_close(y, ref, "mean_pooling", atol=2e-3, rtol=8e-3)
+    blk = construct_block_fwd(x.to(device))
+    refb = O.construct_block(x.float(), cu)
+    assert torch.equal(blk.float().cpu(), refb)
+
+
+@pytest.mark.parametrize("lens", LENS_CASES)
+@pytest.mark.parametrize("QH,KH,D", HEAD_CASES)
+def test_cmp_attn_fwd(device, lens, QH, KH, D):
+    from flash_nsa.ops.compress_kv import mean_pooling_fwd
+    from flash_nsa.ops.compress_attn import cmp_attn_fwd
+    cu = make_cu(lens)
+    T = int(cu[-1])
+    q, k, v, _ = make_qkvw(T, QH, KH, D, seed=10)
+    setup_helper(cu.to(device))
+    ck = mean_pooling_fwd(k.to(device))
+    cv = mean_pooling_fwd(v.to(device))
+    o, lse = cmp_attn_fwd(q.to(device), ck, cv)
+    ro, rl = O.cmp_attn(q.float(), ck.float().cpu(), cv.float().cpu(), cu)
+    assert_close(o, ro, "cmp_o")
+    assert_close(lse, rl, "cmp_lse", atol=1e-3, rtol=1e-4)
+
+
+@pytest.mark.parametrize("lens", LENS_CASES)
+@pytest.mark.parametrize("QH,KH,D", HEAD_CASES)
+def test_swa_fwd(device, lens, QH, KH, D):
+    from flash_nsa.ops.sliding_window_attention import swa_fwd
+    cu = make_cu(lens)
+    T = int(cu[-1])
+    q, k, v, _ = make_qkvw(T, QH, KH, D, seed=20)
+    setup_helper(cu.to(device), window_size=200)
+    o, lse = swa_fwd(q.to(device), k.to(device), v.to(device))
+    ro, rl = O.swa(q.float(), k.float(), v.float(), cu, 200)
+    assert_close(o, ro, "swa_o")
+    assert_close(lse, rl, "swa_lse", atol=1e-3, rtol=1e-4)
+    setup_helper(cu.to(device))
+
+
+@pytest.mark.parametrize("lens", LENS_CASES)
+@pytest.mark.parametrize("QH,KH,D", HEAD_CASES)
+def test_topk_and_slc_fwd(device, lens, QH, KH, D):
+    from flash_nsa.ops.compress_kv import mean_pooling_fwd
+    from flash_nsa.ops.compress_attn import cmp_attn_fwd
+    from flash_nsa.ops.topk import slc_topk_indices
+    from flash_nsa.ops.select_attn import slc_attn_fwd
+    cu = make_cu(lens)
+    T = int(cu[-1])
+    q, k, v, _ = make_qkvw(T, QH, KH, D, seed=30)
+    top_n = 6
+    setup_helper(cu.to(device), top_n=top_n)
+    cfg = O.OracleConfig(top_n=top_n)
+    qd, kd, vd = q.to(device), k.to(device), v.to(device)
+    ck = mean_pooling_fwd(kd)
+    cv = mean_pooling_fwd(vd)
+    _, lse = cmp_attn_fwd(qd, ck, cv)
+    topk, probs = slc_topk_indices(qd, ck, lse, return_slc_prob=True)
+    rt, imps = O.slc_topk(q.float(), ck.float().cpu(), None, cu, cfg, return_importance=True)
+    assert topk.dtype == torch.int32 and topk.shape == (KH, T, top_n)
+    n_rows, n_diff, n_bad = O.topk_mismatch_report(topk.cpu(), rt, imps, cu, 64, top_n, tie_tol=1e-3)
+    assert n_bad == 0, f"{n_bad} rows differ beyond score ties ({n_diff} differing of {n_rows})"
+    assert n_diff <= max(1, n_rows // 200)
+    # slot order and ignore value: rows identical to the oracle wherever the sets agree
+    same = (topk.cpu() == rt).all(-1)
+    assert same.float().mean() > 0.99
+    # block scores returned on request match the oracle's
+    for b in range(len(lens)):
+        a, e = int(cu[b]), int(cu[b + 1])
+        nb = imps[b].shape[-1]
+        if e > a:
+            assert_close(probs[:, a:e, :nb], imps[b], "block scores", atol=2e-3, rtol=2e-3)
+    # selected attention with the device's own indices fed to the oracle
+    o, l2 = slc_attn_fwd(qd, kd, vd, topk)
+    ro, rl = O.slc_attn(q.float(), k.float(), v.float(), topk.cpu(), cu, 64)
+    assert_close(o, ro, "slc_o")
+    assert_close(l2, rl, "slc_lse", atol=1e-3, rtol=1e-4)
+    setup_helper(cu.to(device))
+
+
+def test_combine_fwd(device):
+    from flash_nsa.ops.combine import combine_fwd
+    a, b, c = [randn_bf16(300, 8, 128, seed=s) for s in (1, 2, 3)]
+    w = randn_bf16(300, 8, 3, seed=4)
+    o = combine_fwd(a.to(device), b.to(device), c.to(device), w.to(device))
+    assert_close(o, O.combine(a.float(), b.float(), c.float(), w.float()), "combine")
