@@ -79,6 +79,67 @@ int nsa_slc_attn_fwd(const void* q, int64_t q_st, int64_t q_sh, const void* k, i
                      const int32_t* x_cu, int B, int x_maxlen, int QH, int KH, int D, int VD, int block_size,
                      int top_n, float sm_scale, void* stream);
 
+/* ---- backward ----
+ * dq_mode: 0 = store bf16, 1 = store fp32, 2 = add into an existing fp32 buffer (single writer per element).
+ * delta = rowsum(o * do) of the branch, fp32; lse as produced by the matching forward. */
+
+/* flash_nsa/ops/compress_attn.py:701-736 (_cmp_dq_kernel launch) */
+int nsa_cmp_attn_bwd_dq(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr, int64_t ck_sh,
+                        const void* cv, int64_t cv_sr, int64_t cv_sh, const void* dO, int64_t do_st, int64_t do_sh,
+                        const float* lse, int64_t lse_st, int64_t lse_sh, const float* delta, int64_t delta_st,
+                        int64_t delta_sh, void* dq, int64_t dq_st, int64_t dq_sh, int dq_mode, const int32_t* x_cu,
+                        const int32_t* y_cu, int B, int x_maxlen, int QH, int KH, int D, int VD, int kernel_size,
+                        int stride, float sm_scale, void* stream);
+/* flash_nsa/ops/compress_attn.py:650-690 (_cmp_dkdv_kernel launch, dkdv_repeat=False): fp32 atomic adds into
+ * dck/dcv [y_len,KH,*], which the caller zero-fills; queries are cut into chunks of q_chunk_tokens */
+int nsa_cmp_attn_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr, int64_t ck_sh,
+                          const void* cv, int64_t cv_sr, int64_t cv_sh, const void* dO, int64_t do_st,
+                          int64_t do_sh, const float* lse, int64_t lse_st, int64_t lse_sh, const float* delta,
+                          int64_t delta_st, int64_t delta_sh, float* dck, int64_t dck_sr, int64_t dck_sh,
+                          float* dcv, int64_t dcv_sr, int64_t dcv_sh, const int32_t* x_cu, const int32_t* y_cu,
+                          int B, int x_maxlen, int y_maxlen, int QH, int KH, int D, int VD, int kernel_size,
+                          int stride, int q_chunk_tokens, float sm_scale, void* stream);
+/* flash_nsa/ops/sliding_window_attention.py:98-157 swa_bwd (FlashAttention varlen backward) */
+int nsa_swa_bwd_dq(const void* q, int64_t q_st, int64_t q_sh, const void* k, int64_t k_sr, int64_t k_sh,
+                   const void* v, int64_t v_sr, int64_t v_sh, const void* dO, int64_t do_st, int64_t do_sh,
+                   const float* lse, int64_t lse_st, int64_t lse_sh, const float* delta, int64_t delta_st,
+                   int64_t delta_sh, void* dq, int64_t dq_st, int64_t dq_sh, int dq_mode, const int32_t* x_cu,
+                   int B, int x_maxlen, int QH, int KH, int D, int VD, int window, float sm_scale, void* stream);
+/* same upstream site; dk/dv are stored (every key row has exactly one writer), bf16 or fp32 */
+int nsa_swa_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void* k, int64_t k_sr, int64_t k_sh,
+                     const void* v, int64_t v_sr, int64_t v_sh, const void* dO, int64_t do_st, int64_t do_sh,
+                     const float* lse, int64_t lse_st, int64_t lse_sh, const float* delta, int64_t delta_st,
+                     int64_t delta_sh, void* dk, int64_t dk_sr, int64_t dk_sh, void* dv, int64_t dv_sr,
+                     int64_t dv_sh, int dkv_is_f32, const int32_t* x_cu, int B, int x_maxlen, int QH, int KH, int D,
+                     int VD, int window, float sm_scale, void* stream);
+/* flash_nsa/ops/select_attn.py:650-695 (_dq_kernel launch) */
+int nsa_slc_attn_bwd_dq(const void* q, int64_t q_st, int64_t q_sh, const void* k, int64_t k_sr, int64_t k_sh,
+                        const void* v, int64_t v_sr, int64_t v_sh, const void* dO, int64_t do_st, int64_t do_sh,
+                        const float* lse, int64_t lse_st, int64_t lse_sh, const float* delta, int64_t delta_st,
+                        int64_t delta_sh, const int32_t* topk, int64_t tk_sh, int64_t tk_st, void* dq,
+                        int64_t dq_st, int64_t dq_sh, int dq_mode, const int32_t* x_cu, int B, int x_maxlen, int QH,
+                        int KH, int D, int VD, int block_size, int top_n, float sm_scale, void* stream);
+/* flash_nsa/ops/topk.py:889-945 get_bind_from_find: inverse of the selection as a CSR.
+ *   csr_off  [KH][nblk_total+1] absolute start of each (kv head, global block) list inside csr_tok
+ *   csr_tok  [KH*T*top_n]       query tokens (index local to their sequence), ascending within a list
+ *   item_off [KH][nblk_total+1] prefix count of list chunks of chunk_tokens tokens (work items of the dk/dv pass)
+ *   workspace: int32 scratch of nsa_inverse_index_workspace_elems(T,KH,nblk_total) elements */
+int64_t nsa_inverse_index_workspace_elems(int T, int KH, int nblk_total);
+int nsa_build_inverse_index(const int32_t* topk, int64_t tk_sh, int64_t tk_st, int top_n, const int32_t* x_cu,
+                            const int32_t* kblk_cu, int B, int T, int KH, int nblk_total, int block_size,
+                            int chunk_tokens, int32_t* csr_off, int32_t* csr_tok, int32_t* item_off,
+                            int32_t* workspace, int64_t workspace_elems, void* stream);
+/* flash_nsa/ops/select_attn.py:593-637 (_dkdv_kernel launch): fp32 atomic adds into dk/dv [T,KH,*];
+ * blk_seq [nblk_total] = sequence of each global block; n_items_bound >= max over kv heads of item_off[kh][nblk_total] */
+int nsa_slc_attn_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void* k, int64_t k_sr, int64_t k_sh,
+                          const void* v, int64_t v_sr, int64_t v_sh, const void* dO, int64_t do_st,
+                          int64_t do_sh, const float* lse, int64_t lse_st, int64_t lse_sh, const float* delta,
+                          int64_t delta_st, int64_t delta_sh, float* dk, int64_t dk_sr, int64_t dk_sh, float* dv,
+                          int64_t dv_sr, int64_t dv_sh, const int32_t* x_cu, const int32_t* kblk_cu,
+                          const int32_t* blk_seq, const int32_t* csr_off, const int32_t* csr_tok,
+                          const int32_t* item_off, int nblk_total, int chunk_tokens, int n_items_bound, int B,
+                          int QH, int KH, int D, int VD, int block_size, float sm_scale, void* stream);
+
 /* flash_nsa/inference/compress_kv.py:191-220 mean_pooling_prefill (in-pool write at flat row slot) */
 int nsa_paged_pool_prefill(void* cache, int64_t c_sr, int64_t c_sh, const int32_t* y_cu, const int32_t* block_tables,
                            int table_stride, const int32_t* cmp_slot_mapping, int B, int y_maxlen, int page_size,

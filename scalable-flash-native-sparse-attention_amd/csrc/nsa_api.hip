@@ -142,3 +142,163 @@ int nsa_slc_attn_fwd(const void* q, int64_t q_st, int64_t q_sh, const void* k, i
 }
 
 }  // extern "C"
+
+// ------------------------------------------------------------------------------------------------ backward
+namespace {
+struct BwdCommon {
+  const void* q; int64_t q_st, q_sh;
+  const void* k; int64_t k_sr, k_sh;
+  const void* v; int64_t v_sr, v_sh;
+  const void* dO; int64_t do_st, do_sh;
+  const float* lse; int64_t lse_st, lse_sh;
+  const float* delta; int64_t delta_st, delta_sh;
+};
+NsaBwdTileParams make_bwd(const BwdCommon& c, int QH, int KH, float sm_scale) {
+  NsaBwdTileParams p{};
+  p.q = (const bf16_t*)c.q; p.q_st = c.q_st; p.q_sh = c.q_sh;
+  p.k = (const bf16_t*)c.k; p.k_sr = c.k_sr; p.k_sh = c.k_sh;
+  p.v = (const bf16_t*)c.v; p.v_sr = c.v_sr; p.v_sh = c.v_sh;
+  p.dO = (const bf16_t*)c.dO; p.do_st = c.do_st; p.do_sh = c.do_sh;
+  p.lse = c.lse; p.lse_st = c.lse_st; p.lse_sh = c.lse_sh;
+  p.delta = c.delta; p.delta_st = c.delta_st; p.delta_sh = c.delta_sh;
+  p.G = QH / KH; p.KH = KH;
+  p.scale_log2 = sm_scale * NSA_LOG2E; p.sm_scale = sm_scale;
+  p.kernel_size = 1; p.stride = 1; p.window = 0;
+  return p;
+}
+}  // namespace
+
+extern "C" {
+
+int nsa_cmp_attn_bwd_dq(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr, int64_t ck_sh,
+                        const void* cv, int64_t cv_sr, int64_t cv_sh, const void* dO, int64_t do_st, int64_t do_sh,
+                        const float* lse, int64_t lse_st, int64_t lse_sh, const float* delta, int64_t delta_st,
+                        int64_t delta_sh, void* dq, int64_t dq_st, int64_t dq_sh, int dq_mode, const int32_t* x_cu,
+                        const int32_t* y_cu, int B, int x_maxlen, int QH, int KH, int D, int VD, int kernel_size,
+                        int stride, float sm_scale, void* stream) {
+  int rc = check_heads("cmp_attn_bwd_dq", QH, KH, D, VD);
+  if (rc) return rc;
+  rc = check_nsa_sizes("cmp_attn_bwd_dq", kernel_size, stride, 0);
+  if (rc) return rc;
+  NSA_REQUIRE(dq_mode >= 0 && dq_mode <= 2, NSA_ERR_BAD_ARG, "cmp_attn_bwd_dq: dq_mode %d not in {0,1,2}", dq_mode);
+  BwdCommon c{q, q_st, q_sh, ck, ck_sr, ck_sh, cv, cv_sr, cv_sh, dO, do_st, do_sh, lse, lse_st, lse_sh, delta,
+              delta_st, delta_sh};
+  NsaBwdTileParams p = make_bwd(c, QH, KH, sm_scale);
+  p.dq = dq; p.dq_st = dq_st; p.dq_sh = dq_sh; p.dq_mode = dq_mode;
+  p.x_cu = x_cu; p.k_cu = y_cu;
+  p.kernel_size = kernel_size; p.stride = stride;
+  return nsa_bwd_dq_tile_launch(p, 0, B, x_maxlen, D, VD, (hipStream_t)stream);
+}
+
+int nsa_cmp_attn_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr, int64_t ck_sh,
+                          const void* cv, int64_t cv_sr, int64_t cv_sh, const void* dO, int64_t do_st,
+                          int64_t do_sh, const float* lse, int64_t lse_st, int64_t lse_sh, const float* delta,
+                          int64_t delta_st, int64_t delta_sh, float* dck, int64_t dck_sr, int64_t dck_sh,
+                          float* dcv, int64_t dcv_sr, int64_t dcv_sh, const int32_t* x_cu, const int32_t* y_cu,
+                          int B, int x_maxlen, int y_maxlen, int QH, int KH, int D, int VD, int kernel_size,
+                          int stride, int q_chunk_tokens, float sm_scale, void* stream) {
+  int rc = check_heads("cmp_attn_bwd_dkdv", QH, KH, D, VD);
+  if (rc) return rc;
+  rc = check_nsa_sizes("cmp_attn_bwd_dkdv", kernel_size, stride, 0);
+  if (rc) return rc;
+  NSA_REQUIRE(q_chunk_tokens > 0, NSA_ERR_BAD_ARG, "cmp_attn_bwd_dkdv: q_chunk_tokens must be positive");
+  BwdCommon c{q, q_st, q_sh, ck, ck_sr, ck_sh, cv, cv_sr, cv_sh, dO, do_st, do_sh, lse, lse_st, lse_sh, delta,
+              delta_st, delta_sh};
+  NsaBwdTileParams p = make_bwd(c, QH, KH, sm_scale);
+  p.dk = dck; p.dk_sr = dck_sr; p.dk_sh = dck_sh;
+  p.dv = dcv; p.dv_sr = dcv_sr; p.dv_sh = dcv_sh;
+  p.dkv_mode = 3;
+  p.x_cu = x_cu; p.k_cu = y_cu;
+  p.kernel_size = kernel_size; p.stride = stride;
+  p.q_chunk_tokens = q_chunk_tokens;
+  return nsa_bwd_dkdv_launch(p, 0, B, x_maxlen, y_maxlen, D, VD, 0, (hipStream_t)stream);
+}
+
+int nsa_swa_bwd_dq(const void* q, int64_t q_st, int64_t q_sh, const void* k, int64_t k_sr, int64_t k_sh,
+                   const void* v, int64_t v_sr, int64_t v_sh, const void* dO, int64_t do_st, int64_t do_sh,
+                   const float* lse, int64_t lse_st, int64_t lse_sh, const float* delta, int64_t delta_st,
+                   int64_t delta_sh, void* dq, int64_t dq_st, int64_t dq_sh, int dq_mode, const int32_t* x_cu,
+                   int B, int x_maxlen, int QH, int KH, int D, int VD, int window, float sm_scale, void* stream) {
+  int rc = check_heads("swa_bwd_dq", QH, KH, D, VD);
+  if (rc) return rc;
+  NSA_REQUIRE(dq_mode >= 0 && dq_mode <= 2, NSA_ERR_BAD_ARG, "swa_bwd_dq: dq_mode %d not in {0,1,2}", dq_mode);
+  BwdCommon c{q, q_st, q_sh, k, k_sr, k_sh, v, v_sr, v_sh, dO, do_st, do_sh, lse, lse_st, lse_sh, delta, delta_st,
+              delta_sh};
+  NsaBwdTileParams p = make_bwd(c, QH, KH, sm_scale);
+  p.dq = dq; p.dq_st = dq_st; p.dq_sh = dq_sh; p.dq_mode = dq_mode;
+  p.x_cu = x_cu; p.k_cu = x_cu;
+  p.window = window;
+  return nsa_bwd_dq_tile_launch(p, 1, B, x_maxlen, D, VD, (hipStream_t)stream);
+}
+
+int nsa_swa_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void* k, int64_t k_sr, int64_t k_sh,
+                     const void* v, int64_t v_sr, int64_t v_sh, const void* dO, int64_t do_st, int64_t do_sh,
+                     const float* lse, int64_t lse_st, int64_t lse_sh, const float* delta, int64_t delta_st,
+                     int64_t delta_sh, void* dk, int64_t dk_sr, int64_t dk_sh, void* dv, int64_t dv_sr,
+                     int64_t dv_sh, int dkv_is_f32, const int32_t* x_cu, int B, int x_maxlen, int QH, int KH, int D,
+                     int VD, int window, float sm_scale, void* stream) {
+  int rc = check_heads("swa_bwd_dkdv", QH, KH, D, VD);
+  if (rc) return rc;
+  BwdCommon c{q, q_st, q_sh, k, k_sr, k_sh, v, v_sr, v_sh, dO, do_st, do_sh, lse, lse_st, lse_sh, delta, delta_st,
+              delta_sh};
+  NsaBwdTileParams p = make_bwd(c, QH, KH, sm_scale);
+  p.dk = dk; p.dk_sr = dk_sr; p.dk_sh = dk_sh;
+  p.dv = dv; p.dv_sr = dv_sr; p.dv_sh = dv_sh;
+  p.dkv_mode = dkv_is_f32 ? 1 : 0;
+  p.x_cu = x_cu; p.k_cu = x_cu;
+  p.window = window;
+  return nsa_bwd_dkdv_launch(p, 1, B, x_maxlen, x_maxlen, D, VD, 0, (hipStream_t)stream);
+}
+
+int nsa_slc_attn_bwd_dq(const void* q, int64_t q_st, int64_t q_sh, const void* k, int64_t k_sr, int64_t k_sh,
+                        const void* v, int64_t v_sr, int64_t v_sh, const void* dO, int64_t do_st, int64_t do_sh,
+                        const float* lse, int64_t lse_st, int64_t lse_sh, const float* delta, int64_t delta_st,
+                        int64_t delta_sh, const int32_t* topk, int64_t tk_sh, int64_t tk_st, void* dq,
+                        int64_t dq_st, int64_t dq_sh, int dq_mode, const int32_t* x_cu, int B, int x_maxlen, int QH,
+                        int KH, int D, int VD, int block_size, int top_n, float sm_scale, void* stream) {
+  int rc = check_heads("slc_attn_bwd_dq", QH, KH, D, VD);
+  if (rc) return rc;
+  NSA_REQUIRE(block_size % 64 == 0 && block_size > 0, NSA_ERR_UNSUPPORTED,
+              "slc_attn_bwd_dq: block_size %d must be a multiple of 64", block_size);
+  NSA_REQUIRE(top_n >= 1 && top_n <= 64, NSA_ERR_BAD_ARG, "slc_attn_bwd_dq: top_n %d must be in [1,64]", top_n);
+  NSA_REQUIRE(dq_mode >= 0 && dq_mode <= 2, NSA_ERR_BAD_ARG, "slc_attn_bwd_dq: dq_mode %d not in {0,1,2}", dq_mode);
+  NsaSlcBwdDqParams p{};
+  p.q = (const bf16_t*)q; p.q_st = q_st; p.q_sh = q_sh;
+  p.k = (const bf16_t*)k; p.k_sr = k_sr; p.k_sh = k_sh;
+  p.v = (const bf16_t*)v; p.v_sr = v_sr; p.v_sh = v_sh;
+  p.dO = (const bf16_t*)dO; p.do_st = do_st; p.do_sh = do_sh;
+  p.lse = lse; p.lse_st = lse_st; p.lse_sh = lse_sh;
+  p.delta = delta; p.delta_st = delta_st; p.delta_sh = delta_sh;
+  p.dq = dq; p.dq_st = dq_st; p.dq_sh = dq_sh; p.dq_mode = dq_mode;
+  p.topk = topk; p.tk_sh = tk_sh; p.tk_st = tk_st;
+  p.x_cu = x_cu;
+  p.G = QH / KH; p.KH = KH; p.top_n = top_n; p.block_size = block_size;
+  p.scale_log2 = sm_scale * NSA_LOG2E; p.sm_scale = sm_scale;
+  return nsa_slc_bwd_dq_launch(p, B, x_maxlen, D, VD, (hipStream_t)stream);
+}
+
+int nsa_slc_attn_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void* k, int64_t k_sr, int64_t k_sh,
+                          const void* v, int64_t v_sr, int64_t v_sh, const void* dO, int64_t do_st,
+                          int64_t do_sh, const float* lse, int64_t lse_st, int64_t lse_sh, const float* delta,
+                          int64_t delta_st, int64_t delta_sh, float* dk, int64_t dk_sr, int64_t dk_sh, float* dv,
+                          int64_t dv_sr, int64_t dv_sh, const int32_t* x_cu, const int32_t* kblk_cu,
+                          const int32_t* blk_seq, const int32_t* csr_off, const int32_t* csr_tok,
+                          const int32_t* item_off, int nblk_total, int chunk_tokens, int n_items_bound, int B,
+                          int QH, int KH, int D, int VD, int block_size, float sm_scale, void* stream) {
+  int rc = check_heads("slc_attn_bwd_dkdv", QH, KH, D, VD);
+  if (rc) return rc;
+  NSA_REQUIRE(block_size == 64 || block_size == 128, NSA_ERR_UNSUPPORTED,
+              "slc_attn_bwd_dkdv: block_size %d not built (64 or 128)", block_size);
+  BwdCommon c{q, q_st, q_sh, k, k_sr, k_sh, v, v_sr, v_sh, dO, do_st, do_sh, lse, lse_st, lse_sh, delta, delta_st,
+              delta_sh};
+  NsaBwdTileParams p = make_bwd(c, QH, KH, sm_scale);
+  p.dk = dk; p.dk_sr = dk_sr; p.dk_sh = dk_sh;
+  p.dv = dv; p.dv_sr = dv_sr; p.dv_sh = dv_sh;
+  p.dkv_mode = 3;
+  p.x_cu = x_cu; p.k_cu = x_cu;
+  p.csr_off = csr_off; p.csr_tok = csr_tok; p.item_off = item_off; p.blk_seq = blk_seq; p.kblk_cu = kblk_cu;
+  p.nblk_total = nblk_total; p.chunk_tokens = chunk_tokens; p.block_size = block_size;
+  return nsa_bwd_dkdv_launch(p, 2, B, 0, 0, D, VD, n_items_bound, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -54,3 +54,51 @@ int nsa_fwd_tile_launch(const NsaFwdTileParams& p, int mode, bool paged, int B, 
                         hipStream_t stream);
 int nsa_slc_fwd_launch(const NsaSlcParams& p, bool paged, int B, int max_q_len, int D, int VD, hipStream_t stream);
 int nsa_topk_launch(const NsaTopkParams& p, bool paged, int B, int max_q_len, int D, hipStream_t stream);
+
+// backward of the range-keyed branches and of the gathered (selected) branch
+struct NsaBwdTileParams {
+  const bf16_t* q; int64_t q_st, q_sh;
+  const bf16_t* k; int64_t k_sr, k_sh;
+  const bf16_t* v; int64_t v_sr, v_sh;
+  const bf16_t* dO; int64_t do_st, do_sh;
+  const float* lse; int64_t lse_st, lse_sh;
+  const float* delta; int64_t delta_st, delta_sh;
+  void* dq; int64_t dq_st, dq_sh; int dq_mode;      // 0: store bf16, 1: store fp32, 2: add into fp32
+  void* dk; int64_t dk_sr, dk_sh;                   // dkdv kernels
+  void* dv; int64_t dv_sr, dv_sh;
+  int dkv_mode;                                     // 0: store bf16, 1: store fp32, 3: atomic add into fp32
+  const int32_t* x_cu;
+  const int32_t* k_cu;
+  // gathered (selected-attention) row lists: CSR over (kv head, global selection block)
+  const int32_t* csr_off;      // [KH][nblk_total + 1] absolute positions into csr_tok
+  const int32_t* csr_tok;      // [KH * T * top_n] local token index inside its sequence, ascending per list
+  const int32_t* item_off;     // [KH][nblk_total + 1] prefix of work items (list chunks)
+  const int32_t* blk_seq;      // [nblk_total] sequence id of a global block
+  const int32_t* kblk_cu;      // [B+1] selection-block offsets
+  int nblk_total, chunk_tokens, block_size;
+  int G, KH;
+  float scale_log2, sm_scale;
+  int kernel_size, stride, window;
+  int q_chunk_tokens;          // compressed dkdv: query tokens per grid.x chunk
+  int grid_chunks;             // compressed dkdv: chunks per key tile in grid.x (set by the launcher)
+};
+
+int nsa_bwd_dq_tile_launch(const NsaBwdTileParams& p, int mode, int B, int max_q_len, int D, int VD,
+                           hipStream_t stream);
+int nsa_bwd_dkdv_launch(const NsaBwdTileParams& p, int mode, int B, int max_q_len, int max_k_len, int D, int VD,
+                        int n_items_bound, hipStream_t stream);
+
+struct NsaSlcBwdDqParams {
+  const bf16_t* q; int64_t q_st, q_sh;
+  const bf16_t* k; int64_t k_sr, k_sh;
+  const bf16_t* v; int64_t v_sr, v_sh;
+  const bf16_t* dO; int64_t do_st, do_sh;
+  const float* lse; int64_t lse_st, lse_sh;
+  const float* delta; int64_t delta_st, delta_sh;
+  void* dq; int64_t dq_st, dq_sh; int dq_mode;
+  const int32_t* topk; int64_t tk_sh, tk_st;
+  const int32_t* x_cu;
+  int G, KH, top_n, block_size;
+  float scale_log2, sm_scale;
+};
+int nsa_slc_bwd_dq_launch(const NsaSlcBwdDqParams& p, int B, int max_q_len, int D, int VD, hipStream_t stream);

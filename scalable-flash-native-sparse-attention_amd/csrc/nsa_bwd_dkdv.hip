@@ -1,0 +1,319 @@
+// dK / dV of all three attention branches.  A workgroup owns NW*32 keys (each wave 32 keys whose K and V
+// fragments stay in registers as MFMA B operands) and streams tiles of 64 query rows through LDS; a "row" is a
+// (query token, q-head) pair of the kv-head group, so the GQA reduction over heads happens in the accumulators.
+//   S = Q K^T,  P = exp2(S*c - lse),  dP = dO V^T,  dS = P o (dP - delta),
+//   dV^T += dO^T P,  dK^T += Q^T dS      (Q^T / dO^T fragments via ds_read_b64_tr_b16)
+// MODE_CMP: rows are all later queries of the sequence, split in chunks over grid.x, fp32 atomics
+//           (upstream flash_nsa/ops/compress_attn.py:193-376)
+// MODE_SWA: rows are the <= W+NW*32 queries whose window contains the keys, plain stores
+//           (upstream: FlashAttention backward, flash_nsa/ops/sliding_window_attention.py:98-157)
+// MODE_SLC: rows are gathered through the inverse index (selection block -> tokens that selected it), lists are
+//           cut into chunks over grid.x, fp32 atomics (upstream flash_nsa/ops/select_attn.py:147-328)
+#include "nsa_common.h"
+#include "nsa_api_internal.h"
+
+namespace {
+
+constexpr int MODE_CMP = 0;
+constexpr int MODE_SWA = 1;
+constexpr int MODE_SLC = 2;
+
+template <int D, int VD, int MODE, int NW>
+__global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
+  constexpr int NT = NW * 64;
+  constexpr int KW = NW * 32;
+  constexpr int RT = 64;
+  constexpr int QLD = D + 8;
+  constexpr int OLD = VD + 8;
+  __shared__ __attribute__((aligned(16))) bf16_t Qs[RT * QLD];
+  __shared__ __attribute__((aligned(16))) bf16_t dOs[RT * OLD];
+  __shared__ __attribute__((aligned(16))) float lse_s[RT];
+  __shared__ __attribute__((aligned(16))) float delta_s[RT];
+  __shared__ __attribute__((aligned(16))) int t_s[RT];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int l32 = lane & 31;
+  const int hl = lane >> 5;
+  const int g16 = lane >> 4, i16 = lane & 15;
+  const int kh = blockIdx.z;
+  const int G = p.G;
+
+  int b, key0, row_begin, row_end;  // rows in the group-row space of sequence b (MODE_SLC: positions in the list)
+  const int32_t* list = nullptr;
+  if (MODE == MODE_SLC) {
+    const int32_t* ioff = p.item_off + (int64_t)kh * (p.nblk_total + 1);
+    const int w = blockIdx.x;
+    if (w >= ioff[p.nblk_total]) return;
+    int lo = 0, hi = p.nblk_total;  // last jb with ioff[jb] <= w
+    while (hi - lo > 1) {
+      int mid = (lo + hi) >> 1;
+      if (ioff[mid] <= w) lo = mid; else hi = mid;
+    }
+    const int jb = lo;
+    const int c = w - ioff[jb];
+    b = p.blk_seq[jb];
+    key0 = (jb - p.kblk_cu[b]) * p.block_size;
+    const int s0 = p.csr_off[(int64_t)kh * (p.nblk_total + 1) + jb];
+    const int s1 = p.csr_off[(int64_t)kh * (p.nblk_total + 1) + jb + 1];
+    const int a = s0 + c * p.chunk_tokens;
+    list = p.csr_tok + a;
+    row_begin = 0;
+    row_end = (min(s1, a + p.chunk_tokens) - a) * G;
+  } else {
+    b = blockIdx.y;
+  }
+  const int x0 = p.x_cu[b];
+  const int xl = p.x_cu[b + 1] - x0;
+  int nkeys, kbase;
+  if (MODE == MODE_CMP) {
+    kbase = p.k_cu[b];
+    nkeys = p.k_cu[b + 1] - kbase;
+    const int nch = cdiv_i(xl, p.q_chunk_tokens);
+    const int ktile = blockIdx.x / p.grid_chunks;
+    const int ch = blockIdx.x - ktile * p.grid_chunks;
+    key0 = ktile * KW;
+    if (key0 >= nkeys || ch >= nch) return;
+    const int first = p.stride * key0 + p.kernel_size - 1;
+    const int ta = max(ch * p.q_chunk_tokens, first);
+    const int tb = min((ch + 1) * p.q_chunk_tokens, xl);
+    if (ta >= tb) return;
+    row_begin = ta * G;
+    row_end = tb * G;
+  } else {
+    kbase = x0;
+    nkeys = xl;
+    if (MODE == MODE_SWA) {
+      key0 = blockIdx.x * KW;
+      if (key0 >= nkeys) return;
+      row_begin = key0 * G;
+      row_end = min(xl, key0 + KW + p.window) * G;
+    } else if (key0 >= nkeys) {
+      return;
+    }
+  }
+
+  // ---- this wave's keys: K and V fragments as B operands ----
+  const int kw0 = key0 + wave * 32;
+  const int my_key = kw0 + l32;
+  bf16x8 kf[D / 16], vf[VD / 16];
+  {
+    const int kr = min(my_key, nkeys - 1);
+    const bf16_t* kp = p.k + ((int64_t)kbase + kr) * p.k_sr + (int64_t)kh * p.k_sh + hl * 8;
+#pragma unroll
+    for (int kc = 0; kc < D / 16; kc++) kf[kc] = ld_global_b128(kp + kc * 16);
+    const bf16_t* vp = p.v + ((int64_t)kbase + kr) * p.v_sr + (int64_t)kh * p.v_sh + hl * 8;
+#pragma unroll
+    for (int kc = 0; kc < VD / 16; kc++) vf[kc] = ld_global_b128(vp + kc * 16);
+  }
+  f32x16 dkacc[D / 32], dvacc[VD / 32];
+#pragma unroll
+  for (int dt = 0; dt < D / 32; dt++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) dkacc[dt][i] = 0.f;
+#pragma unroll
+  for (int dt = 0; dt < VD / 32; dt++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) dvacc[dt][i] = 0.f;
+  const float sc = p.scale_log2;
+  const bool wave_has_keys = kw0 < nkeys;
+
+  for (int rt0 = row_begin; rt0 < row_end; rt0 += RT) {
+    __syncthreads();
+    // ---- stage 64 rows of Q, dO, lse, delta, position ----
+    {
+      constexpr int QP = D / 8;
+#pragma unroll
+      for (int j = 0; j < (RT * QP) / NT; j++) {
+        int pc = tid + j * NT;
+        int rl = pc / QP, dp = pc - rl * QP;
+        int rr = rt0 + rl;
+        bf16x8 val = zero_bf16x8();
+        if (rr < row_end) {
+          int n = rr / G, g = rr - n * G;
+          if (MODE == MODE_SLC) n = list[n];
+          val = ld_global_b128(p.q + (int64_t)(x0 + n) * p.q_st + (int64_t)(kh * G + g) * p.q_sh + dp * 8);
+        }
+        *reinterpret_cast<bf16x8*>(&Qs[rl * QLD + dp * 8]) = val;
+      }
+      constexpr int OP = VD / 8;
+#pragma unroll
+      for (int j = 0; j < (RT * OP) / NT; j++) {
+        int pc = tid + j * NT;
+        int rl = pc / OP, dp = pc - rl * OP;
+        int rr = rt0 + rl;
+        bf16x8 val = zero_bf16x8();
+        if (rr < row_end) {
+          int n = rr / G, g = rr - n * G;
+          if (MODE == MODE_SLC) n = list[n];
+          val = ld_global_b128(p.dO + (int64_t)(x0 + n) * p.do_st + (int64_t)(kh * G + g) * p.do_sh + dp * 8);
+        }
+        *reinterpret_cast<bf16x8*>(&dOs[rl * OLD + dp * 8]) = val;
+      }
+      if (tid < RT) {
+        int rr = rt0 + tid;
+        float l = 0.f, dl = 0.f;
+        int tt = -0x40000000;
+        if (rr < row_end) {
+          int n = rr / G, g = rr - n * G;
+          if (MODE == MODE_SLC) n = list[n];
+          int64_t tok = x0 + n;
+          int head = kh * G + g;
+          l = p.lse[tok * p.lse_st + (int64_t)head * p.lse_sh];
+          dl = p.delta[tok * p.delta_st + (int64_t)head * p.delta_sh];
+          tt = n;
+        }
+        lse_s[tid] = l;
+        delta_s[tid] = dl;
+        t_s[tid] = tt;
+      }
+    }
+    __syncthreads();
+    if (!wave_has_keys) continue;
+
+    // tile position range (rows ascend in position for all three modes)
+    const int t_min = t_s[0];
+    const int n_in = min(RT, row_end - rt0);
+    const int t_max = t_s[n_in - 1];
+    bool any_vis, full_vis;
+    if (MODE == MODE_CMP) {
+      any_vis = t_max >= p.stride * kw0 + p.kernel_size - 1;
+      full_vis = (n_in == RT) && (t_min >= p.stride * (kw0 + 31) + p.kernel_size - 1) && (kw0 + 31 < nkeys);
+    } else if (MODE == MODE_SWA) {
+      any_vis = (kw0 <= t_max) && (kw0 + 31 >= t_min - p.window);
+      full_vis = (n_in == RT) && (kw0 + 31 <= t_min) && (kw0 >= t_max - p.window) && (kw0 + 31 < nkeys);
+    } else {
+      any_vis = kw0 <= t_max;
+      full_vis = (n_in == RT) && (kw0 + 31 <= t_min) && (kw0 + 31 < nkeys);
+    }
+    if (!any_vis) continue;
+
+#pragma unroll
+    for (int mt = 0; mt < 2; mt++) {
+      f32x16 sacc, pacc;
+#pragma unroll
+      for (int i = 0; i < 16; i++) { sacc[i] = 0.f; pacc[i] = 0.f; }
+      const bf16_t* qp = &Qs[(mt * 32 + l32) * QLD + hl * 8];
+#pragma unroll
+      for (int kc = 0; kc < D / 16; kc++)
+        sacc = mfma32(*reinterpret_cast<const bf16x8*>(qp + kc * 16), kf[kc], sacc);
+      const bf16_t* dp = &dOs[(mt * 32 + l32) * OLD + hl * 8];
+#pragma unroll
+      for (int kc = 0; kc < VD / 16; kc++)
+        pacc = mfma32(*reinterpret_cast<const bf16x8*>(dp + kc * 16), vf[kc], pacc);
+#pragma unroll
+      for (int i4 = 0; i4 < 4; i4++) {
+        const int rbase = mt * 32 + i4 * 8 + hl * 4;
+        f32x4 l4 = *reinterpret_cast<const f32x4*>(&lse_s[rbase]);
+        f32x4 d4 = *reinterpret_cast<const f32x4*>(&delta_s[rbase]);
+#pragma unroll
+        for (int ii = 0; ii < 4; ii++) {
+          const int i = i4 * 4 + ii;
+          bool vis = true;
+          if (!full_vis) {
+            int tr = t_s[rbase + ii];
+            if (MODE == MODE_CMP) vis = (my_key < nkeys) && (tr >= p.stride * my_key + p.kernel_size - 1);
+            else if (MODE == MODE_SWA) vis = (my_key <= tr) && (my_key >= tr - p.window);
+            else vis = (my_key <= tr);
+          }
+          float pv = vis ? fast_exp2(sacc[i] * sc - l4[ii]) : 0.f;
+          sacc[i] = pv;
+          pacc[i] = pv * (pacc[i] - d4[ii]);
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < 2; c++) {
+        bf16x8 pf = pack8(sacc[c * 8 + 0], sacc[c * 8 + 1], sacc[c * 8 + 2], sacc[c * 8 + 3], sacc[c * 8 + 4],
+                          sacc[c * 8 + 5], sacc[c * 8 + 6], sacc[c * 8 + 7]);
+        bf16x8 df = pack8(pacc[c * 8 + 0], pacc[c * 8 + 1], pacc[c * 8 + 2], pacc[c * 8 + 3], pacc[c * 8 + 4],
+                          pacc[c * 8 + 5], pacc[c * 8 + 6], pacc[c * 8 + 7]);
+        const int rb0 = mt * 32 + (2 * c) * 8 + hl * 4 + (i16 >> 2);
+        const int rb1 = rb0 + 8;
+#pragma unroll
+        for (int dt = 0; dt < VD / 32; dt++) {
+          const int col = dt * 32 + (g16 & 1) * 16 + 4 * (i16 & 3);
+          bf16x4 a0 = lds_read_tr(&dOs[rb0 * OLD + col]);
+          bf16x4 a1 = lds_read_tr(&dOs[rb1 * OLD + col]);
+          dvacc[dt] = mfma32(cat4(a0, a1), pf, dvacc[dt]);
+        }
+#pragma unroll
+        for (int dt = 0; dt < D / 32; dt++) {
+          const int col = dt * 32 + (g16 & 1) * 16 + 4 * (i16 & 3);
+          bf16x4 a0 = lds_read_tr(&Qs[rb0 * QLD + col]);
+          bf16x4 a1 = lds_read_tr(&Qs[rb1 * QLD + col]);
+          dkacc[dt] = mfma32(cat4(a0, a1), df, dkacc[dt]);
+        }
+      }
+    }
+  }
+
+  if (my_key >= nkeys) return;
+  const float osc = p.sm_scale;
+  const int64_t koff = ((int64_t)kbase + my_key) * p.dk_sr + (int64_t)kh * p.dk_sh;
+  const int64_t voff = ((int64_t)kbase + my_key) * p.dv_sr + (int64_t)kh * p.dv_sh;
+  auto emit = [&](void* base, int64_t off, f32x4 val) {
+    if (p.dkv_mode == 0) {
+      *reinterpret_cast<bf16x4*>((bf16_t*)base + off) = pack4(val[0], val[1], val[2], val[3]);
+    } else if (p.dkv_mode == 1) {
+      *reinterpret_cast<f32x4*>((float*)base + off) = val;
+    } else {
+      float* dst = (float*)base + off;
+#pragma unroll
+      for (int e = 0; e < 4; e++) unsafeAtomicAdd(dst + e, val[e]);
+    }
+  };
+#pragma unroll
+  for (int dt = 0; dt < D / 32; dt++)
+#pragma unroll
+    for (int i4 = 0; i4 < 4; i4++) {
+      int d = dt * 32 + i4 * 8 + hl * 4;
+      emit(p.dk, koff + d, f32x4{dkacc[dt][i4 * 4 + 0] * osc, dkacc[dt][i4 * 4 + 1] * osc,
+                                 dkacc[dt][i4 * 4 + 2] * osc, dkacc[dt][i4 * 4 + 3] * osc});
+    }
+#pragma unroll
+  for (int dt = 0; dt < VD / 32; dt++)
+#pragma unroll
+    for (int i4 = 0; i4 < 4; i4++) {
+      int d = dt * 32 + i4 * 8 + hl * 4;
+      emit(p.dv, voff + d, f32x4{dvacc[dt][i4 * 4 + 0], dvacc[dt][i4 * 4 + 1], dvacc[dt][i4 * 4 + 2],
+                                 dvacc[dt][i4 * 4 + 3]});
+    }
+}
+
+template <int D, int VD>
+int launch(const NsaBwdTileParams& p0, int mode, int B, int max_q_len, int max_k_len, int n_items_bound,
+           hipStream_t stream) {
+  NsaBwdTileParams p = p0;
+  if (mode == MODE_CMP) {
+    if (B <= 0 || max_k_len <= 0) return NSA_OK;
+    p.grid_chunks = cdiv_i(max_q_len, p.q_chunk_tokens);
+    dim3 grid(cdiv_i(max_k_len, 128) * p.grid_chunks, B, p.KH);
+    bwd_dkdv_kernel<D, VD, MODE_CMP, 4><<<grid, 256, 0, stream>>>(p);
+  } else if (mode == MODE_SWA) {
+    if (B <= 0 || max_k_len <= 0) return NSA_OK;
+    dim3 grid(cdiv_i(max_k_len, 128), B, p.KH);
+    bwd_dkdv_kernel<D, VD, MODE_SWA, 4><<<grid, 256, 0, stream>>>(p);
+  } else {
+    if (n_items_bound <= 0) return NSA_OK;
+    dim3 grid(n_items_bound, 1, p.KH);
+    if (p.block_size == 64) bwd_dkdv_kernel<D, VD, MODE_SLC, 2><<<grid, 128, 0, stream>>>(p);
+    else if (p.block_size == 128) bwd_dkdv_kernel<D, VD, MODE_SLC, 4><<<grid, 256, 0, stream>>>(p);
+    else {
+      nsa_set_error("selected attention dk/dv: block_size %d not built (64 or 128)", p.block_size);
+      return NSA_ERR_UNSUPPORTED;
+    }
+  }
+  return nsa_check_launch("bwd_dkdv_kernel");
+}
+
+}  // namespace
+
+int nsa_bwd_dkdv_launch(const NsaBwdTileParams& p, int mode, int B, int max_q_len, int max_k_len, int D, int VD,
+                        int n_items_bound, hipStream_t stream) {
+  if (D == 128 && VD == 128) return launch<128, 128>(p, mode, B, max_q_len, max_k_len, n_items_bound, stream);
+  if (D == 64 && VD == 64) return launch<64, 64>(p, mode, B, max_q_len, max_k_len, n_items_bound, stream);
+  if (D == 192 && VD == 128) return launch<192, 128>(p, mode, B, max_q_len, max_k_len, n_items_bound, stream);
+  nsa_set_error("attention dk/dv: unsupported head dims D=%d VD=%d", D, VD);
+  return NSA_ERR_UNSUPPORTED;
+}

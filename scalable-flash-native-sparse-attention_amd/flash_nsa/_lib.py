@@ -23,7 +23,7 @@ def parse_header(path=HEADER_PATH):
     text = open(path).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     protos = {}
-    for m in re.finditer(r"(const char\*|int)\s+(nsa_\w+)\s*\(([^)]*)\)\s*;", text):
+    for m in re.finditer(r"(const char\*|int64_t|int)\s+(nsa_\w+)\s*\(([^)]*)\)\s*;", text):
         ret, name, args = m.group(1), m.group(2), m.group(3).strip()
         argtypes = []
         if args and args != "void":
@@ -34,7 +34,8 @@ def parse_header(path=HEADER_PATH):
                 else:
                     ty = a.replace("const", "").split()[0]
                     argtypes.append(_CTYPE[ty])
-        protos[name] = (ctypes.c_char_p if "char" in ret else ctypes.c_int, argtypes)
+        restype = ctypes.c_char_p if "char" in ret else (ctypes.c_int64 if ret == "int64_t" else ctypes.c_int)
+        protos[name] = (restype, argtypes)
     return protos
 
 
@@ -59,6 +60,10 @@ class _Lib:
         self._dll = dll
         return dll
 
+    def value(self, name, *args):
+        """call an entry point that returns a value rather than a status"""
+        return getattr(self.load(), name)(*args)
+
     def call(self, name, *args):
         dll = self.load()
         rc = getattr(dll, name)(*args)
@@ -72,6 +77,10 @@ LIB = _Lib()
 
 def call(name, *args):
     LIB.call(name, *args)
+
+
+def value(name, *args):
+    return LIB.value(name, *args)
 
 
 def stream_ptr():

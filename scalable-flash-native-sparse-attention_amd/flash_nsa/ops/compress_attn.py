@@ -3,7 +3,7 @@ import torch
 
 from .. import _lib
 from ..utils import NSAHelper
-from ._common import check_thd, default_scale
+from ._common import check_thd, default_scale, delta_of, dq_target
 
 
 def cmp_attn_fwd(q, k, v, sm_scale=None, helper=NSAHelper):
@@ -22,3 +22,55 @@ def cmp_attn_fwd(q, k, v, sm_scale=None, helper=NSAHelper):
               helper.batch, helper.x_maxlen, QH, KH, D, VD, helper.kernel_size, helper.stride, sm_scale,
               _lib.stream_ptr())
     return o, lse
+
+
+def cmp_attn_bwd(q, k, v, o, lse, do, dq=None, dkdv_repeat=False, sm_scale=None, helper=NSAHelper, delta=None,
+                 q_chunk_tokens=2048):
+    """Backward of compressed attention.  Returns (dq, dk, dv).
+    dq: fresh bf16 tensor, or the caller's fp32 buffer, which is added into.
+    dk, dv: fp32 [y_len,KH,*] accumulated with atomics over the q-heads of a group and over query chunks
+    (non-deterministic summation order, as upstream's dkdv_repeat=False path); `dkdv_repeat` is accepted for call
+    compatibility and ignored.  delta may be passed when already known (delta[T,QH] fp32 = rowsum(o*do))."""
+    check_thd(do, "do")
+    T, QH, D = q.shape
+    Y, KH, VD = v.shape
+    sm_scale = default_scale(q, sm_scale)
+    if delta is None:
+        delta = delta_of(o, do)
+    dq_buf, mode = dq_target(q, dq)
+    common = (q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), k.stride(0), k.stride(1), v.data_ptr(),
+              v.stride(0), v.stride(1), do.data_ptr(), do.stride(0), do.stride(1), lse.data_ptr(), lse.stride(1),
+              lse.stride(0), delta.data_ptr(), delta.stride(0), delta.stride(1))
+    _lib.call("nsa_cmp_attn_bwd_dq", *common, dq_buf.data_ptr(), dq_buf.stride(0), dq_buf.stride(1), mode,
+              helper.x_cu_seqlens.data_ptr(), helper.y_cu_seqlens.data_ptr(), helper.batch, helper.x_maxlen, QH, KH,
+              D, VD, helper.kernel_size, helper.stride, sm_scale, _lib.stream_ptr())
+    dk = torch.zeros(Y, KH, D, device=q.device, dtype=torch.float32)
+    dv = torch.zeros(Y, KH, VD, device=q.device, dtype=torch.float32)
+    _lib.call("nsa_cmp_attn_bwd_dkdv", *common, dk.data_ptr(), dk.stride(0), dk.stride(1), dv.data_ptr(),
+              dv.stride(0), dv.stride(1), helper.x_cu_seqlens.data_ptr(), helper.y_cu_seqlens.data_ptr(),
+              helper.batch, helper.x_maxlen, helper.y_maxlen, QH, KH, D, VD, helper.kernel_size, helper.stride,
+              q_chunk_tokens, sm_scale, _lib.stream_ptr())
+    return dq_buf, dk, dv
+
+
+class _CompressAttn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, sm_scale):
+        o, lse = cmp_attn_fwd(q, k, v, sm_scale)
+        ctx.save_for_backward(q, k, v, o, lse)
+        ctx.sm_scale = sm_scale
+        ctx.helper = NSAHelper.get_bwd_helper()
+        ctx.mark_non_differentiable(lse)
+        return o, lse
+
+    @staticmethod
+    def backward(ctx, do, _dlse):
+        q, k, v, o, lse = ctx.saved_tensors
+        do = do if do.stride(-1) == 1 else do.contiguous()
+        dq, dk, dv = cmp_attn_bwd(q, k, v, o, lse, do, sm_scale=ctx.sm_scale, helper=ctx.helper)
+        return dq, dk.to(k.dtype), dv.to(v.dtype), None
+
+
+def compress_attn(q, k, v, sm_scale=None):
+    """Differentiable compressed attention -> (o, lse)."""
+    return _CompressAttn.apply(q, k, v, sm_scale)

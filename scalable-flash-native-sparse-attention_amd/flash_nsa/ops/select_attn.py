@@ -3,7 +3,7 @@ import torch
 
 from .. import _lib
 from ..utils import NSAHelper
-from ._common import check_thd, default_scale
+from ._common import check_thd, default_scale, delta_of, dq_target
 
 
 def slc_attn_fwd(q, k, v, topk, sm_scale=None, helper=NSAHelper):
@@ -22,3 +22,60 @@ def slc_attn_fwd(q, k, v, topk, sm_scale=None, helper=NSAHelper):
               helper.x_cu_seqlens.data_ptr(), helper.batch, helper.x_maxlen, QH, KH, D, VD, helper.block_size,
               topk.size(-1), sm_scale, _lib.stream_ptr())
     return o, lse
+
+
+def slc_attn_bwd(q, k, v, topk, o, lse, do, dq=None, dk=None, dv=None, sm_scale=None, helper=NSAHelper, delta=None,
+                 bind=None):
+    """Backward of selected attention.  Returns (dq, dk, dv).
+    dq: fresh bf16 tensor, or the caller's fp32 buffer (added into).  dk/dv: fp32 [T,KH,*]; the caller's buffers
+    are added into with atomics (summation order is not deterministic, as upstream), otherwise zero-filled ones are
+    created.  `bind` is the inverse index from get_bind_from_find (built here when absent)."""
+    from .topk import get_bind_from_find
+    check_thd(do, "do")
+    T, QH, D = q.shape
+    _, KH, VD = v.shape
+    sm_scale = default_scale(q, sm_scale)
+    if delta is None:
+        delta = delta_of(o, do)
+    dq_buf, mode = dq_target(q, dq)
+    common = (q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), k.stride(0), k.stride(1), v.data_ptr(),
+              v.stride(0), v.stride(1), do.data_ptr(), do.stride(0), do.stride(1), lse.data_ptr(), lse.stride(0),
+              lse.stride(1), delta.data_ptr(), delta.stride(0), delta.stride(1))
+    _lib.call("nsa_slc_attn_bwd_dq", *common, topk.data_ptr(), topk.stride(0), topk.stride(1), dq_buf.data_ptr(),
+              dq_buf.stride(0), dq_buf.stride(1), mode, helper.x_cu_seqlens.data_ptr(), helper.batch,
+              helper.x_maxlen, QH, KH, D, VD, helper.block_size, topk.size(-1), sm_scale, _lib.stream_ptr())
+    if dk is None:
+        dk = torch.zeros(T, KH, D, device=q.device, dtype=torch.float32)
+    if dv is None:
+        dv = torch.zeros(T, KH, VD, device=q.device, dtype=torch.float32)
+    assert dk.dtype == torch.float32 and dv.dtype == torch.float32
+    if bind is None:
+        bind = get_bind_from_find(topk, helper)
+    _lib.call("nsa_slc_attn_bwd_dkdv", *common, dk.data_ptr(), dk.stride(0), dk.stride(1), dv.data_ptr(),
+              dv.stride(0), dv.stride(1), helper.x_cu_seqlens.data_ptr(), helper.k_cu_seqlens.data_ptr(),
+              helper.blk_seq.data_ptr(), bind["csr_off"].data_ptr(), bind["csr_tok"].data_ptr(),
+              bind["item_off"].data_ptr(), bind["nblk"], bind["chunk_tokens"], bind["n_items_bound"], helper.batch,
+              QH, KH, D, VD, helper.block_size, sm_scale, _lib.stream_ptr())
+    return dq_buf, dk, dv
+
+
+class _SelectAttn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, topk, sm_scale):
+        o, lse = slc_attn_fwd(q, k, v, topk, sm_scale)
+        ctx.save_for_backward(q, k, v, topk, o, lse)
+        ctx.sm_scale = sm_scale
+        ctx.helper = NSAHelper.get_bwd_helper()
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, topk, o, lse = ctx.saved_tensors
+        do = do if do.stride(-1) == 1 else do.contiguous()
+        dq, dk, dv = slc_attn_bwd(q, k, v, topk, o, lse, do, sm_scale=ctx.sm_scale, helper=ctx.helper)
+        return dq, dk.to(k.dtype), dv.to(v.dtype), None, None
+
+
+def select_attn(q, k, v, topk, sm_scale=None):
+    """Differentiable selected-block attention (no gradient flows into topk)."""
+    return _SelectAttn.apply(q, k, v, topk, sm_scale)

@@ -42,3 +42,25 @@ def slc_topk_indices(q, k, lse, sm_scale=None, return_slc_prob=False, align=True
               helper.stride, helper.block_size, helper.top_n, helper.num_init_blocks, helper.num_local_blocks,
               ignore_index, sm_scale, _lib.stream_ptr())
     return topk, probs
+
+
+@torch.no_grad()
+def get_bind_from_find(topk, helper=NSAHelper, chunk_tokens=256):
+    """Inverse of the selection: for every (kv head, selection block) the ascending list of query tokens that
+    selected it.  Returns a dict with the CSR (csr_off [KH,nblk+1], csr_tok [KH*T*top_n]), the work-item prefix
+    (item_off [KH,nblk+1]) and the static bound on the number of work items per kv head."""
+    KH, T, N = topk.shape
+    dev = topk.device
+    nblk = helper.k_len
+    csr_off = torch.empty(KH, nblk + 1, device=dev, dtype=torch.int32)
+    item_off = torch.empty(KH, nblk + 1, device=dev, dtype=torch.int32)
+    csr_tok = torch.empty(KH * T * N, device=dev, dtype=torch.int32)
+    ws_elems = _lib.value("nsa_inverse_index_workspace_elems", T, KH, nblk)
+    ws = torch.empty(ws_elems, device=dev, dtype=torch.int32)
+    _lib.call("nsa_build_inverse_index", topk.data_ptr(), topk.stride(0), topk.stride(1), N,
+              helper.x_cu_seqlens.data_ptr(), helper.k_cu_seqlens.data_ptr(), helper.batch, T, KH, nblk,
+              helper.block_size, chunk_tokens, csr_off.data_ptr(), csr_tok.data_ptr(), item_off.data_ptr(),
+              ws.data_ptr(), ws_elems, _lib.stream_ptr())
+    n_items_bound = (T * N + chunk_tokens - 1) // chunk_tokens + nblk
+    return dict(csr_off=csr_off, csr_tok=csr_tok, item_off=item_off, n_items_bound=n_items_bound,
+                chunk_tokens=chunk_tokens, nblk=nblk)

@@ -54,6 +54,7 @@ class NSAHelper:
     k_seqlens = None
     k_maxlen = 0
     k_len = 0
+    blk_seq = None  # [k_len] sequence id of every selection block (used by the inverse index)
     batch = 0
     _key = None
     _host_cu = None
@@ -145,6 +146,8 @@ class NSAHelper:
         cls.k_cu_seqlens = torch.tensor(cum(ks), dtype=torch.int32, device=dev)
         cls.k_maxlen = max(ks)
         cls.k_len = sum(ks)
+        cls.blk_seq = torch.repeat_interleave(torch.arange(len(ks), dtype=torch.int32), torch.tensor(ks)).to(
+            device=dev, dtype=torch.int32)
         cls._host_cu = host
         cls._key = (x_cu_seqlens.data_ptr(), x_cu_seqlens._version, x_cu_seqlens.numel(), x_cu_seqlens.device)
 
@@ -164,7 +167,7 @@ class BwdNSAHelper:
     between a forward and its backward (upstream flash_nsa/utils.py:465-482)."""
     _FIELDS = ("kernel_size", "stride", "block_size", "window_size", "top_n", "num_init_blocks", "num_local_blocks",
                "x_cu_seqlens", "x_seqlens", "x_maxlen", "y_cu_seqlens", "y_seqlens", "y_maxlen", "y_len",
-               "k_cu_seqlens", "k_seqlens", "k_maxlen", "k_len", "batch", "cmp_k_method", "cmp_v_method")
+               "k_cu_seqlens", "k_seqlens", "k_maxlen", "k_len", "blk_seq", "batch", "cmp_k_method", "cmp_v_method")
 
     def __init__(self):
         for f in self._FIELDS:

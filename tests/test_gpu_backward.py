@@ -1,0 +1,206 @@
+"""GPU parity of the backward operators and of the composed modules against torch.autograd through the CPU
+oracle (same seeded bf16 inputs, fp32 oracle arithmetic).  Mirrors upstream test.py --func cmp/slc/combine/nsa
+(test.py:131-353) with asserted tolerances."""
+import pytest
+import torch
+
+from oracle import nsa_oracle as O
+from gpu_util import make_cu, make_qkvw, randn_bf16, assert_close
+
+pytestmark = pytest.mark.gpu
+
+LENS_CASES = [[1000], [5, 31, 32, 47, 48, 100, 333, 700], [64, 0, 129, 513]]
+HEAD_CASES = [(16, 1, 128), (8, 2, 128), (4, 4, 64)]
+
+
+def setup_helper(cu_dev, **kw):
+    from flash_nsa import NSAHelper
+    NSAHelper.set_hyperparameters(**kw)
+    NSAHelper.init_cu_seqlens(cu_dev)
+    return NSAHelper
+
+
+def leaf(x):
+    return x.float().clone().requires_grad_()
+
+
+@pytest.mark.parametrize("lens", LENS_CASES)
+def test_mean_pooling_bwd(device, lens):
+    from flash_nsa.ops.compress_kv import mean_pooling_bwd, construct_block_bwd
+    cu = make_cu(lens)
+    T = int(cu[-1])
+    x = randn_bf16(T, 2, 128, seed=1)
+    setup_helper(cu.to(device))
+    xr = leaf(x)
+    y = O.mean_pooling(xr, cu)
+    dy = randn_bf16(*y.shape, seed=2)
+    y.backward(dy.float())
+    dx = mean_pooling_bwd(x.to(device), dy.to(device))
+    assert_close(dx, xr.grad, "pool dx", atol=2e-3, rtol=1e-2)
+    acc = torch.ones(T, 2, 128, device=device, dtype=torch.float32)
+    mean_pooling_bwd(x.to(device), dy.to(device), acc)
+    assert_close(acc, xr.grad + 1, "pool dx accumulate", atol=1e-5, rtol=1e-5)
+    xb = leaf(x)
+    blk = O.construct_block(xb, cu)
+    dblk = randn_bf16(*blk.shape, seed=3)
+    blk.backward(dblk.float())
+    dxb = construct_block_bwd(x.to(device), dblk.to(device))
+    assert_close(dxb, xb.grad, "construct_block dx", atol=1e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("lens", LENS_CASES)
+@pytest.mark.parametrize("QH,KH,D", HEAD_CASES)
+def test_cmp_attn_bwd(device, lens, QH, KH, D):
+    from flash_nsa.ops.compress_kv import mean_pooling_fwd
+    from flash_nsa.ops.compress_attn import cmp_attn_fwd, cmp_attn_bwd
+    cu = make_cu(lens)
+    T = int(cu[-1])
+    q, k, v, _ = make_qkvw(T, QH, KH, D, seed=40)
+    do = randn_bf16(T, QH, D, seed=44)
+    setup_helper(cu.to(device))
+    qd = q.to(device)
+    ck, cv = mean_pooling_fwd(k.to(device)), mean_pooling_fwd(v.to(device))
+    o, lse = cmp_attn_fwd(qd, ck, cv)
+    dq, dck, dcv = cmp_attn_bwd(qd, ck, cv, o, lse, do.to(device), q_chunk_tokens=256)
+    qr, ckr, cvr = leaf(q), leaf(ck.cpu()), leaf(cv.cpu())
+    ro, _ = O.cmp_attn(qr, ckr, cvr, cu)
+    ro.backward(do.float())
+    assert_close(dq, qr.grad, "cmp dq")
+    if ck.numel():
+        assert_close(dck, ckr.grad, "cmp dk", row_scale=True)
+        assert_close(dcv, cvr.grad, "cmp dv", row_scale=True)
+
+
+@pytest.mark.parametrize("lens", LENS_CASES)
+@pytest.mark.parametrize("QH,KH,D", HEAD_CASES)
+def test_swa_bwd(device, lens, QH, KH, D):
+    from flash_nsa.ops.sliding_window_attention import swa_fwd, swa_bwd
+    cu = make_cu(lens)
+    T = int(cu[-1])
+    q, k, v, _ = make_qkvw(T, QH, KH, D, seed=50)
+    do = randn_bf16(T, QH, D, seed=54)
+    setup_helper(cu.to(device), window_size=200)
+    qd, kd, vd = q.to(device), k.to(device), v.to(device)
+    o, lse = swa_fwd(qd, kd, vd)
+    dq, dk, dv = swa_bwd(qd, kd, vd, o, lse, do.to(device), dkv_fp32=True)
+    qr, kr, vr = leaf(q), leaf(k), leaf(v)
+    ro, _ = O.swa(qr, kr, vr, cu, 200)
+    ro.backward(do.float())
+    assert_close(dq, qr.grad, "swa dq")
+    assert_close(dk, kr.grad, "swa dk", row_scale=True)
+    assert_close(dv, vr.grad, "swa dv", row_scale=True)
+    setup_helper(cu.to(device))
+
+
+@pytest.mark.parametrize("lens", LENS_CASES)
+@pytest.mark.parametrize("QH,KH,D", HEAD_CASES)
+def test_slc_attn_bwd(device, lens, QH, KH, D):
+    from flash_nsa.ops.compress_kv import mean_pooling_fwd
+    from flash_nsa.ops.compress_attn import cmp_attn_fwd
+    from flash_nsa.ops.topk import slc_topk_indices, get_bind_from_find
+    from flash_nsa.ops.select_attn import slc_attn_fwd, slc_attn_bwd
+    from flash_nsa import NSAHelper
+    cu = make_cu(lens)
+    T = int(cu[-1])
+    q, k, v, _ = make_qkvw(T, QH, KH, D, seed=60)
+    do = randn_bf16(T, QH, D, seed=64)
+    top_n = 6
+    setup_helper(cu.to(device), top_n=top_n)
+    qd, kd, vd = q.to(device), k.to(device), v.to(device)
+    ck = mean_pooling_fwd(kd)
+    _, lse_c = cmp_attn_fwd(qd, ck, ck)
+    topk, _ = slc_topk_indices(qd, ck, lse_c)
+    # inverse index: every (token, valid slot) appears exactly once, lists ascending
+    bind = get_bind_from_find(topk, chunk_tokens=64)
+    off = bind["csr_off"].cpu()
+    tok = bind["csr_tok"].cpu()
+    tk = topk.cpu()
+    kcu = NSAHelper.k_cu_seqlens.cpu()
+    for kh in range(KH):
+        exp = {}
+        for b in range(len(lens)):
+            for n in range(lens[b]):
+                for s in range(min(top_n, n // 64 + 1)):
+                    exp.setdefault(int(kcu[b]) + int(tk[kh, int(cu[b]) + n, s]), []).append(n)
+        for jb in range(int(kcu[-1])):
+            got = tok[int(off[kh, jb]):int(off[kh, jb + 1])].tolist()
+            assert got == sorted(exp.get(jb, [])), (kh, jb)
+    o, lse = slc_attn_fwd(qd, kd, vd, topk)
+    dq, dk, dv = slc_attn_bwd(qd, kd, vd, topk, o, lse, do.to(device), bind=bind)
+    qr, kr, vr = leaf(q), leaf(k), leaf(v)
+    ro, _ = O.slc_attn(qr, kr, vr, tk, cu, 64)
+    ro.backward(do.float())
+    assert_close(dq, qr.grad, "slc dq")
+    assert_close(dk, kr.grad, "slc dk", row_scale=True)
+    assert_close(dv, vr.grad, "slc dv", row_scale=True)
+    setup_helper(cu.to(device))
+
+
+def test_combine_bwd(device):
+    from flash_nsa.ops.combine import combine_bwd
+    a, b, c = [randn_bf16(300, 8, 128, seed=s) for s in (1, 2, 3)]
+    w = randn_bf16(300, 8, 3, seed=4)
+    do = randn_bf16(300, 8, 128, seed=5)
+    ar, br, cr, wr = leaf(a), leaf(b), leaf(c), leaf(w)
+    O.combine(ar, br, cr, wr).backward(do.float())
+    da, db, dc, dw, delta = combine_bwd(a.to(device), b.to(device), c.to(device), w.to(device), do.to(device),
+                                        return_delta=True)
+    assert_close(da, ar.grad, "da")
+    assert_close(db, br.grad, "db")
+    assert_close(dc, cr.grad, "dc")
+    assert_close(dw, wr.grad, "dw", atol=5e-2, rtol=1e-2)
+    for i, (x, g) in enumerate(((a, ar), (b, br), (c, cr))):
+        assert_close(delta[i], (x.float() * g.grad).sum(-1), f"delta{i}", atol=2e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("core", ["hf", "megatron"])
+@pytest.mark.parametrize("lens,QH,KH,D,methods", [
+    ([1500], 16, 1, 128, ("mean", "mean")),
+    ([5, 31, 48, 333, 700, 900], 8, 2, 128, ("mean", "sigmoid-mul")),
+    ([300, 800], 4, 2, 64, ("linear", "swiglu")),
+])
+def test_nsa_core_fwd_bwd(device, core, lens, QH, KH, D, methods):
+    """HFNSACore and NSACore against the composed oracle (upstream only compares them with each other)."""
+    from flash_nsa import NSAConfig, HFNSACore, NSACore
+    from flash_nsa.ops.compress_attn import cmp_attn_fwd
+    from flash_nsa.ops.topk import slc_topk_indices
+    cu = make_cu(lens)
+    T = int(cu[-1])
+    q, k, v, w = make_qkvw(T, QH, KH, D, seed=70)
+    do = randn_bf16(T, QH, D, seed=75)
+    cfg = NSAConfig(head_dim=D, num_heads=QH, num_kv_heads=KH, top_n=8, window_size=128, cmp_k_method=methods[0],
+                    cmp_v_method=methods[1])
+    torch.manual_seed(0)
+    mod = (HFNSACore(cfg) if core == "hf" else NSACore(cfg)).to(device=device, dtype=torch.bfloat16)
+    if core == "hf":
+        wk = mod.compress_k.fc.weight if methods[0] != "mean" else None
+        wv = mod.compress_v.fc.weight if methods[1] != "mean" else None
+    else:
+        wk, wv = mod.cmp_k_weight, mod.cmp_v_weight
+    qd, kd, vd, wd = [t.to(device).requires_grad_() for t in (q, k, v, w)]
+    out = mod(qd, kd, vd, wd, cu.to(device))
+    out.backward(do.to(device))
+
+    ocfg = O.OracleConfig(top_n=8, window_size=128, cmp_k_method=methods[0], cmp_v_method=methods[1])
+    qr, kr, vr, wr = leaf(q), leaf(k), leaf(v), leaf(w)
+    wkr = leaf(wk.detach().cpu()) if wk is not None else None
+    wvr = leaf(wv.detach().cpu()) if wv is not None else None
+    # indices: take the device's selection (checked against the oracle's in the forward tests) so that a
+    # near-tie cannot change which keys the two sides attend
+    with torch.no_grad():
+        from flash_nsa.modules.megatron_level_nsa import compress_kv_fwd
+        ck = compress_kv_fwd(kd.detach(), wk, methods[0])[2]
+        cv = compress_kv_fwd(vd.detach(), wv, methods[1])[2]
+        _, lse = cmp_attn_fwd(qd.detach(), ck, cv)
+        topk, _ = slc_topk_indices(qd.detach(), ck, lse)
+    ro = O.nsa_forward(qr, kr, vr, wr, cu, ocfg, wk=wkr, wv=wvr, topk=topk.cpu())
+    ro.backward(do.float())
+    assert_close(out, ro, "o")
+    assert_close(qd.grad, qr.grad, "dq")
+    assert_close(kd.grad, kr.grad, "dk", row_scale=True)
+    assert_close(vd.grad, vr.grad, "dv", row_scale=True)
+    assert_close(wd.grad, wr.grad, "dw", atol=5e-2)
+    if wk is not None:
+        assert_close(wk.grad, wkr.grad, "dWk", atol=5e-2, rtol=2e-2, row_scale=True)
+    if wv is not None:
+        assert_close(wv.grad, wvr.grad, "dWv", atol=5e-2, rtol=2e-2, row_scale=True)
