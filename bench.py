@@ -1,0 +1,276 @@
+"""Benchmark of the NSA hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--seq-len T] [--no-cpu] [--no-decode]
+
+A step is one forward+backward of the NSA core (NSACore: mean K-compression, sigmoid-mul V-compression,
+kernel 32 / stride 16 / block 64 / top-16 / window 512) on one causal sequence of T=65536 tokens,
+64 q-heads / 4 kv-heads / head dim 128, bf16, synthetic N(0,1) inputs resident in HBM.
+Prints ONE JSON line: whole-step throughput in algorithmic TFLOP/s, per-stage milliseconds measured with HIP
+events on the launch stream, the roofline of the dominant kernel, and the CPU oracle timed on the host.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "scalable-flash-native-sparse-attention_amd"))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0
+
+
+def branch_counts(lens, kernel=32, stride=16, block=64, top_n=16, window=512):
+    """(N_c, N_s, N_w): visible (query, key) pairs per q-head of the three branches, summed over sequences."""
+    import numpy as np
+    nc = ns = nw = 0
+    for L in lens:
+        t = np.arange(L, dtype=np.int64)
+        y = max((L - kernel) // stride + 1, 0)
+        nc += int(np.clip((t - (kernel - 1)) // stride + 1, 0, y).sum())
+        ns += int((block * np.minimum(top_n, t // block + 1)).sum())
+        nw += int(np.minimum(t + 1, window + 1).sum())
+    return nc, ns, nw
+
+
+def stage_flops(lens, QH, D, VD, **kw):
+    nc, ns, nw = branch_counts(lens, **kw)
+    f = dict(cmp_fwd=QH * 2 * (D + VD) * nc, topk=QH * 2 * D * nc, slc_fwd=QH * 2 * (D + VD) * ns,
+             swa_fwd=QH * 2 * (D + VD) * nw)
+    # backward: S, dP, dV, dK (2.0x forward) are attributed to the dk/dv kernel, dQ (0.5x) to the dq kernel;
+    # the dq kernel's own recomputation of S and dP is overhead and not counted
+    for br in ("cmp", "slc", "swa"):
+        f[br + "_dkdv"] = 2.0 * f[br + "_fwd"]
+        f[br + "_dq"] = 0.5 * f[br + "_fwd"]
+    f["fwd_total"] = f["cmp_fwd"] + f["topk"] + f["slc_fwd"] + f["swa_fwd"]
+    f["bwd_total"] = 2.5 * (f["cmp_fwd"] + f["slc_fwd"] + f["swa_fwd"])
+    return f
+
+
+class StageTimer:
+    """HIP-event timing of named stages on the current stream."""
+
+    def __init__(self):
+        self.events = []
+
+    def run(self, name, fn):
+        import torch
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        out = fn()
+        e.record()
+        self.events.append((name, s, e))
+        return out
+
+    def summary(self):
+        import torch
+        torch.cuda.synchronize()
+        acc = {}
+        for name, s, e in self.events:
+            acc.setdefault(name, []).append(s.elapsed_time(e))
+        return {k: sum(v) / len(v) for k, v in acc.items()}
+
+
+def staged_step(timer, q, k, v, w, wv, do, sm_scale):
+    """The same launches as NSAFunction.forward/backward, stage by stage under event timers."""
+    import torch
+    from flash_nsa.ops.compress_kv import mean_pooling_fwd, construct_block_fwd, construct_block_bwd, mean_pooling_bwd
+    from flash_nsa.ops.act import sigmoid_mul_fwd, sigmoid_mul_bwd
+    from flash_nsa.ops.compress_attn import cmp_attn_fwd, cmp_attn_bwd
+    from flash_nsa.ops.topk import slc_topk_indices, get_bind_from_find
+    from flash_nsa.ops.select_attn import slc_attn_fwd, slc_attn_bwd
+    from flash_nsa.ops.sliding_window_attention import swa_fwd, swa_bwd
+    from flash_nsa.ops.combine import combine_fwd, combine_bwd
+    from flash_nsa import _lib
+    from flash_nsa.utils import NSAHelper as H
+    from flash_nsa.modules.megatron_level_nsa import _store_into
+
+    R = timer.run
+    cmp_k = R("pool_k", lambda: mean_pooling_fwd(k))
+    win_v = R("im2col_v", lambda: construct_block_fwd(v))
+    hid_v = R("gemm_cmp_v", lambda: torch.matmul(win_v.flatten(-2, -1), wv.t()))
+    cmp_v = R("sigmoid_mul", lambda: sigmoid_mul_fwd(hid_v))
+    cmp_o, cmp_lse = R("cmp_fwd", lambda: cmp_attn_fwd(q, cmp_k, cmp_v, sm_scale=sm_scale))
+    topk, _ = R("topk", lambda: slc_topk_indices(q, cmp_k, cmp_lse, sm_scale=sm_scale))
+    slc_o, slc_lse = R("slc_fwd", lambda: slc_attn_fwd(q, k, v, topk, sm_scale=sm_scale))
+    swa_o, swa_lse = R("swa_fwd", lambda: swa_fwd(q, k, v, sm_scale=sm_scale))
+    R("combine_fwd", lambda: combine_fwd(cmp_o, slc_o, swa_o, w))
+
+    dcmp_o, dslc_o, dswa_o, dw, delta = R("combine_bwd", lambda: combine_bwd(cmp_o, slc_o, swa_o, w, do, True))
+    dq = torch.empty(q.shape, device=q.device, dtype=torch.float32)
+    T, QH, D = q.shape
+    _, KH, VD = v.shape
+
+    def common(kk, vv, lse, lse_st, lse_sh, dlt, dout):
+        return (q.data_ptr(), q.stride(0), q.stride(1), kk.data_ptr(), kk.stride(0), kk.stride(1), vv.data_ptr(),
+                vv.stride(0), vv.stride(1), dout.data_ptr(), dout.stride(0), dout.stride(1), lse.data_ptr(), lse_st,
+                lse_sh, dlt.data_ptr(), dlt.stride(0), dlt.stride(1))
+
+    st = _lib.stream_ptr()
+    dk = torch.empty(T, KH, D, device=q.device, dtype=torch.float32)
+    dv = torch.empty(T, KH, VD, device=q.device, dtype=torch.float32)
+    cs = common(k, v, swa_lse, swa_lse.stride(0), swa_lse.stride(1), delta[2], dswa_o)
+    R("swa_dq", lambda: _lib.call("nsa_swa_bwd_dq", *cs, dq.data_ptr(), dq.stride(0), dq.stride(1), 1,
+                                  H.x_cu_seqlens.data_ptr(), H.batch, H.x_maxlen, QH, KH, D, VD, H.window_size,
+                                  sm_scale, st))
+    R("swa_dkdv", lambda: _lib.call("nsa_swa_bwd_dkdv", *cs, dk.data_ptr(), dk.stride(0), dk.stride(1),
+                                    dv.data_ptr(), dv.stride(0), dv.stride(1), 1, H.x_cu_seqlens.data_ptr(), H.batch,
+                                    H.x_maxlen, QH, KH, D, VD, H.window_size, sm_scale, st))
+    cl = common(k, v, slc_lse, slc_lse.stride(0), slc_lse.stride(1), delta[1], dslc_o)
+    R("slc_dq", lambda: _lib.call("nsa_slc_attn_bwd_dq", *cl, topk.data_ptr(), topk.stride(0), topk.stride(1),
+                                  dq.data_ptr(), dq.stride(0), dq.stride(1), 2, H.x_cu_seqlens.data_ptr(), H.batch,
+                                  H.x_maxlen, QH, KH, D, VD, H.block_size, topk.size(-1), sm_scale, st))
+    bind = R("inverse_index", lambda: get_bind_from_find(topk))
+    R("slc_dkdv", lambda: _lib.call("nsa_slc_attn_bwd_dkdv", *cl, dk.data_ptr(), dk.stride(0), dk.stride(1),
+                                    dv.data_ptr(), dv.stride(0), dv.stride(1), H.x_cu_seqlens.data_ptr(),
+                                    H.k_cu_seqlens.data_ptr(), H.blk_seq.data_ptr(), bind["csr_off"].data_ptr(),
+                                    bind["csr_tok"].data_ptr(), bind["item_off"].data_ptr(), bind["nblk"],
+                                    bind["chunk_tokens"], bind["n_items_bound"], H.batch, QH, KH, D, VD,
+                                    H.block_size, sm_scale, st))
+    cc = common(cmp_k, cmp_v, cmp_lse, cmp_lse.stride(1), cmp_lse.stride(0), delta[0], dcmp_o)
+    R("cmp_dq", lambda: _lib.call("nsa_cmp_attn_bwd_dq", *cc, dq.data_ptr(), dq.stride(0), dq.stride(1), 2,
+                                  H.x_cu_seqlens.data_ptr(), H.y_cu_seqlens.data_ptr(), H.batch, H.x_maxlen, QH, KH,
+                                  D, VD, H.kernel_size, H.stride, sm_scale, st))
+    dck = torch.zeros(cmp_k.shape, device=q.device, dtype=torch.float32)
+    dcv = torch.zeros(cmp_v.shape, device=q.device, dtype=torch.float32)
+    R("cmp_dkdv", lambda: _lib.call("nsa_cmp_attn_bwd_dkdv", *cc, dck.data_ptr(), dck.stride(0), dck.stride(1),
+                                    dcv.data_ptr(), dcv.stride(0), dcv.stride(1), H.x_cu_seqlens.data_ptr(),
+                                    H.y_cu_seqlens.data_ptr(), H.batch, H.x_maxlen, H.y_maxlen, QH, KH, D, VD,
+                                    H.kernel_size, H.stride, 2048, sm_scale, st))
+    R("pool_k_bwd", lambda: mean_pooling_bwd(k, dck.to(k.dtype), dk))
+
+    def cmp_v_bwd():
+        dhid = sigmoid_mul_bwd(hid_v, dcv.to(v.dtype), inplace=False)
+        dwin = torch.matmul(dhid, wv).view(*win_v.shape)
+        construct_block_bwd(v, dwin, dv)
+        return torch.matmul(dhid.flatten(0, 1).t(), win_v.flatten(-2, -1).flatten(0, 1))
+
+    R("cmp_v_bwd", cmp_v_bwd)
+    R("dq_cast", lambda: dq.to(q.dtype))
+
+
+def cpu_baseline():
+    """Oracle forward+backward of the reference's CPU-runnable case (T=4096, 16 q / 1 kv heads, fp32)."""
+    import torch
+    from oracle import nsa_oracle as O
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    T, QH, KH, D = 4096, 16, 1, 128
+    g = torch.Generator().manual_seed(0)
+    q, k, v, w = [torch.randn(*s, generator=g).requires_grad_() for s in
+                  ((T, QH, D), (T, KH, D), (T, KH, D), (T, QH, 3))]
+    t0 = time.perf_counter()
+    o = O.nsa_forward(q, k, v, w, [0, T])
+    t1 = time.perf_counter()
+    o.backward(torch.ones_like(o))
+    t2 = time.perf_counter()
+    fl = stage_flops([T], QH, D, D)
+    total = fl["fwd_total"] + fl["bwd_total"]
+    return {"value": total / (t2 - t0) / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"one forward+backward of the CPU oracle, T={T}, {QH}q/{KH}kv heads, d={D}, fp32, "
+                      f"torch {torch.__version__} with {torch.get_num_threads()} threads",
+            "fwd_s": t1 - t0, "bwd_s": t2 - t1}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--seq-len", type=int, default=65536)
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-decode", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (--gpus 1); multi-GPU sharding is a design note only",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from flash_nsa import NSAConfig, NSACore
+    from flash_nsa import _lib
+    _lib.LIB.load()  # fail loudly if the HIP library is missing
+    dev = torch.device("cuda:0")
+    T, QH, KH, D = args.seq_len, 64, 4, 128
+    g = torch.Generator(device=dev).manual_seed(0)
+    rnd = lambda *s: torch.randn(*s, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    q, k, v, w, do = rnd(T, QH, D), rnd(T, KH, D), rnd(T, KH, D), rnd(T, QH, 3), rnd(T, QH, D)
+    cu = torch.tensor([0, T], device=dev, dtype=torch.int32)
+    cfg = NSAConfig(head_dim=D, num_heads=QH, num_kv_heads=KH, cmp_k_method="mean", cmp_v_method="sigmoid-mul")
+    torch.manual_seed(0)
+    core = NSACore(cfg).to(device=dev, dtype=torch.bfloat16)
+    for t in (q, k, v, w):
+        t.requires_grad_()
+
+    def step():
+        for t in (q, k, v, w):
+            t.grad = None
+        core.cmp_v_weight.grad = None
+        out = core(q, k, v, w, cu)
+        out.backward(do)
+        return out
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # forward-only and per-stage times (HIP events on the launch stream)
+    with torch.no_grad():
+        core(q, k, v, w, cu)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            core(q, k, v, w, cu)
+        torch.cuda.synchronize()
+        fwd_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        timer = StageTimer()
+        qd, kd, vd, wd = q.detach(), k.detach(), v.detach(), w.detach()
+        staged_step(StageTimer(), qd, kd, vd, wd, core.cmp_v_weight.detach(), do, core.sm_scale)  # warm
+        for _ in range(max(args.steps, 3)):
+            staged_step(timer, qd, kd, vd, wd, core.cmp_v_weight.detach(), do, core.sm_scale)
+        stages = timer.summary()
+
+    fl = stage_flops([T], QH, D, D)
+    total_flops = fl["fwd_total"] + fl["bwd_total"]
+    mfma_stages = {s: stages[s] for s in stages if s in fl}
+    dom = max(mfma_stages, key=mfma_stages.get)
+    achieved = fl[dom] / (stages[dom] * 1e-3) / 1e12
+    result = {
+        "metric": "NSA fwd+bwd ms & TFLOP/s @T=64K bf16; paged decode us/step bs64 ctx<=32K",
+        "value": total_flops / (ms_per_step * 1e-3) / 1e12,
+        "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"NSA forward+backward, one causal sequence T={T}, 64q/4kv heads, d=128, mean K / "
+                               "sigmoid-mul V compression (kernel 32, stride 16), block 64, top-16, window 512",
+                   "seq_len": T, "q_heads": QH, "kv_heads": KH, "head_dim": D},
+        "fwd_ms": fwd_ms, "bwd_ms": ms_per_step - fwd_ms,
+        "fwd_tflops": fl["fwd_total"] / (fwd_ms * 1e-3) / 1e12,
+        "algorithmic_tflop": {"fwd": fl["fwd_total"] / 1e12, "bwd": fl["bwd_total"] / 1e12},
+        "stage_ms": {k_: round(v_, 4) for k_, v_ in stages.items()},
+        "stage_tflops": {s: round(fl[s] / (stages[s] * 1e-3) / 1e12, 1) for s in mfma_stages},
+        "roofline": {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None},
+    }
+    if not args.no_decode:
+        try:
+            from bench_decode import decode_bench
+            result["decode"] = decode_bench(dev)
+        except ImportError:
+            result["decode"] = None
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

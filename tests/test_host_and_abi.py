@@ -1,0 +1,78 @@
+"""CPU-side checks: the built library exports every symbol the C header declares (no compute calls), the host
+metadata logic, and the config validation."""
+import ctypes
+import os
+
+import pytest
+import torch
+
+
+def test_library_exports_every_declared_symbol():
+    from flash_nsa import _lib
+    protos = _lib.parse_header()
+    assert len(protos) >= 25
+    assert os.path.exists(_lib.LIB_PATH), "libnsa_hip.so is not built (run __graft_entry__.build())"
+    dll = ctypes.CDLL(_lib.LIB_PATH)
+    for name in protos:
+        assert hasattr(dll, name), f"{name} is declared in include/nsa_hip.h but not exported"
+    dll.nsa_abi_version.restype = ctypes.c_int
+    assert dll.nsa_abi_version() >= 1
+
+
+def test_entry_points_reject_bad_arguments_without_a_gpu():
+    from flash_nsa import _lib
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        _lib.call("nsa_mean_pool_fwd", None, 0, 0, None, 0, 0, None, None, 1, 1, 1, 12, 32, 16, None)
+    with pytest.raises(RuntimeError, match="power of 2"):
+        _lib.call("nsa_cmp_attn_fwd", None, 0, 0, None, 0, 0, None, 0, 0, None, 0, 0, None, 0, 0, None, None, 1, 8, 16,
+                  1, 128, 128, 32, 12, 1.0, None)
+    with pytest.raises(RuntimeError, match="kv heads"):
+        _lib.call("nsa_swa_fwd", None, 0, 0, None, 0, 0, None, 0, 0, None, 0, 0, None, 0, 0, None, 1, 8, 16, 3, 128,
+                  128, 512, 1.0, None)
+    with pytest.raises(RuntimeError, match="unsupported head dims"):
+        _lib.call("nsa_swa_fwd", None, 0, 0, None, 0, 0, None, 0, 0, None, 0, 0, None, 0, 0, None, 1, 8, 16, 1, 96,
+                  96, 512, 1.0, None)
+
+
+def test_nsa_helper_metadata():
+    from flash_nsa import NSAHelper
+    NSAHelper.set_hyperparameters()
+    cu = torch.tensor([0, 31, 63, 163, 163, 4259], dtype=torch.int32)
+    NSAHelper.init_cu_seqlens(cu)
+    assert NSAHelper.batch == 5
+    assert NSAHelper.x_maxlen == 4096
+    assert NSAHelper.y_seqlens.tolist() == [0, 1, 5, 0, 255]
+    assert NSAHelper.y_cu_seqlens.tolist() == [0, 0, 1, 6, 6, 261]
+    assert NSAHelper.k_seqlens.tolist() == [1, 1, 2, 0, 64]
+    assert NSAHelper.k_len == 68 and NSAHelper.y_len == 261 and NSAHelper.y_maxlen == 255
+    assert NSAHelper.blk_seq.tolist() == [0, 1, 2, 2] + [4] * 64
+    # changing the hyper-parameters invalidates the cached batch
+    NSAHelper.set_hyperparameters(kernel_size=64, stride=32, block_size=128)
+    NSAHelper.init_cu_seqlens(cu)
+    assert NSAHelper.y_seqlens.tolist() == [0, 0, 2, 0, 127]
+    NSAHelper.set_hyperparameters()
+
+
+def test_config_validation(tmp_path):
+    from flash_nsa import NSAConfig
+    c = NSAConfig(head_dim=64)
+    assert c.qk_head_dim == 64 and c.v_head_dim == 64
+    with pytest.raises(AssertionError):
+        NSAConfig(stride=12)
+    with pytest.raises(AssertionError):
+        NSAConfig(kernel_size=40)
+    with pytest.raises(AssertionError):
+        NSAConfig(block_size=16)
+    p = tmp_path / "c.json"
+    p.write_text('{"num_heads": 32, "top_n": 8, "slc_block_size": 64}')
+    c = NSAConfig.from_json(str(p))
+    assert c.num_heads == 32 and c.top_n == 8 and c.slc_block_size == 64
+
+
+def test_bench_flop_model_matches_closed_form():
+    import bench
+    nc, ns, nw = bench.branch_counts([65536])
+    assert (nc, ns, nw) == (134123535, 66617344, 33488640)
+    f = bench.stage_flops([65536], 64, 128, 128)
+    assert abs(f["fwd_total"] / 1e12 - 9.87) < 0.01
+    assert abs(f["bwd_total"] / 1e12 - 19.19) < 0.01
