@@ -140,6 +140,41 @@ int nsa_slc_attn_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void*
                           const int32_t* item_off, int nblk_total, int chunk_tokens, int n_items_bound, int B,
                           int QH, int KH, int D, int VD, int block_size, float sm_scale, void* stream);
 
+/* ---- paged KV (inference).  Caches are [num_pages, page_size, KH, D]; *_sr is the stride of a flat row
+ * (page*page_size + offset), *_sh the head stride.  Request b's raw token n lives at flat row
+ * block_tables[b][n/page]*page + n%page; its compressed row i at cmp_block_tables[b][i/page]*page + i%page of the
+ * SAME pool.  x_cu counts only the new query tokens; query n of request b sits at absolute position
+ * n + context_lens[b] - x_len[b].  page_size must be a multiple of 64. */
+
+/* flash_nsa/inference/compress_attn.py:486-538 cmp_attn_prefill (and, with one query per request, :540-667 decode) */
+int nsa_paged_cmp_attn_fwd(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr,
+                           int64_t k_sh, const void* v_cache, int64_t v_sr, int64_t v_sh, void* o, int64_t o_st,
+                           int64_t o_sh, float* lse, int64_t lse_st, int64_t lse_sh, const int32_t* x_cu,
+                           const int32_t* context_lens, const int32_t* cmp_block_tables, int table_stride,
+                           int page_size, int B, int x_maxlen, int QH, int KH, int D, int VD, int kernel_size,
+                           int stride, float sm_scale, void* stream);
+/* flash_nsa/inference/__init__.py:125-155 (FlashAttention with page table and window) */
+int nsa_paged_swa_fwd(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr, int64_t k_sh,
+                      const void* v_cache, int64_t v_sr, int64_t v_sh, void* o, int64_t o_st, int64_t o_sh,
+                      float* lse, int64_t lse_st, int64_t lse_sh, const int32_t* x_cu, const int32_t* context_lens,
+                      const int32_t* block_tables, int table_stride, int page_size, int B, int x_maxlen, int QH,
+                      int KH, int D, int VD, int window, float sm_scale, void* stream);
+/* flash_nsa/inference/topk.py:184-298 topk_prefill / :495-623 topk_decode (causality is masked per row here) */
+int nsa_paged_topk_select(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr,
+                          int64_t k_sh, const float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk,
+                          int64_t tk_sh, int64_t tk_st, const int32_t* x_cu, const int32_t* context_lens,
+                          const int32_t* cmp_block_tables, int table_stride, int page_size, int B, int x_maxlen,
+                          int fixed_num_slc_blocks, int QH, int KH, int D, int kernel_size, int stride,
+                          int block_size, int top_n, int num_init, int num_local, int ignore_index, float sm_scale,
+                          void* stream);
+/* flash_nsa/inference/select_attn.py:103-166 slc_attn_prefill */
+int nsa_paged_slc_attn_fwd(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr,
+                           int64_t k_sh, const void* v_cache, int64_t v_sr, int64_t v_sh, const int32_t* topk,
+                           int64_t tk_sh, int64_t tk_st, void* o, int64_t o_st, int64_t o_sh, float* lse,
+                           int64_t lse_st, int64_t lse_sh, const int32_t* x_cu, const int32_t* context_lens,
+                           const int32_t* block_tables, int table_stride, int page_size, int B, int x_maxlen,
+                           int QH, int KH, int D, int VD, int block_size, int top_n, float sm_scale, void* stream);
+
 /* flash_nsa/inference/compress_kv.py:191-220 mean_pooling_prefill (in-pool write at flat row slot) */
 int nsa_paged_pool_prefill(void* cache, int64_t c_sr, int64_t c_sh, const int32_t* y_cu, const int32_t* block_tables,
                            int table_stride, const int32_t* cmp_slot_mapping, int B, int y_maxlen, int page_size,

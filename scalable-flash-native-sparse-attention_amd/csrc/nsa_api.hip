@@ -302,3 +302,124 @@ int nsa_slc_attn_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void*
 }
 
 }  // extern "C"
+
+// ------------------------------------------------------------------------------------------------ paged KV
+namespace {
+int check_page(const char* who, int page_size) {
+  NSA_REQUIRE(page_size > 0 && page_size % 64 == 0, NSA_ERR_BAD_ARG, "%s: page_size %d must be a multiple of 64", who,
+              page_size);
+  return NSA_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int nsa_paged_cmp_attn_fwd(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr,
+                           int64_t k_sh, const void* v_cache, int64_t v_sr, int64_t v_sh, void* o, int64_t o_st,
+                           int64_t o_sh, float* lse, int64_t lse_st, int64_t lse_sh, const int32_t* x_cu,
+                           const int32_t* context_lens, const int32_t* cmp_block_tables, int table_stride,
+                           int page_size, int B, int x_maxlen, int QH, int KH, int D, int VD, int kernel_size,
+                           int stride, float sm_scale, void* stream) {
+  int rc = check_heads("paged_cmp_attn_fwd", QH, KH, D, VD);
+  if (rc) return rc;
+  rc = check_nsa_sizes("paged_cmp_attn_fwd", kernel_size, stride, 0);
+  if (rc) return rc;
+  rc = check_page("paged_cmp_attn_fwd", page_size);
+  if (rc) return rc;
+  NsaFwdTileParams p{};
+  p.q = (const bf16_t*)q; p.q_st = q_st; p.q_sh = q_sh;
+  p.k = (const bf16_t*)k_cache; p.k_sr = k_sr; p.k_sh = k_sh;
+  p.v = (const bf16_t*)v_cache; p.v_sr = v_sr; p.v_sh = v_sh;
+  p.o = (bf16_t*)o; p.o_st = o_st; p.o_sh = o_sh;
+  p.lse = lse; p.lse_st = lse_st; p.lse_sh = lse_sh;
+  p.x_cu = x_cu; p.ctx_lens = context_lens;
+  p.table = cmp_block_tables; p.table_stride = table_stride; p.page_size = page_size;
+  p.G = QH / KH; p.KH = KH;
+  p.scale_log2 = sm_scale * NSA_LOG2E;
+  p.kernel_size = kernel_size; p.stride = stride; p.window = 0;
+  return nsa_fwd_tile_launch(p, 0, true, B, x_maxlen, D, VD, (hipStream_t)stream);
+}
+
+int nsa_paged_swa_fwd(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr, int64_t k_sh,
+                      const void* v_cache, int64_t v_sr, int64_t v_sh, void* o, int64_t o_st, int64_t o_sh,
+                      float* lse, int64_t lse_st, int64_t lse_sh, const int32_t* x_cu, const int32_t* context_lens,
+                      const int32_t* block_tables, int table_stride, int page_size, int B, int x_maxlen, int QH,
+                      int KH, int D, int VD, int window, float sm_scale, void* stream) {
+  int rc = check_heads("paged_swa_fwd", QH, KH, D, VD);
+  if (rc) return rc;
+  rc = check_page("paged_swa_fwd", page_size);
+  if (rc) return rc;
+  NsaFwdTileParams p{};
+  p.q = (const bf16_t*)q; p.q_st = q_st; p.q_sh = q_sh;
+  p.k = (const bf16_t*)k_cache; p.k_sr = k_sr; p.k_sh = k_sh;
+  p.v = (const bf16_t*)v_cache; p.v_sr = v_sr; p.v_sh = v_sh;
+  p.o = (bf16_t*)o; p.o_st = o_st; p.o_sh = o_sh;
+  p.lse = lse; p.lse_st = lse_st; p.lse_sh = lse_sh;
+  p.x_cu = x_cu; p.ctx_lens = context_lens;
+  p.table = block_tables; p.table_stride = table_stride; p.page_size = page_size;
+  p.G = QH / KH; p.KH = KH;
+  p.scale_log2 = sm_scale * NSA_LOG2E;
+  p.kernel_size = 1; p.stride = 1; p.window = window;
+  return nsa_fwd_tile_launch(p, 1, true, B, x_maxlen, D, VD, (hipStream_t)stream);
+}
+
+int nsa_paged_topk_select(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr,
+                          int64_t k_sh, const float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk,
+                          int64_t tk_sh, int64_t tk_st, const int32_t* x_cu, const int32_t* context_lens,
+                          const int32_t* cmp_block_tables, int table_stride, int page_size, int B, int x_maxlen,
+                          int fixed_num_slc_blocks, int QH, int KH, int D, int kernel_size, int stride,
+                          int block_size, int top_n, int num_init, int num_local, int ignore_index, float sm_scale,
+                          void* stream) {
+  int rc = check_heads("paged_topk_select", QH, KH, D, 32);
+  if (rc) return rc;
+  rc = check_nsa_sizes("paged_topk_select", kernel_size, stride, block_size);
+  if (rc) return rc;
+  rc = check_page("paged_topk_select", page_size);
+  if (rc) return rc;
+  NSA_REQUIRE(top_n >= 1 && top_n <= 64, NSA_ERR_BAD_ARG, "paged_topk_select: top_n %d must be in [1,64]", top_n);
+  NSA_REQUIRE(num_init >= 0 && num_local >= 0 && num_init + num_local <= top_n, NSA_ERR_BAD_ARG,
+              "paged_topk_select: num_init %d + num_local %d must be <= top_n %d", num_init, num_local, top_n);
+  NSA_REQUIRE(fixed_num_slc_blocks >= 1, NSA_ERR_BAD_ARG, "paged_topk_select: fixed_num_slc_blocks must be >= 1");
+  NsaTopkParams p{};
+  p.q = (const bf16_t*)q; p.q_st = q_st; p.q_sh = q_sh;
+  p.ck = (const bf16_t*)k_cache; p.ck_sr = k_sr; p.ck_sh = k_sh;
+  p.lse = lse; p.lse_st = lse_st; p.lse_sh = lse_sh;
+  p.topk = topk; p.tk_sh = tk_sh; p.tk_st = tk_st;
+  p.x_cu = x_cu; p.ctx_lens = context_lens;
+  p.table = cmp_block_tables; p.table_stride = table_stride; p.page_size = page_size;
+  p.G = QH / KH; p.KH = KH;
+  p.scale_log2 = sm_scale * NSA_LOG2E;
+  p.kernel_size = kernel_size; p.stride = stride; p.block_size = block_size;
+  p.top_n = top_n; p.num_init = num_init; p.num_local = num_local; p.ignore_index = ignore_index;
+  p.nb_max = fixed_num_slc_blocks;
+  return nsa_topk_launch(p, true, B, x_maxlen, D, (hipStream_t)stream);
+}
+
+int nsa_paged_slc_attn_fwd(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr,
+                           int64_t k_sh, const void* v_cache, int64_t v_sr, int64_t v_sh, const int32_t* topk,
+                           int64_t tk_sh, int64_t tk_st, void* o, int64_t o_st, int64_t o_sh, float* lse,
+                           int64_t lse_st, int64_t lse_sh, const int32_t* x_cu, const int32_t* context_lens,
+                           const int32_t* block_tables, int table_stride, int page_size, int B, int x_maxlen,
+                           int QH, int KH, int D, int VD, int block_size, int top_n, float sm_scale, void* stream) {
+  int rc = check_heads("paged_slc_attn_fwd", QH, KH, D, VD);
+  if (rc) return rc;
+  rc = check_page("paged_slc_attn_fwd", page_size);
+  if (rc) return rc;
+  NSA_REQUIRE(block_size % 64 == 0 && block_size > 0, NSA_ERR_UNSUPPORTED,
+              "paged_slc_attn_fwd: block_size %d must be a multiple of 64", block_size);
+  NSA_REQUIRE(top_n >= 1 && top_n <= 64, NSA_ERR_BAD_ARG, "paged_slc_attn_fwd: top_n %d must be in [1,64]", top_n);
+  NsaSlcParams p{};
+  p.q = (const bf16_t*)q; p.q_st = q_st; p.q_sh = q_sh;
+  p.k = (const bf16_t*)k_cache; p.k_sr = k_sr; p.k_sh = k_sh;
+  p.v = (const bf16_t*)v_cache; p.v_sr = v_sr; p.v_sh = v_sh;
+  p.o = (bf16_t*)o; p.o_st = o_st; p.o_sh = o_sh;
+  p.lse = lse; p.lse_st = lse_st; p.lse_sh = lse_sh;
+  p.topk = topk; p.tk_sh = tk_sh; p.tk_st = tk_st;
+  p.x_cu = x_cu; p.ctx_lens = context_lens;
+  p.table = block_tables; p.table_stride = table_stride; p.page_size = page_size;
+  p.G = QH / KH; p.KH = KH; p.top_n = top_n; p.block_size = block_size;
+  p.scale_log2 = sm_scale * NSA_LOG2E;
+  return nsa_slc_fwd_launch(p, true, B, x_maxlen, D, VD, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,62 @@
+"""Paged-KV inference entry points (mirrors upstream flash_nsa/inference/__init__.py:21-257).
+
+Both functions expect the new tokens' K/V to be already written into the pool and `context_lens` to include
+them; they write the newly completed compressed rows into the same pool (mean pooling only, as upstream) and
+never synchronise with the host, so the decode step can be captured in a HIP graph."""
+from .stages import (mean_pooling_prefill, kv_mean_pooling_decode, cmp_attn_prefill, cmp_attn_decode, topk_prefill,
+                     topk_decode, slc_attn_prefill, fused_slc_swa_attn_decode, swa_prefill, combine_prefill,
+                     combine_decode, mean_pooling_decode, slc_attn_decode)
+
+
+def nsa_prefill(q, k, v, w, x_cu_seqlens, y_cu_seqlens, x_maxlen, y_maxlen, context_lens, block_tables,
+                cmp_slot_mapping, cmp_block_tables, fixed_y_maxlen=8192, fixed_num_slc_blocks=2048, kernel_size=32,
+                stride=16, block_size=64, top_n=16, num_init_blocks=1, num_local_blocks=2, window_size=512,
+                sm_scale=None):
+    """Chunked / prefix-cached prefill.
+    q [t,QH,D] new tokens only; k, v [pages, page_size, KH, D|VD] pools; w [t,QH,3];
+    x_cu_seqlens [B+1] offsets of the new tokens; y_cu_seqlens [B+1] offsets of ALL compressed rows per request;
+    context_lens [B] total lengths; block_tables [B,N1]; cmp_slot_mapping [y_cu[-1]] flat destination row of each
+    compressed row or -1 if it was pooled by an earlier chunk; cmp_block_tables [B,N2].  Returns o [t,QH,VD]."""
+    assert k.size(1) % 64 == 0, "page size must be a multiple of 64"
+    if sm_scale is None:
+        sm_scale = q.size(-1) ** -0.5
+    mean_pooling_prefill(k, y_cu_seqlens, y_maxlen, block_table=block_tables, slot_mapping=cmp_slot_mapping,
+                         kernel_size=kernel_size, stride=stride)
+    mean_pooling_prefill(v, y_cu_seqlens, y_maxlen, block_table=block_tables, slot_mapping=cmp_slot_mapping,
+                         kernel_size=kernel_size, stride=stride)
+    cmp_o, lse = cmp_attn_prefill(q, k, v, x_cu_seqlens, x_maxlen, block_tables=cmp_block_tables,
+                                  context_lens=context_lens, kernel_size=kernel_size, stride=stride,
+                                  sm_scale=sm_scale)
+    topk = topk_prefill(q, k, lse, x_cu_seqlens, x_maxlen, y_maxlen, block_tables=cmp_block_tables,
+                        context_lens=context_lens, fixed_y_maxlen=fixed_y_maxlen,
+                        fixed_num_slc_blocks=fixed_num_slc_blocks, sm_scale=sm_scale, kernel_size=kernel_size,
+                        stride=stride, block_size=block_size, top_n=top_n, num_inital=num_init_blocks,
+                        num_local=num_local_blocks)
+    slc_o, _ = slc_attn_prefill(q, k, v, topk, x_cu_seqlens, x_maxlen, block_tables=block_tables,
+                                context_lens=context_lens, block_size=block_size, top_n=top_n, sm_scale=sm_scale)
+    swa_o = swa_prefill(q, k, v, x_cu_seqlens, x_maxlen, block_tables=block_tables, context_lens=context_lens,
+                        window_size=window_size, sm_scale=sm_scale)
+    return combine_prefill(cmp_o, slc_o, swa_o, w)
+
+
+def nsa_decode(q, k, v, w, context_lens, block_tables, cmp_slot_mapping, cmp_block_tables, cmp_num_splits=0,
+               slc_num_splits=0, fixed_y_maxlen=8192, fixed_num_slc_blocks=2048, kernel_size=32, stride=16,
+               block_size=64, top_n=16, num_init_blocks=1, num_local_blocks=2, window_size=512, sm_scale=None):
+    """One query token per request.  q [B,QH,D]; w [B,QH,3]; cmp_slot_mapping [B] (-1: no compressed row completes
+    at this step).  Rows with context_lens == 0 (graph padding) produce zeros.  Returns o [B,QH,VD]."""
+    assert k.size(1) % 64 == 0, "page size must be a multiple of 64"
+    if sm_scale is None:
+        sm_scale = q.size(-1) ** -0.5
+    kv_mean_pooling_decode(k, v, block_table=block_tables, slot_mapping=cmp_slot_mapping, context_lens=context_lens,
+                           kernel_size=kernel_size, stride=stride)
+    cmp_o, lse = cmp_attn_decode(q, k, v, block_tables=cmp_block_tables, context_lens=context_lens,
+                                 num_splits=cmp_num_splits, kernel_size=kernel_size, stride=stride,
+                                 sm_scale=sm_scale)
+    topk = topk_decode(q, k, lse, fixed_y_maxlen=fixed_y_maxlen, fixed_num_slc_blocks=fixed_num_slc_blocks,
+                       block_tables=cmp_block_tables, context_lens=context_lens, kernel_size=kernel_size,
+                       stride=stride, block_size=block_size, top_n=top_n, num_inital=num_init_blocks,
+                       num_local=num_local_blocks, sm_scale=sm_scale)
+    slc_o, swa_o = fused_slc_swa_attn_decode(q, k, v, topk, num_splits=slc_num_splits, block_tables=block_tables,
+                                             context_lens=context_lens, block_size=block_size, top_n=top_n,
+                                             window_size=window_size, sm_scale=sm_scale)
+    return combine_decode(cmp_o, slc_o, swa_o, w)

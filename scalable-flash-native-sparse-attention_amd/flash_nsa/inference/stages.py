@@ -1,0 +1,179 @@
+"""Stages of the paged-KV inference path (mirrors the stage functions of upstream flash_nsa/inference/*.py).
+Prefill stages take the new tokens of every request packed as [t, heads, dim] with x_cu_seqlens; decode stages
+take one token per request [B, heads, dim]."""
+import torch
+
+from .. import _lib
+from ..ops._common import check_bf16
+from ..ops.combine import combine_fwd
+
+_ARANGE = {}
+
+
+def _decode_cu(B, device):
+    """[0,1,...,B] int32 on the device, cached so that a captured decode step allocates nothing for it."""
+    key = (B, str(device))
+    t = _ARANGE.get(key)
+    if t is None:
+        t = torch.arange(B + 1, dtype=torch.int32, device=device)
+        _ARANGE[key] = t
+    return t
+
+
+def _pool_args(cache):
+    assert cache.dim() == 4 and cache.is_contiguous(), "cache must be a contiguous [pages, page_size, KH, D] tensor"
+    check_bf16(cache)
+    P, page, KH, D = cache.shape
+    return page, KH, D, cache.stride(1), cache.stride(2)
+
+
+def _i32(t):
+    assert t.dtype == torch.int32 and t.is_contiguous(), "index tensors must be contiguous int32"
+    return t
+
+
+# ------------------------------------------------------------------------------------------------ pooling
+def mean_pooling_prefill(x, y_cu_seqlens, y_maxlen, block_table, slot_mapping, kernel_size=32, stride=16):
+    """In place: every compressed row whose slot != -1 is pooled from the raw rows (read through block_table)
+    and written to flat pool row `slot` of the same tensor x [pages, page_size, H, D]."""
+    page, H, D, sr, sh = _pool_args(x)
+    B = y_cu_seqlens.numel() - 1
+    _lib.call("nsa_paged_pool_prefill", x.data_ptr(), sr, sh, _i32(y_cu_seqlens).data_ptr(),
+              _i32(block_table).data_ptr(), block_table.stride(0), _i32(slot_mapping).data_ptr(), B, int(y_maxlen),
+              page, H, D, kernel_size, stride, _lib.stream_ptr())
+    return x
+
+
+def kv_mean_pooling_decode(k, v, block_table, slot_mapping, context_lens, kernel_size=32, stride=16):
+    """In place: requests with slot != -1 and len >= kernel pool their last complete window of K and V."""
+    page, H, Dk, ksr, ksh = _pool_args(k)
+    _, _, Dv, vsr, vsh = _pool_args(v)
+    B = context_lens.numel()
+    _lib.call("nsa_paged_pool_decode", k.data_ptr(), ksr, ksh, Dk, v.data_ptr(), vsr, vsh, Dv,
+              _i32(context_lens).data_ptr(), _i32(block_table).data_ptr(), block_table.stride(0),
+              _i32(slot_mapping).data_ptr(), B, page, H, kernel_size, stride, _lib.stream_ptr())
+
+
+def mean_pooling_decode(x, block_table, slot_mapping, context_lens, kernel_size=32, stride=16):
+    kv_mean_pooling_decode(x, x, block_table, slot_mapping, context_lens, kernel_size, stride)
+
+
+# ------------------------------------------------------------------------------------------------ compressed attn
+def cmp_attn_prefill(q, k, v, x_cu_seqlens, x_maxlen, block_tables, context_lens, kernel_size=32, stride=16,
+                     sm_scale=None):
+    """-> (o [t,QH,VD], lse [QH,t] fp32 log2).  block_tables: the COMPRESSED-row tables."""
+    check_bf16(q)
+    page, KH, D, ksr, ksh = _pool_args(k)
+    _, _, VD, vsr, vsh = _pool_args(v)
+    t, QH, _ = q.shape
+    B = x_cu_seqlens.numel() - 1
+    sm_scale = q.size(-1) ** -0.5 if sm_scale is None else sm_scale
+    o = torch.empty(t, QH, VD, device=q.device, dtype=q.dtype)
+    lse = torch.empty(QH, t, device=q.device, dtype=torch.float32)
+    _lib.call("nsa_paged_cmp_attn_fwd", q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), ksr, ksh, v.data_ptr(),
+              vsr, vsh, o.data_ptr(), o.stride(0), o.stride(1), lse.data_ptr(), lse.stride(1), lse.stride(0),
+              _i32(x_cu_seqlens).data_ptr(), _i32(context_lens).data_ptr(), _i32(block_tables).data_ptr(),
+              block_tables.stride(0), page, B, int(x_maxlen), QH, KH, D, VD, kernel_size, stride, sm_scale,
+              _lib.stream_ptr())
+    return o, lse
+
+
+def cmp_attn_decode(q, k, v, block_tables, context_lens, num_splits=0, kernel_size=32, stride=16, sm_scale=None,
+                    bench=False):
+    """q [B,QH,D] -> (o [B,QH,VD], lse [B,QH]).  num_splits is accepted for call compatibility."""
+    B = q.size(0)
+    o, lse = cmp_attn_prefill(q, k, v, _decode_cu(B, q.device), 1, block_tables, context_lens, kernel_size, stride,
+                              sm_scale)
+    return o, lse.t()
+
+
+# ------------------------------------------------------------------------------------------------ top-k
+def topk_prefill(q, k, lse, x_cu_seqlens, x_maxlen, y_maxlen, block_tables, context_lens, fixed_y_maxlen=8192,
+                 fixed_num_slc_blocks=2048, sm_scale=None, kernel_size=32, stride=16, block_size=64, top_n=16,
+                 num_inital=1, num_local=2):
+    """-> topk [KH,t,top_n] int32, unused slots = -1.  lse [QH,t] from cmp_attn_prefill."""
+    check_bf16(q)
+    page, KH, D, ksr, ksh = _pool_args(k)
+    t, QH, _ = q.shape
+    B = x_cu_seqlens.numel() - 1
+    sm_scale = q.size(-1) ** -0.5 if sm_scale is None else sm_scale
+    assert lse.dtype == torch.float32 and lse.shape == (QH, t)
+    topk = torch.empty(KH, t, top_n, device=q.device, dtype=torch.int32)
+    _lib.call("nsa_paged_topk_select", q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), ksr, ksh, lse.data_ptr(),
+              lse.stride(1), lse.stride(0), topk.data_ptr(), topk.stride(0), topk.stride(1),
+              _i32(x_cu_seqlens).data_ptr(), _i32(context_lens).data_ptr(), _i32(block_tables).data_ptr(),
+              block_tables.stride(0), page, B, int(x_maxlen), int(fixed_num_slc_blocks), QH, KH, D, kernel_size,
+              stride, block_size, top_n, num_inital, num_local, -1, sm_scale, _lib.stream_ptr())
+    return topk
+
+
+def topk_decode(q, k, lse, block_tables, context_lens, fixed_y_maxlen=8192, fixed_num_slc_blocks=2048,
+                kernel_size=32, stride=16, block_size=64, top_n=16, num_inital=1, num_local=2, sm_scale=None):
+    """q [B,QH,D], lse [B,QH] -> topk [KH,B,top_n] int32"""
+    B = q.size(0)
+    return topk_prefill(q, k, lse.t(), _decode_cu(B, q.device), 1, fixed_y_maxlen, block_tables, context_lens,
+                        fixed_y_maxlen, fixed_num_slc_blocks, sm_scale, kernel_size, stride, block_size, top_n,
+                        num_inital, num_local)
+
+
+# ------------------------------------------------------------------------------------------------ selected / window
+def slc_attn_prefill(q, k, v, topk, x_cu_seqlens, x_maxlen, block_tables, context_lens, block_size=64, top_n=16,
+                     sm_scale=None):
+    """-> (o [t,QH,VD], lse [t,QH])"""
+    check_bf16(q)
+    page, KH, D, ksr, ksh = _pool_args(k)
+    _, _, VD, vsr, vsh = _pool_args(v)
+    t, QH, _ = q.shape
+    B = x_cu_seqlens.numel() - 1
+    sm_scale = q.size(-1) ** -0.5 if sm_scale is None else sm_scale
+    assert topk.dtype == torch.int32 and topk.shape == (KH, t, top_n) and topk.stride(-1) == 1
+    o = torch.empty(t, QH, VD, device=q.device, dtype=q.dtype)
+    lse = torch.empty(t, QH, device=q.device, dtype=torch.float32)
+    _lib.call("nsa_paged_slc_attn_fwd", q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), ksr, ksh, v.data_ptr(),
+              vsr, vsh, topk.data_ptr(), topk.stride(0), topk.stride(1), o.data_ptr(), o.stride(0), o.stride(1),
+              lse.data_ptr(), lse.stride(0), lse.stride(1), _i32(x_cu_seqlens).data_ptr(),
+              _i32(context_lens).data_ptr(), _i32(block_tables).data_ptr(), block_tables.stride(0), page, B,
+              int(x_maxlen), QH, KH, D, VD, block_size, top_n, sm_scale, _lib.stream_ptr())
+    return o, lse
+
+
+def swa_prefill(q, k, v, x_cu_seqlens, x_maxlen, block_tables, context_lens, window_size=512, sm_scale=None):
+    """Paged causal sliding-window attention (upstream calls FlashAttention with a page table here)."""
+    check_bf16(q)
+    page, KH, D, ksr, ksh = _pool_args(k)
+    _, _, VD, vsr, vsh = _pool_args(v)
+    t, QH, _ = q.shape
+    B = x_cu_seqlens.numel() - 1
+    sm_scale = q.size(-1) ** -0.5 if sm_scale is None else sm_scale
+    o = torch.empty(t, QH, VD, device=q.device, dtype=q.dtype)
+    _lib.call("nsa_paged_swa_fwd", q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), ksr, ksh, v.data_ptr(), vsr,
+              vsh, o.data_ptr(), o.stride(0), o.stride(1), None, 0, 0, _i32(x_cu_seqlens).data_ptr(),
+              _i32(context_lens).data_ptr(), _i32(block_tables).data_ptr(), block_tables.stride(0), page, B,
+              int(x_maxlen), QH, KH, D, VD, window_size, sm_scale, _lib.stream_ptr())
+    return o
+
+
+def slc_attn_decode(q, k, v, topk, block_tables, context_lens, num_splits=0, block_size=64, top_n=16,
+                    sm_scale=None):
+    B = q.size(0)
+    return slc_attn_prefill(q, k, v, topk, _decode_cu(B, q.device), 1, block_tables, context_lens, block_size,
+                            top_n, sm_scale)
+
+
+def fused_slc_swa_attn_decode(q, k, v, topk, block_tables, context_lens, num_splits=0, block_size=64, top_n=16,
+                              window_size=512, sm_scale=None, bench=False):
+    """-> (slc_o, swa_o), each [B,QH,VD]"""
+    B = q.size(0)
+    cu = _decode_cu(B, q.device)
+    slc_o, _ = slc_attn_prefill(q, k, v, topk, cu, 1, block_tables, context_lens, block_size, top_n, sm_scale)
+    swa_o = swa_prefill(q, k, v, cu, 1, block_tables, context_lens, window_size, sm_scale)
+    return slc_o, swa_o
+
+
+# ------------------------------------------------------------------------------------------------ combine
+def combine_prefill(a, b, c, w):
+    return combine_fwd(a, b, c, w)
+
+
+def combine_decode(a, b, c, w):
+    return combine_fwd(a, b, c, w)
