@@ -2,6 +2,7 @@
 // that a kernel is never launched on shapes its tiling does not cover.
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <math.h>
 #include "nsa_common.h"
 #include "nsa_api_internal.h"
@@ -13,6 +14,11 @@ void nsa_set_error(const char* fmt, ...) {
   va_start(ap, fmt);
   vsnprintf(g_err, sizeof(g_err), fmt, ap);
   va_end(ap);
+}
+
+int nsa_tuning_knob(const char* env_name, int default_value) {
+  const char* v = getenv(env_name);
+  return (v && *v) ? atoi(v) : default_value;
 }
 
 int nsa_check_launch(const char* what) {

@@ -25,6 +25,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
   constexpr int RT = 64;
   constexpr int QLD = D + 8;
   constexpr int OLD = VD + 8;
+  constexpr int T_INVALID = -0x40000000;
   __shared__ __attribute__((aligned(16))) bf16_t Qs[RT * QLD];
   __shared__ __attribute__((aligned(16))) bf16_t dOs[RT * OLD];
   __shared__ __attribute__((aligned(16))) float lse_s[RT];
@@ -33,12 +34,13 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31;
   const int hl = lane >> 5;
   const int g16 = lane >> 4, i16 = lane & 15;
   const int kh = blockIdx.z;
   const int G = p.G;
+  const int gshift = (G & (G - 1)) == 0 ? __builtin_ctz(G) : -1;  // power-of-two groups avoid the division
 
   int b, key0, row_begin, row_end;  // rows in the group-row space of sequence b (MODE_SLC: positions in the list)
   const int32_t* list = nullptr;
@@ -93,6 +95,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
       return;
     }
   }
+  if (row_begin >= row_end) return;
 
   // ---- this wave's keys: K and V fragments as B operands ----
   const int kw0 = key0 + wave * 32;
@@ -119,63 +122,75 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
   const float sc = p.scale_log2;
   const bool wave_has_keys = kw0 < nkeys;
 
+  // ---- software pipeline over 64-row tiles: registers hold the next tile while the current one is computed.
+  // Rows past the end of the range are replaced by the last valid row and flagged with an invalid position,
+  // which zeroes their probabilities.
+  constexpr int QP = D / 8, OP = VD / 8;
+  constexpr int QJ = (RT * QP) / NT, OJ = (RT * OP) / NT;
+  bf16x8 qreg[QJ], oreg[OJ];
+  float lse_reg = 0.f, delta_reg = 0.f;
+  int t_reg = T_INVALID;
+  auto row_of = [&](int rr, int& n, int& g) {  // group-row -> (token local to the sequence, head in group)
+    if (gshift >= 0) { n = rr >> gshift; g = rr & (G - 1); }
+    else { n = rr / G; g = rr - n * G; }
+    if (MODE == MODE_SLC) n = list[n];
+  };
+  auto gload = [&](int rt0) {
+#pragma unroll
+    for (int j = 0; j < QJ; j++) {
+      int pc = tid + j * NT;
+      int rr = min(rt0 + pc / QP, row_end - 1), dp = pc % QP;
+      int n, g;
+      row_of(rr, n, g);
+      qreg[j] = ld_global_b128(p.q + (int64_t)(x0 + n) * p.q_st + (int64_t)(kh * G + g) * p.q_sh + dp * 8);
+    }
+#pragma unroll
+    for (int j = 0; j < OJ; j++) {
+      int pc = tid + j * NT;
+      int rr = min(rt0 + pc / OP, row_end - 1), dp = pc % OP;
+      int n, g;
+      row_of(rr, n, g);
+      oreg[j] = ld_global_b128(p.dO + (int64_t)(x0 + n) * p.do_st + (int64_t)(kh * G + g) * p.do_sh + dp * 8);
+    }
+    if (tid < RT) {
+      int rr = rt0 + tid;
+      bool ok = rr < row_end;
+      int n, g;
+      row_of(ok ? rr : row_end - 1, n, g);
+      int64_t tok = x0 + n;
+      int head = kh * G + g;
+      lse_reg = p.lse[tok * p.lse_st + (int64_t)head * p.lse_sh];
+      delta_reg = p.delta[tok * p.delta_st + (int64_t)head * p.delta_sh];
+      t_reg = ok ? n : T_INVALID;
+    }
+  };
+  gload(row_begin);
+
   for (int rt0 = row_begin; rt0 < row_end; rt0 += RT) {
     __syncthreads();
-    // ---- stage 64 rows of Q, dO, lse, delta, position ----
-    {
-      constexpr int QP = D / 8;
 #pragma unroll
-      for (int j = 0; j < (RT * QP) / NT; j++) {
-        int pc = tid + j * NT;
-        int rl = pc / QP, dp = pc - rl * QP;
-        int rr = rt0 + rl;
-        bf16x8 val = zero_bf16x8();
-        if (rr < row_end) {
-          int n = rr / G, g = rr - n * G;
-          if (MODE == MODE_SLC) n = list[n];
-          val = ld_global_b128(p.q + (int64_t)(x0 + n) * p.q_st + (int64_t)(kh * G + g) * p.q_sh + dp * 8);
-        }
-        *reinterpret_cast<bf16x8*>(&Qs[rl * QLD + dp * 8]) = val;
-      }
-      constexpr int OP = VD / 8;
+    for (int j = 0; j < QJ; j++) {
+      int pc = tid + j * NT;
+      *reinterpret_cast<bf16x8*>(&Qs[(pc / QP) * QLD + (pc % QP) * 8]) = qreg[j];
+    }
 #pragma unroll
-      for (int j = 0; j < (RT * OP) / NT; j++) {
-        int pc = tid + j * NT;
-        int rl = pc / OP, dp = pc - rl * OP;
-        int rr = rt0 + rl;
-        bf16x8 val = zero_bf16x8();
-        if (rr < row_end) {
-          int n = rr / G, g = rr - n * G;
-          if (MODE == MODE_SLC) n = list[n];
-          val = ld_global_b128(p.dO + (int64_t)(x0 + n) * p.do_st + (int64_t)(kh * G + g) * p.do_sh + dp * 8);
-        }
-        *reinterpret_cast<bf16x8*>(&dOs[rl * OLD + dp * 8]) = val;
-      }
-      if (tid < RT) {
-        int rr = rt0 + tid;
-        float l = 0.f, dl = 0.f;
-        int tt = -0x40000000;
-        if (rr < row_end) {
-          int n = rr / G, g = rr - n * G;
-          if (MODE == MODE_SLC) n = list[n];
-          int64_t tok = x0 + n;
-          int head = kh * G + g;
-          l = p.lse[tok * p.lse_st + (int64_t)head * p.lse_sh];
-          dl = p.delta[tok * p.delta_st + (int64_t)head * p.delta_sh];
-          tt = n;
-        }
-        lse_s[tid] = l;
-        delta_s[tid] = dl;
-        t_s[tid] = tt;
-      }
+    for (int j = 0; j < OJ; j++) {
+      int pc = tid + j * NT;
+      *reinterpret_cast<bf16x8*>(&dOs[(pc / OP) * OLD + (pc % OP) * 8]) = oreg[j];
+    }
+    if (tid < RT) {
+      lse_s[tid] = lse_reg;
+      delta_s[tid] = delta_reg;
+      t_s[tid] = t_reg;
     }
     __syncthreads();
+    if (rt0 + RT < row_end) gload(rt0 + RT);
     if (!wave_has_keys) continue;
 
-    // tile position range (rows ascend in position for all three modes)
-    const int t_min = t_s[0];
+    // tile position range (rows ascend in position for all three modes); scalar values
     const int n_in = min(RT, row_end - rt0);
-    const int t_max = t_s[n_in - 1];
+    const int t_min = __builtin_amdgcn_readfirstlane(t_s[0]);
+    const int t_max = __builtin_amdgcn_readfirstlane(t_s[n_in - 1]);
     bool any_vis, full_vis;
     if (MODE == MODE_CMP) {
       any_vis = t_max >= p.stride * kw0 + p.kernel_size - 1;
@@ -195,32 +210,43 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
 #pragma unroll
       for (int i = 0; i < 16; i++) { sacc[i] = 0.f; pacc[i] = 0.f; }
       const bf16_t* qp = &Qs[(mt * 32 + l32) * QLD + hl * 8];
+      const bf16_t* dp = &dOs[(mt * 32 + l32) * OLD + hl * 8];
 #pragma unroll
       for (int kc = 0; kc < D / 16; kc++)
         sacc = mfma32(*reinterpret_cast<const bf16x8*>(qp + kc * 16), kf[kc], sacc);
-      const bf16_t* dp = &dOs[(mt * 32 + l32) * OLD + hl * 8];
 #pragma unroll
       for (int kc = 0; kc < VD / 16; kc++)
         pacc = mfma32(*reinterpret_cast<const bf16x8*>(dp + kc * 16), vf[kc], pacc);
+      // P = exp2(S*c - lse);  dS = P o (dP - delta)
 #pragma unroll
       for (int i4 = 0; i4 < 4; i4++) {
         const int rbase = mt * 32 + i4 * 8 + hl * 4;
         f32x4 l4 = *reinterpret_cast<const f32x4*>(&lse_s[rbase]);
+#pragma unroll
+        for (int ii = 0; ii < 4; ii++)
+          sacc[i4 * 4 + ii] = fast_exp2(__builtin_fmaf(sacc[i4 * 4 + ii], sc, -l4[ii]));
+      }
+      if (!full_vis) {  // wave-uniform: only tiles that straddle a visibility boundary pay for the mask
+#pragma unroll
+        for (int i4 = 0; i4 < 4; i4++) {
+          const int rbase = mt * 32 + i4 * 8 + hl * 4;
+#pragma unroll
+          for (int ii = 0; ii < 4; ii++) {
+            int tr = t_s[rbase + ii];
+            bool vis;
+            if (MODE == MODE_CMP) vis = (my_key < nkeys) && (tr >= p.stride * my_key + p.kernel_size - 1);
+            else if (MODE == MODE_SWA) vis = (my_key <= tr) && (my_key >= tr - p.window) && (my_key < nkeys);
+            else vis = (my_key <= tr) && (my_key < nkeys);
+            sacc[i4 * 4 + ii] = vis ? sacc[i4 * 4 + ii] : 0.f;
+          }
+        }
+      }
+#pragma unroll
+      for (int i4 = 0; i4 < 4; i4++) {
+        const int rbase = mt * 32 + i4 * 8 + hl * 4;
         f32x4 d4 = *reinterpret_cast<const f32x4*>(&delta_s[rbase]);
 #pragma unroll
-        for (int ii = 0; ii < 4; ii++) {
-          const int i = i4 * 4 + ii;
-          bool vis = true;
-          if (!full_vis) {
-            int tr = t_s[rbase + ii];
-            if (MODE == MODE_CMP) vis = (my_key < nkeys) && (tr >= p.stride * my_key + p.kernel_size - 1);
-            else if (MODE == MODE_SWA) vis = (my_key <= tr) && (my_key >= tr - p.window);
-            else vis = (my_key <= tr);
-          }
-          float pv = vis ? fast_exp2(sacc[i] * sc - l4[ii]) : 0.f;
-          sacc[i] = pv;
-          pacc[i] = pv * (pacc[i] - d4[ii]);
-        }
+        for (int ii = 0; ii < 4; ii++) pacc[i4 * 4 + ii] = sacc[i4 * 4 + ii] * (pacc[i4 * 4 + ii] - d4[ii]);
       }
 #pragma unroll
       for (int c = 0; c < 2; c++) {

@@ -11,8 +11,8 @@ namespace {
 constexpr int MODE_CMP = 0;
 constexpr int MODE_SWA = 1;
 
-template <int D, int VD, int MODE>
-__global__ __launch_bounds__(256) void bwd_dq_tile_kernel(NsaBwdTileParams p) {
+template <int D, int VD, int MODE, int MINB>
+__global__ __launch_bounds__(256, MINB) void bwd_dq_tile_kernel(NsaBwdTileParams p) {
   constexpr int ROWS_W = 32;
   constexpr int ROWS_WG = 4 * ROWS_W;
   constexpr int KT = 64;
@@ -23,7 +23,7 @@ __global__ __launch_bounds__(256) void bwd_dq_tile_kernel(NsaBwdTileParams p) {
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31;
   const int hl = lane >> 5;
   const int b = blockIdx.y;
@@ -90,31 +90,42 @@ __global__ __launch_bounds__(256) void bwd_dq_tile_kernel(NsaBwdTileParams p) {
   const float sc = p.scale_log2;
   const int g16 = lane >> 4, i16 = lane & 15;
 
+  // software pipeline: next tile's global loads fly while the current tile is computed; rows past the end of
+  // the key range are replaced by the last valid row (their probabilities are masked to zero)
+  constexpr int KP = D / 8, VP = VD / 8;
+  constexpr int KJ = (KT * KP) / 256, VJ = (KT * VP) / 256;
+  bf16x8 kreg[KJ], vreg[VJ];
+  auto gload = [&](int kt) {
+    const int last = key_end - 1 - kt;
+#pragma unroll
+    for (int j = 0; j < KJ; j++) {
+      int pc = tid + j * 256;
+      int kr = min(pc / KP, last), dp = pc % KP;
+      kreg[j] = ld_global_b128(p.k + ((int64_t)kbase + kt + kr) * p.k_sr + (int64_t)kh * p.k_sh + dp * 8);
+    }
+#pragma unroll
+    for (int j = 0; j < VJ; j++) {
+      int pc = tid + j * 256;
+      int kr = min(pc / VP, last), dp = pc % VP;
+      vreg[j] = ld_global_b128(p.v + ((int64_t)kbase + kt + kr) * p.v_sr + (int64_t)kh * p.v_sh + dp * 8);
+    }
+  };
+  if (key_begin < key_end) gload(key_begin);
+
   for (int kt = key_begin; kt < key_end; kt += KT) {
     __syncthreads();
-    {
-      constexpr int KP = D / 8;
 #pragma unroll
-      for (int j = 0; j < (KT * KP) / 256; j++) {
-        int pc = tid + j * 256;
-        int kr = pc / KP, dp = pc - kr * KP;
-        bf16x8 val = zero_bf16x8();
-        if (kt + kr < key_end)
-          val = ld_global_b128(p.k + ((int64_t)kbase + kt + kr) * p.k_sr + (int64_t)kh * p.k_sh + dp * 8);
-        *reinterpret_cast<bf16x8*>(&Ks[kr * KLD + dp * 8]) = val;
-      }
-      constexpr int VP = VD / 8;
+    for (int j = 0; j < KJ; j++) {
+      int pc = tid + j * 256;
+      *reinterpret_cast<bf16x8*>(&Ks[(pc / KP) * KLD + (pc % KP) * 8]) = kreg[j];
+    }
 #pragma unroll
-      for (int j = 0; j < (KT * VP) / 256; j++) {
-        int pc = tid + j * 256;
-        int kr = pc / VP, dp = pc - kr * VP;
-        bf16x8 val = zero_bf16x8();
-        if (kt + kr < key_end)
-          val = ld_global_b128(p.v + ((int64_t)kbase + kt + kr) * p.v_sr + (int64_t)kh * p.v_sh + dp * 8);
-        *reinterpret_cast<bf16x8*>(&Vs[kr * VLD + dp * 8]) = val;
-      }
+    for (int j = 0; j < VJ; j++) {
+      int pc = tid + j * 256;
+      *reinterpret_cast<bf16x8*>(&Vs[(pc / VP) * VLD + (pc % VP) * 8]) = vreg[j];
     }
     __syncthreads();
+    if (kt + KT < key_end) gload(kt + KT);
     if (!wave_active) continue;
     bool any_vis, full_vis;
     if (MODE == MODE_CMP) {
@@ -128,31 +139,44 @@ __global__ __launch_bounds__(256) void bwd_dq_tile_kernel(NsaBwdTileParams p) {
 
     f32x16 sacc[2], pacc[2];
 #pragma unroll
-    for (int nt = 0; nt < 2; nt++) {
+    for (int i = 0; i < 16; i++) { sacc[0][i] = 0.f; sacc[1][i] = 0.f; pacc[0][i] = 0.f; pacc[1][i] = 0.f; }
+    {
+      const bf16_t* kp0 = &Ks[l32 * KLD + hl * 8];
+      const bf16_t* kp1 = kp0 + 32 * KLD;
 #pragma unroll
-      for (int i = 0; i < 16; i++) { sacc[nt][i] = 0.f; pacc[nt][i] = 0.f; }
-      const bf16_t* kp = &Ks[(nt * 32 + l32) * KLD + hl * 8];
+      for (int kc = 0; kc < D / 16; kc++) {
+        sacc[0] = mfma32(*reinterpret_cast<const bf16x8*>(kp0 + kc * 16), qf[kc], sacc[0]);
+        sacc[1] = mfma32(*reinterpret_cast<const bf16x8*>(kp1 + kc * 16), qf[kc], sacc[1]);
+      }
+      const bf16_t* vp0 = &Vs[l32 * VLD + hl * 8];
+      const bf16_t* vp1 = vp0 + 32 * VLD;
 #pragma unroll
-      for (int kc = 0; kc < D / 16; kc++)
-        sacc[nt] = mfma32(*reinterpret_cast<const bf16x8*>(kp + kc * 16), qf[kc], sacc[nt]);
-      const bf16_t* vp = &Vs[(nt * 32 + l32) * VLD + hl * 8];
+      for (int kc = 0; kc < VD / 16; kc++) {
+        pacc[0] = mfma32(*reinterpret_cast<const bf16x8*>(vp0 + kc * 16), dof[kc], pacc[0]);
+        pacc[1] = mfma32(*reinterpret_cast<const bf16x8*>(vp1 + kc * 16), dof[kc], pacc[1]);
+      }
+    }
+    const float lsc = lse;
 #pragma unroll
-      for (int kc = 0; kc < VD / 16; kc++)
-        pacc[nt] = mfma32(*reinterpret_cast<const bf16x8*>(vp + kc * 16), dof[kc], pacc[nt]);
+    for (int nt = 0; nt < 2; nt++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) sacc[nt][i] = fast_exp2(__builtin_fmaf(sacc[nt][i], sc, -lsc));
+    if (!full_vis) {  // wave-uniform
+#pragma unroll
+      for (int nt = 0; nt < 2; nt++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          int key = kt + nt * 32 + (i >> 2) * 8 + hl * 4 + (i & 3);
+          bool vis;
+          if (MODE == MODE_CMP) vis = (key < nkeys) && (t >= p.stride * key + p.kernel_size - 1);
+          else vis = (key <= t) && (key >= t - p.window);
+          sacc[nt][i] = vis ? sacc[nt][i] : 0.f;
+        }
     }
 #pragma unroll
     for (int nt = 0; nt < 2; nt++)
 #pragma unroll
-      for (int i = 0; i < 16; i++) {
-        bool vis = true;
-        if (!full_vis) {
-          int key = kt + nt * 32 + (i >> 2) * 8 + hl * 4 + (i & 3);
-          if (MODE == MODE_CMP) vis = (key < nkeys) && (t >= p.stride * key + p.kernel_size - 1);
-          else vis = (key <= t) && (key >= t - p.window);
-        }
-        float pv = vis ? fast_exp2(sacc[nt][i] * sc - lse) : 0.f;
-        sacc[nt][i] = pv * (pacc[nt][i] - delta);  // dS^T (without the softmax scale)
-      }
+      for (int i = 0; i < 16; i++) sacc[nt][i] *= (pacc[nt][i] - delta);  // dS^T (without the softmax scale)
 #pragma unroll
     for (int c = 0; c < 4; c++) {
       const int nt = c >> 1, ch = c & 1;
@@ -194,9 +218,12 @@ template <int MODE>
 int dispatch(const NsaBwdTileParams& p, int B, int max_q_len, int D, int VD, hipStream_t stream) {
   if (B <= 0 || max_q_len <= 0) return NSA_OK;
   dim3 grid(cdiv_i(max_q_len * p.G, 128), B, p.KH);
-  if (D == 128 && VD == 128) bwd_dq_tile_kernel<128, 128, MODE><<<grid, 256, 0, stream>>>(p);
-  else if (D == 64 && VD == 64) bwd_dq_tile_kernel<64, 64, MODE><<<grid, 256, 0, stream>>>(p);
-  else if (D == 192 && VD == 128) bwd_dq_tile_kernel<192, 128, MODE><<<grid, 256, 0, stream>>>(p);
+  static const int minb = nsa_tuning_knob("NSA_DQ_MINB", 1);
+  if (D == 128 && VD == 128) {
+    if (minb == 2) bwd_dq_tile_kernel<128, 128, MODE, 2><<<grid, 256, 0, stream>>>(p);
+    else bwd_dq_tile_kernel<128, 128, MODE, 1><<<grid, 256, 0, stream>>>(p);
+  } else if (D == 64 && VD == 64) bwd_dq_tile_kernel<64, 64, MODE, 2><<<grid, 256, 0, stream>>>(p);
+  else if (D == 192 && VD == 128) bwd_dq_tile_kernel<192, 128, MODE, 1><<<grid, 256, 0, stream>>>(p);
   else {
     nsa_set_error("attention dq: unsupported head dims D=%d VD=%d", D, VD);
     return NSA_ERR_UNSUPPORTED;

@@ -100,6 +100,7 @@ enum {
 };
 
 void nsa_set_error(const char* fmt, ...);
+int nsa_tuning_knob(const char* env_name, int default_value);  // integer tuning override read from the environment
 int nsa_check_launch(const char* what);
 
 #define NSA_REQUIRE(cond, code, ...)        \

@@ -12,14 +12,16 @@
 // operand comes from ds_read_b64_tr_b16 so V never needs an explicit transpose.
 #include "nsa_common.h"
 #include "nsa_api_internal.h"
+#include <type_traits>
 
 namespace {
 
 constexpr int MODE_CMP = 0;
 constexpr int MODE_SWA = 1;
 
-template <int D, int VD, int MODE, bool PAGED, int RS>
-__global__ __launch_bounds__(256) void fwd_tile_kernel(NsaFwdTileParams p) {
+template <int D, int VD, int MODE, bool PAGED, int RS, int MINB>
+__global__ __launch_bounds__(256, MINB) void fwd_tile_kernel(NsaFwdTileParams p) {
+  static_assert(RS == 1 || RS == 2, "one or two 32-row sets per wave");
   constexpr int ROWS_W = 32 * RS;
   constexpr int ROWS_WG = 4 * ROWS_W;
   constexpr int KT = 64;
@@ -30,9 +32,10 @@ __global__ __launch_bounds__(256) void fwd_tile_kernel(NsaFwdTileParams p) {
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31;
   const int hl = lane >> 5;
+  const int g16 = lane >> 4, i16 = lane & 15;
   const int b = blockIdx.y;
   const int kh = blockIdx.z;
   const int G = p.G;
@@ -74,13 +77,12 @@ __global__ __launch_bounds__(256) void fwd_tile_kernel(NsaFwdTileParams p) {
 #pragma unroll
     for (int kc = 0; kc < D / 16; kc++) qf[rs][kc] = ld_global_b128(qp + kc * 16);
   }
-  // wave-uniform position range
+  // wave-uniform position range (scalar registers)
   const int rw_lo = r0 + wave * ROWS_W;
   const int rw_hi = min(rw_lo + ROWS_W - 1, rows_total - 1);
   const bool wave_active = rw_lo < rows_total;
   const int tw_lo = (wave_active ? rw_lo / G : 0) + qoff;
   const int tw_hi = (wave_active ? rw_hi / G : 0) + qoff;
-  // workgroup position range
   const int t_lo = r0 / G + qoff;
   const int t_hi = min(r0 + ROWS_WG - 1, rows_total - 1) / G + qoff;
 
@@ -104,44 +106,131 @@ __global__ __launch_bounds__(256) void fwd_tile_kernel(NsaFwdTileParams p) {
 #pragma unroll
       for (int i = 0; i < 16; i++) oacc[rs][dt][i] = 0.f;
   }
-
   const float sc = p.scale_log2;
+
+  // software pipeline: the next tile's global loads are in flight while the current tile is computed.
+  // Rows past the end of the key range are replaced by the last valid row; their scores are masked, so the
+  // duplicated data never contributes.
+  constexpr int KP = D / 8, VP = VD / 8;
+  constexpr int KJ = (KT * KP) / 256, VJ = (KT * VP) / 256;
+  bf16x8 kreg[KJ], vreg[VJ];
+  auto gload = [&](int kt) {
+    int64_t page_row0 = 0;
+    if (PAGED) {
+      int pg = table[kt / p.page_size];
+      page_row0 = (int64_t)pg * p.page_size + (kt % p.page_size);
+    }
+    const int last = key_end - 1 - kt;  // >= 0
+#pragma unroll
+    for (int j = 0; j < KJ; j++) {
+      int pc = tid + j * 256;
+      int kr = min(pc / KP, last), dp = pc % KP;
+      int64_t row = PAGED ? page_row0 + kr : (int64_t)kbase + kt + kr;
+      kreg[j] = ld_global_b128(p.k + row * p.k_sr + (int64_t)kh * p.k_sh + dp * 8);
+    }
+#pragma unroll
+    for (int j = 0; j < VJ; j++) {
+      int pc = tid + j * 256;
+      int kr = min(pc / VP, last), dp = pc % VP;
+      int64_t row = PAGED ? page_row0 + kr : (int64_t)kbase + kt + kr;
+      vreg[j] = ld_global_b128(p.v + row * p.v_sr + (int64_t)kh * p.v_sh + dp * 8);
+    }
+  };
+
+  // one 64-key tile for one row set
+  auto process = [&](bool masked, auto rs_tag, int kt) {
+    constexpr int rs = decltype(rs_tag)::value;
+    // ---- S^T = K Q^T : two 32-key sub tiles, interleaved accumulators ----
+    f32x16 sacc[2];
+#pragma unroll
+    for (int i = 0; i < 16; i++) { sacc[0][i] = 0.f; sacc[1][i] = 0.f; }
+    const bf16_t* kp0 = &Ks[l32 * KLD + hl * 8];
+    const bf16_t* kp1 = kp0 + 32 * KLD;
+#pragma unroll
+    for (int kc = 0; kc < D / 16; kc++) {
+      bf16x8 k0 = *reinterpret_cast<const bf16x8*>(kp0 + kc * 16);
+      bf16x8 k1 = *reinterpret_cast<const bf16x8*>(kp1 + kc * 16);
+      sacc[0] = mfma32(k0, qf[rs][kc], sacc[0]);
+      sacc[1] = mfma32(k1, qf[rs][kc], sacc[1]);
+    }
+    // ---- mask, online softmax (running max in raw score units; scale folded into the exp2 fma) ----
+    if (masked) {  // wave-uniform: only tiles that straddle a visibility boundary pay for the mask
+      const int t = t_row[rs];
+#pragma unroll
+      for (int nt = 0; nt < 2; nt++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          int key = kt + nt * 32 + (i >> 2) * 8 + hl * 4 + (i & 3);
+          bool vis;
+          if (MODE == MODE_CMP) vis = (key < nkeys) && (t >= p.stride * key + p.kernel_size - 1);
+          else vis = (key <= t) && (key >= t - p.window);
+          sacc[nt][i] = vis ? sacc[nt][i] : NSA_NEG_INF;
+        }
+    }
+    float tmax = NSA_NEG_INF;
+#pragma unroll
+    for (int nt = 0; nt < 2; nt++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) tmax = fmaxf(tmax, sacc[nt][i]);
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_old = m_run[rs];
+    const float m_new = fmaxf(m_old, tmax);
+    const float m_safe = (m_new == NSA_NEG_INF) ? 0.f : m_new;
+    const float msc = m_safe * sc;
+    m_run[rs] = m_new;
+    float psum = 0.f;
+#pragma unroll
+    for (int nt = 0; nt < 2; nt++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        float pv = fast_exp2(__builtin_fmaf(sacc[nt][i], sc, -msc));
+        sacc[nt][i] = pv;
+        psum += pv;
+      }
+    if (__builtin_amdgcn_ballot_w64(m_new != m_old) != 0) {  // rescale only when some row's max moved
+      const float alpha = fast_exp2((m_old - m_safe) * sc);
+      l_run[rs] *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < VD / 32; dt++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) oacc[rs][dt][i] *= alpha;
+    }
+    l_run[rs] += psum;
+
+    // ---- O^T += V^T P^T ----
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      const int nt = c >> 1, ch = c & 1;
+      bf16x8 pf = pack8(sacc[nt][ch * 8 + 0], sacc[nt][ch * 8 + 1], sacc[nt][ch * 8 + 2], sacc[nt][ch * 8 + 3],
+                        sacc[nt][ch * 8 + 4], sacc[nt][ch * 8 + 5], sacc[nt][ch * 8 + 6], sacc[nt][ch * 8 + 7]);
+      const int kb0 = nt * 32 + (2 * ch) * 8 + hl * 4;
+      const int kb1 = kb0 + 8;
+#pragma unroll
+      for (int dt = 0; dt < VD / 32; dt++) {
+        const int col = dt * 32 + (g16 & 1) * 16 + 4 * (i16 & 3);
+        bf16x4 v0 = lds_read_tr(&Vs[(kb0 + (i16 >> 2)) * VLD + col]);
+        bf16x4 v1 = lds_read_tr(&Vs[(kb1 + (i16 >> 2)) * VLD + col]);
+        oacc[rs][dt] = mfma32(cat4(v0, v1), pf, oacc[rs][dt]);
+      }
+    }
+  };
+
+  if (key_begin < key_end) gload(key_begin);
 
   for (int kt = key_begin; kt < key_end; kt += KT) {
     __syncthreads();
-    // ---- stage K and V tiles ----
-    {
-      int64_t page_row0 = 0;
-      if (PAGED) {
-        int pg = table[kt / p.page_size];
-        page_row0 = (int64_t)pg * p.page_size + (kt % p.page_size);
-      }
-      constexpr int KP = D / 8;
 #pragma unroll
-      for (int j = 0; j < (KT * KP) / 256; j++) {
-        int pc = tid + j * 256;
-        int kr = pc / KP, dp = pc - kr * KP;
-        bf16x8 val = zero_bf16x8();
-        if (kt + kr < key_end) {
-          int64_t row = PAGED ? page_row0 + kr : (int64_t)kbase + kt + kr;
-          val = ld_global_b128(p.k + row * p.k_sr + (int64_t)kh * p.k_sh + dp * 8);
-        }
-        *reinterpret_cast<bf16x8*>(&Ks[kr * KLD + dp * 8]) = val;
-      }
-      constexpr int VP = VD / 8;
+    for (int j = 0; j < KJ; j++) {
+      int pc = tid + j * 256;
+      *reinterpret_cast<bf16x8*>(&Ks[(pc / KP) * KLD + (pc % KP) * 8]) = kreg[j];
+    }
 #pragma unroll
-      for (int j = 0; j < (KT * VP) / 256; j++) {
-        int pc = tid + j * 256;
-        int kr = pc / VP, dp = pc - kr * VP;
-        bf16x8 val = zero_bf16x8();
-        if (kt + kr < key_end) {
-          int64_t row = PAGED ? page_row0 + kr : (int64_t)kbase + kt + kr;
-          val = ld_global_b128(p.v + row * p.v_sr + (int64_t)kh * p.v_sh + dp * 8);
-        }
-        *reinterpret_cast<bf16x8*>(&Vs[kr * VLD + dp * 8]) = val;
-      }
+    for (int j = 0; j < VJ; j++) {
+      int pc = tid + j * 256;
+      *reinterpret_cast<bf16x8*>(&Vs[(pc / VP) * VLD + (pc % VP) * 8]) = vreg[j];
     }
     __syncthreads();
+    if (kt + KT < key_end) gload(kt + KT);
     if (!wave_active) continue;
 
     // wave-uniform visibility classification of this tile
@@ -154,79 +243,8 @@ __global__ __launch_bounds__(256) void fwd_tile_kernel(NsaFwdTileParams p) {
       full_vis = (kt + KT - 1 <= tw_lo) && (kt >= tw_hi - p.window);
     }
     if (!any_vis) continue;
-
-#pragma unroll
-    for (int rs = 0; rs < RS; rs++) {
-      // ---- S^T = K Q^T : two 32-key sub tiles ----
-      f32x16 sacc[2];
-#pragma unroll
-      for (int nt = 0; nt < 2; nt++) {
-#pragma unroll
-        for (int i = 0; i < 16; i++) sacc[nt][i] = 0.f;
-        const bf16_t* kp = &Ks[(nt * 32 + l32) * KLD + hl * 8];
-#pragma unroll
-        for (int kc = 0; kc < D / 16; kc++) {
-          bf16x8 kf = *reinterpret_cast<const bf16x8*>(kp + kc * 16);
-          sacc[nt] = mfma32(kf, qf[rs][kc], sacc[nt]);
-        }
-      }
-      // ---- scale, mask, online softmax ----
-      const int t = t_row[rs];
-      float tmax = NSA_NEG_INF;
-#pragma unroll
-      for (int nt = 0; nt < 2; nt++) {
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-          float s = sacc[nt][i] * sc;
-          if (!full_vis) {
-            int key = kt + nt * 32 + (i >> 2) * 8 + hl * 4 + (i & 3);
-            bool vis;
-            if (MODE == MODE_CMP) vis = (key < nkeys) && (t >= p.stride * key + p.kernel_size - 1);
-            else vis = (key <= t) && (key >= t - p.window);
-            s = vis ? s : NSA_NEG_INF;
-          }
-          sacc[nt][i] = s;
-          tmax = fmaxf(tmax, s);
-        }
-      }
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-      float m_new = fmaxf(m_run[rs], tmax);
-      float m_safe = (m_new == NSA_NEG_INF) ? 0.f : m_new;
-      float alpha = fast_exp2(m_run[rs] - m_safe);
-      m_run[rs] = m_new;
-      float psum = 0.f;
-#pragma unroll
-      for (int nt = 0; nt < 2; nt++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-          float pv = fast_exp2(sacc[nt][i] - m_safe);
-          sacc[nt][i] = pv;
-          psum += pv;
-        }
-      l_run[rs] = l_run[rs] * alpha + psum;
-#pragma unroll
-      for (int dt = 0; dt < VD / 32; dt++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) oacc[rs][dt][i] *= alpha;
-
-      // ---- O^T += V^T P^T ----
-      const int g16 = lane >> 4, i16 = lane & 15;
-#pragma unroll
-      for (int c = 0; c < 4; c++) {
-        const int nt = c >> 1, ch = c & 1;
-        bf16x8 pf = pack8(sacc[nt][ch * 8 + 0], sacc[nt][ch * 8 + 1], sacc[nt][ch * 8 + 2], sacc[nt][ch * 8 + 3],
-                          sacc[nt][ch * 8 + 4], sacc[nt][ch * 8 + 5], sacc[nt][ch * 8 + 6], sacc[nt][ch * 8 + 7]);
-        const int kb0 = nt * 32 + (2 * ch) * 8 + hl * 4;
-        const int kb1 = kb0 + 8;
-#pragma unroll
-        for (int dt = 0; dt < VD / 32; dt++) {
-          const int col = dt * 32 + (g16 & 1) * 16 + 4 * (i16 & 3);
-          bf16x4 v0 = lds_read_tr(&Vs[(kb0 + (i16 >> 2)) * VLD + col]);
-          bf16x4 v1 = lds_read_tr(&Vs[(kb1 + (i16 >> 2)) * VLD + col]);
-          oacc[rs][dt] = mfma32(cat4(v0, v1), pf, oacc[rs][dt]);
-        }
-      }
-    }
+    process(!full_vis, std::integral_constant<int, 0>{}, kt);
+    if constexpr (RS > 1) process(!full_vis, std::integral_constant<int, RS - 1>{}, kt);
   }
 
   // ---- epilogue ----
@@ -246,7 +264,7 @@ __global__ __launch_bounds__(256) void fwd_tile_kernel(NsaFwdTileParams p) {
         *reinterpret_cast<bf16x4*>(op + d) = w;
       }
     if (hl == 0 && p.lse != nullptr) {
-      float lse2 = l_tot > 0.f ? m_run[rs] + fast_log2(l_tot) : 0.f;
+      float lse2 = l_tot > 0.f ? m_run[rs] * sc + fast_log2(l_tot) : 0.f;
       p.lse[tok[rs] * p.lse_st + (int64_t)head[rs] * p.lse_sh] = lse2;
     }
   }
@@ -254,11 +272,18 @@ __global__ __launch_bounds__(256) void fwd_tile_kernel(NsaFwdTileParams p) {
 
 template <int D, int VD, int MODE, bool PAGED>
 int launch_fwd_tile(const NsaFwdTileParams& p, int B, int max_q_len, hipStream_t stream) {
-  constexpr int RS = 1;
-  constexpr int ROWS_WG = 128 * RS;
   if (B <= 0 || max_q_len <= 0) return NSA_OK;
-  dim3 grid(cdiv_i(max_q_len * p.G, ROWS_WG), B, p.KH);
-  fwd_tile_kernel<D, VD, MODE, PAGED, RS><<<grid, 256, 0, stream>>>(p);
+  static const int variant = nsa_tuning_knob("NSA_FWD_VARIANT", 1);
+  if (variant == 1) {
+    dim3 grid(cdiv_i(max_q_len * p.G, 128), B, p.KH);
+    fwd_tile_kernel<D, VD, MODE, PAGED, 1, 2><<<grid, 256, 0, stream>>>(p);
+  } else if (variant == 2) {
+    dim3 grid(cdiv_i(max_q_len * p.G, 256), B, p.KH);
+    fwd_tile_kernel<D, VD, MODE, PAGED, 2, 1><<<grid, 256, 0, stream>>>(p);
+  } else {
+    dim3 grid(cdiv_i(max_q_len * p.G, 128), B, p.KH);
+    fwd_tile_kernel<D, VD, MODE, PAGED, 1, 1><<<grid, 256, 0, stream>>>(p);
+  }
   return nsa_check_launch("fwd_tile_kernel");
 }
 
