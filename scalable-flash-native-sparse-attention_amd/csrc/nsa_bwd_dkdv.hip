@@ -23,8 +23,8 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
   constexpr int NT = NW * 64;
   constexpr int KW = NW * 32;
   constexpr int RT = 64;
-  constexpr int QLD = D + 8;
-  constexpr int OLD = VD + 8;
+  constexpr int QLD = D + NSA_LDS_PAD;
+  constexpr int OLD = VD + NSA_LDS_PAD;
   constexpr int T_INVALID = -0x40000000;
   __shared__ __attribute__((aligned(16))) bf16_t Qs[RT * QLD];
   __shared__ __attribute__((aligned(16))) bf16_t dOs[RT * OLD];

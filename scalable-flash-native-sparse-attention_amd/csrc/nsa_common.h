@@ -27,6 +27,11 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 #define NSA_DEVICE __device__ __forceinline__
 #define LDS_PTR(T) __attribute__((address_space(3))) T*
 
+// Row padding (bf16 elements) of LDS tiles.  With 128-wide rows the stride is 76 dwords = 12 mod 64 banks: the
+// 16-byte row-fragment reads of 16 consecutive rows and the 4-row x 32-byte groups of the transpose reads both
+// land on distinct banks.
+constexpr int NSA_LDS_PAD = 24;
+
 constexpr float NSA_LOG2E = 1.4426950408889634f;
 constexpr float NSA_LN2 = 0.6931471805599453f;
 constexpr float NSA_NEG_INF = -__builtin_huge_valf();

@@ -25,8 +25,8 @@ __global__ __launch_bounds__(256, MINB) void fwd_tile_kernel(NsaFwdTileParams p)
   constexpr int ROWS_W = 32 * RS;
   constexpr int ROWS_WG = 4 * ROWS_W;
   constexpr int KT = 64;
-  constexpr int KLD = D + 8;
-  constexpr int VLD = VD + 8;
+  constexpr int KLD = D + NSA_LDS_PAD;
+  constexpr int VLD = VD + NSA_LDS_PAD;
   __shared__ __attribute__((aligned(16))) bf16_t Ks[KT * KLD];
   __shared__ __attribute__((aligned(16))) bf16_t Vs[KT * VLD];
 

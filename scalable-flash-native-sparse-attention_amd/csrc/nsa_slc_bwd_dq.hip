@@ -10,7 +10,7 @@ namespace {
 
 template <int D, int VD>
 __global__ __launch_bounds__(256) void slc_dq_kernel(NsaSlcBwdDqParams p) {
-  constexpr int KLD = D + 8;
+  constexpr int KLD = D + NSA_LDS_PAD;
   __shared__ __attribute__((aligned(16))) bf16_t Ks_all[4 * 64 * KLD];
   const int tid = threadIdx.x;
   const int lane = tid & 63;

@@ -12,13 +12,18 @@
 namespace {
 
 template <int D, int VD, bool PAGED>
-__global__ __launch_bounds__(256) void slc_fwd_kernel(NsaSlcParams p) {
-  constexpr int VLD = VD + 8;
-  __shared__ __attribute__((aligned(16))) bf16_t Vs_all[4 * 64 * VLD];
+__global__ __launch_bounds__(256, 2) void slc_fwd_kernel(NsaSlcParams p) {
+  // Work unit = 32 keys (half of a 64-key tile).  The K fragments and the V rows of unit u+1 are loaded into
+  // registers while unit u is computed, so the gather latency overlaps the MFMAs of the previous unit.
+  constexpr int VLD = VD + NSA_LDS_PAD;
+  constexpr int UK = 32;                      // keys per unit
+  constexpr int KC = D / 32;                  // K fragments per 16-key tile
+  constexpr int VJ = (UK * (VD / 8)) / 64;    // 16-byte V loads per lane and unit
+  __shared__ __attribute__((aligned(16))) bf16_t Vs_all[4 * UK * VLD];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
-  bf16_t* Vs = Vs_all + wave * 64 * VLD;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  bf16_t* Vs = Vs_all + wave * UK * VLD;
   const int l16 = lane & 15;
   const int kq = lane >> 4;
   const int b = blockIdx.y;
@@ -35,18 +40,21 @@ __global__ __launch_bounds__(256) void slc_fwd_kernel(NsaSlcParams p) {
   const int64_t tok = x0 + n;
   const int32_t* table = PAGED ? p.table + (int64_t)b * p.table_stride : nullptr;
   const int Bs = p.block_size;
-  const int nvalid = min(p.top_n, t / Bs + 1);
+  const int nvalid = t >= 0 ? min(p.top_n, t / Bs + 1) : 0;  // t < 0: padded request, output row = 0
+  const int upb = Bs / UK;                    // units per selection block
+  const int nu = nvalid * upb;
+  const int key_last = min(ctx - 1, t);       // last key this token may attend
 
   int g = hc * 16 + l16;
   const bool head_ok = g < p.G;
   if (!head_ok) g = p.G - 1;
   const int head = kh * p.G + g;
 
-  bf16x8 qf[D / 32];
+  bf16x8 qf[KC];
   {
     const bf16_t* qp = p.q + tok * p.q_st + (int64_t)head * p.q_sh + kq * 8;
 #pragma unroll
-    for (int kc = 0; kc < D / 32; kc++) qf[kc] = ld_global_b128(qp + kc * 32);
+    for (int kc = 0; kc < KC; kc++) qf[kc] = ld_global_b128(qp + kc * 32);
   }
   int my_blk = 0;
   if (lane < nvalid) my_blk = p.topk[(int64_t)kh * p.tk_sh + tok * p.tk_st + lane];
@@ -56,100 +64,110 @@ __global__ __launch_bounds__(256) void slc_fwd_kernel(NsaSlcParams p) {
   for (int dt = 0; dt < VD / 16; dt++) oacc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m_run = NSA_NEG_INF, l_run = 0.f;
   const float sc = p.scale_log2;
-  const int subs = Bs / 64;
 
-  for (int slot = 0; slot < nvalid; slot++) {
-    const int blk = __shfl(my_blk, slot, 64);
-    for (int sub = 0; sub < subs; sub++) {
-      const int key0 = blk * Bs + sub * 64;
-      if (key0 > t || key0 < 0) continue;  // nothing visible (also guards ignore values)
-      int64_t row0;
-      if (PAGED) {
-        int pg = table[key0 / p.page_size];
-        row0 = (int64_t)pg * p.page_size + (key0 % p.page_size);
-      } else {
-        row0 = (int64_t)x0 + key0;
-      }
-      const int kmax = min(ctx - 1, t) - key0;  // last usable key offset inside this tile (>= 0)
-
-      // ---- V tile -> registers (issued early), K fragments -> registers ----
-      bf16x8 vreg[(64 * (VD / 8)) / 64];
+  // first key of unit u (negative block ids -- ignore values -- are clamped; such units are fully masked)
+  auto unit_key0 = [&](int u) {
+    int slot = u / upb;
+    int blk = __shfl(my_blk, slot, 64);
+    return blk * Bs + (u - slot * upb) * UK;
+  };
+  auto row_of_key = [&](int key) -> int64_t {  // flat K/V row of an absolute key position
+    if (PAGED) return (int64_t)table[key / p.page_size] * p.page_size + (key % p.page_size);
+    return (int64_t)x0 + key;
+  };
+  auto issue = [&](int key0, bf16x8 (&kf)[2][KC], bf16x8 (&vr)[VJ]) {
+    // out-of-range keys are replaced by the last attendable key; their scores are masked
 #pragma unroll
-      for (int j = 0; j < (VD / 8); j++) {
-        int pc = lane + j * 64;
-        int kr = pc / (VD / 8), dp = pc - kr * (VD / 8);
-        int krc = min(kr, kmax);
-        vreg[j] = ld_global_b128(p.v + (row0 + krc) * p.v_sr + (int64_t)kh * p.v_sh + dp * 8);
-      }
-      f32x4 sacc[4];
+    for (int jt = 0; jt < 2; jt++) {
+      int key = max(0, min(key0 + jt * 16 + l16, key_last));
+      const bf16_t* kp = p.k + row_of_key(key) * p.k_sr + (int64_t)kh * p.k_sh + kq * 8;
 #pragma unroll
-      for (int jt = 0; jt < 4; jt++) {
-        sacc[jt] = f32x4{0.f, 0.f, 0.f, 0.f};
-        int kr = min(jt * 16 + l16, kmax);
-        const bf16_t* kp = p.k + (row0 + kr) * p.k_sr + (int64_t)kh * p.k_sh + kq * 8;
+      for (int kc = 0; kc < KC; kc++) kf[jt][kc] = ld_global_b128(kp + kc * 32);
+    }
 #pragma unroll
-        for (int kc = 0; kc < D / 32; kc++) {
-          bf16x8 kf = ld_global_b128(kp + kc * 32);
-          sacc[jt] = mfma16(kf, qf[kc], sacc[jt]);
-        }
-      }
-      // ---- softmax over this tile ----
-      float tmax = NSA_NEG_INF;
+    for (int j = 0; j < VJ; j++) {
+      int pc = lane + j * 64;
+      int kr = pc / (VD / 8), dp = pc % (VD / 8);
+      int key = max(0, min(key0 + kr, key_last));
+      vr[j] = ld_global_b128(p.v + row_of_key(key) * p.v_sr + (int64_t)kh * p.v_sh + dp * 8);
+    }
+  };
+  auto compute = [&](int key0, bf16x8 (&kf)[2][KC], bf16x8 (&vr)[VJ]) {
+    f32x4 sacc[2];
 #pragma unroll
-      for (int jt = 0; jt < 4; jt++)
+    for (int jt = 0; jt < 2; jt++) {
+      sacc[jt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kc = 0; kc < KC; kc++) sacc[jt] = mfma16(kf[jt][kc], qf[kc], sacc[jt]);
+    }
+    // V rows -> wave-private LDS (previous unit's transpose reads are complete: LDS ops of a wave are in order)
+#pragma unroll
+    for (int j = 0; j < VJ; j++) {
+      int pc = lane + j * 64;
+      *reinterpret_cast<bf16x8*>(&Vs[(pc / (VD / 8)) * VLD + (pc % (VD / 8)) * 8]) = vr[j];
+    }
+    const int kmax = key_last - key0;  // last usable key offset inside this unit (may be negative)
+    if (key0 < 0 || kmax < UK - 1) {   // wave-uniform: only the unit holding the causal boundary is masked
+#pragma unroll
+      for (int jt = 0; jt < 2; jt++)
 #pragma unroll
         for (int i = 0; i < 4; i++) {
           int ko = jt * 16 + kq * 4 + i;
-          float s = ko <= kmax ? sacc[jt][i] * sc : NSA_NEG_INF;
-          sacc[jt][i] = s;
-          tmax = fmaxf(tmax, s);
+          if (key0 < 0 || ko > kmax) sacc[jt][i] = NSA_NEG_INF;
         }
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-      float m_new = fmaxf(m_run, tmax);  // finite: key0 <= t guarantees at least one visible key
-      float alpha = fast_exp2(m_run - m_new);
-      m_run = m_new;
-      float psum = 0.f;
+    }
+    float tmax = fmaxf(fmaxf(fmaxf(sacc[0][0], sacc[0][1]), fmaxf(sacc[0][2], sacc[0][3])),
+                       fmaxf(fmaxf(sacc[1][0], sacc[1][1]), fmaxf(sacc[1][2], sacc[1][3])));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_old = m_run;
+    const float m_new = fmaxf(m_old, tmax);
+    const float m_safe = (m_new == NSA_NEG_INF) ? 0.f : m_new;
+    const float msc = m_safe * sc;
+    m_run = m_new;
+    float psum = 0.f;
 #pragma unroll
-      for (int jt = 0; jt < 4; jt++)
+    for (int jt = 0; jt < 2; jt++)
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-          float pv = fast_exp2(sacc[jt][i] - m_new);
-          sacc[jt][i] = pv;
-          psum += pv;
-        }
-      l_run = l_run * alpha + psum;
+      for (int i = 0; i < 4; i++) {
+        float pv = fast_exp2(__builtin_fmaf(sacc[jt][i], sc, -msc));
+        sacc[jt][i] = pv;
+        psum += pv;
+      }
+    if (__builtin_amdgcn_ballot_w64(m_new != m_old) != 0) {
+      const float alpha = fast_exp2((m_old - m_safe) * sc);
+      l_run *= alpha;
 #pragma unroll
       for (int dt = 0; dt < VD / 16; dt++) oacc[dt] *= alpha;
+    }
+    l_run += psum;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // O^T += V^T P^T over the 32 keys of the unit
+    bf16x8 pf = pack8(sacc[0][0], sacc[0][1], sacc[0][2], sacc[0][3], sacc[1][0], sacc[1][1], sacc[1][2], sacc[1][3]);
+    const int kb0 = kq * 4 + (l16 >> 2);
+    const int kb1 = kb0 + 16;
+#pragma unroll
+    for (int dt = 0; dt < VD / 16; dt++) {
+      const int col = dt * 16 + 4 * (l16 & 3);
+      bf16x4 v0 = lds_read_tr(&Vs[kb0 * VLD + col]);
+      bf16x4 v1 = lds_read_tr(&Vs[kb1 * VLD + col]);
+      oacc[dt] = mfma16(cat4(v0, v1), pf, oacc[dt]);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  };
 
-      // ---- V registers -> wave-private LDS ----
-#pragma unroll
-      for (int j = 0; j < (VD / 8); j++) {
-        int pc = lane + j * 64;
-        int kr = pc / (VD / 8), dp = pc - kr * (VD / 8);
-        *reinterpret_cast<bf16x8*>(&Vs[kr * VLD + dp * 8]) = vreg[j];
-      }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-
-      // ---- O^T += V^T P^T ----
-#pragma unroll
-      for (int c = 0; c < 2; c++) {
-        bf16x8 pf = pack8(sacc[2 * c][0], sacc[2 * c][1], sacc[2 * c][2], sacc[2 * c][3], sacc[2 * c + 1][0],
-                          sacc[2 * c + 1][1], sacc[2 * c + 1][2], sacc[2 * c + 1][3]);
-        const int kb0 = (2 * c) * 16 + kq * 4 + (l16 >> 2);
-        const int kb1 = kb0 + 16;
-#pragma unroll
-        for (int dt = 0; dt < VD / 16; dt++) {
-          const int col = dt * 16 + 4 * (l16 & 3);
-          bf16x4 v0 = lds_read_tr(&Vs[kb0 * VLD + col]);
-          bf16x4 v1 = lds_read_tr(&Vs[kb1 * VLD + col]);
-          oacc[dt] = mfma16(cat4(v0, v1), pf, oacc[dt]);
-        }
-      }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
+  bf16x8 kfA[2][KC], kfB[2][KC], vrA[VJ], vrB[VJ];
+  int keyA = 0, keyB = 0;
+  if (nu > 0) { keyA = unit_key0(0); issue(keyA, kfA, vrA); }
+  for (int u = 0; u < nu; u += 2) {
+    if (u + 1 < nu) { keyB = unit_key0(u + 1); issue(keyB, kfB, vrB); }
+    compute(keyA, kfA, vrA);
+    if (u + 1 < nu) {
+      if (u + 2 < nu) { keyA = unit_key0(u + 2); issue(keyA, kfA, vrA); }
+      compute(keyB, kfB, vrB);
     }
   }
 
@@ -164,7 +182,7 @@ __global__ __launch_bounds__(256) void slc_fwd_kernel(NsaSlcParams p) {
     *reinterpret_cast<bf16x4*>(op + dt * 16) = w;
   }
   if (kq == 0 && p.lse != nullptr) {
-    p.lse[tok * p.lse_st + (int64_t)head * p.lse_sh] = l_tot > 0.f ? m_run + fast_log2(l_tot) : 0.f;
+    p.lse[tok * p.lse_st + (int64_t)head * p.lse_sh] = l_tot > 0.f ? m_run * sc + fast_log2(l_tot) : 0.f;
   }
 }
 

@@ -30,7 +30,7 @@ struct SlotMap {
 template <int D, int GP, bool PAGED>
 __global__ __launch_bounds__(256) void topk_kernel(NsaTopkParams p) {
   constexpr int KT = 64;
-  constexpr int KLD = D + 8;
+  constexpr int KLD = D + NSA_LDS_PAD;
   constexpr int TPW = 32 / GP;  // tokens per wave
   constexpr int TWG = 4 * TPW;  // tokens per workgroup
   constexpr int PLD = KT + 1;
@@ -249,7 +249,7 @@ template <int D, int GP, bool PAGED>
 int launch_topk(const NsaTopkParams& p, int B, int max_q_len, hipStream_t stream) {
   constexpr int TWG = 4 * (32 / GP);
   size_t dyn = (size_t)TWG * p.nb_max * sizeof(float);
-  size_t stat = 64 * (D + 8) * 2 + 4 * (32 / GP) * 65 * 4;
+  size_t stat = 64 * (D + NSA_LDS_PAD) * 2 + 4 * (32 / GP) * 65 * 4;
   if (dyn + stat > 160 * 1024) {
     nsa_set_error("top-k: %d selection blocks x %d tokens per workgroup do not fit LDS", p.nb_max, TWG);
     return NSA_ERR_UNSUPPORTED;
