@@ -185,6 +185,28 @@ int nsa_paged_pool_decode(void* k_cache, int64_t k_sr, int64_t k_sh, int Dk, voi
                           int table_stride, const int32_t* cmp_slot_mapping, int B, int page_size, int H,
                           int kernel_size, int stride, void* stream);
 
+/* ---- fused decode step (one query token per request; q [B,QH,D], at most 16 q-heads per kv head) ----
+ * Replaces flash_nsa/inference/compress_attn.py:540-667 (cmp_attn_decode) + inference/topk.py:495-623 (topk_decode):
+ * compressed attention (cmp_o [B,QH,VD], optional lse addressed b*lse_st + head*lse_sh) and the top-n selection
+ * topk[kh*tk_sh + b*tk_st + slot]; call after nsa_paged_pool_decode. */
+int nsa_decode_cmp_topk(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr, int64_t k_sh,
+                        const void* v_cache, int64_t v_sr, int64_t v_sh, void* cmp_o, int64_t co_st, int64_t co_sh,
+                        float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk, int64_t tk_sh, int64_t tk_st,
+                        const int32_t* context_lens, const int32_t* cmp_block_tables, int cmp_table_stride,
+                        int page_size, int B, int QH, int KH, int D, int VD, int fixed_y_maxlen,
+                        int fixed_num_slc_blocks, int kernel_size, int stride, int block_size, int top_n,
+                        int num_init, int num_local, int ignore_index, float sm_scale, void* stream);
+/* Replaces flash_nsa/inference/select_attn.py:655-787 (fused_slc_swa_attn_decode) + inference/combine.py:104-127
+ * (combine_decode): selected-block and window attention; slc_o / swa_o (optional, same strides as cmp_o) receive the
+ * branch outputs; out (optional) = cmp_o*sig(w0) + slc_o*sig(w1) + swa_o*sig(w2). */
+int nsa_decode_slc_swa_combine(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr,
+                               int64_t k_sh, const void* v_cache, int64_t v_sr, int64_t v_sh, const void* w,
+                               int64_t w_st, int64_t w_sh, const int32_t* topk, int64_t tk_sh, int64_t tk_st,
+                               const void* cmp_o, void* slc_o, void* swa_o, int64_t co_st, int64_t co_sh, void* out,
+                               int64_t o_st, int64_t o_sh, const int32_t* context_lens, const int32_t* block_tables,
+                               int table_stride, int page_size, int B, int QH, int KH, int D, int VD, int block_size,
+                               int top_n, int window, float sm_scale, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -102,3 +102,25 @@ struct NsaSlcBwdDqParams {
   float scale_log2, sm_scale;
 };
 int nsa_slc_bwd_dq_launch(const NsaSlcBwdDqParams& p, int B, int max_q_len, int D, int VD, hipStream_t stream);
+
+// fused paged decode (one query token per request)
+struct NsaDecodeParams {
+  const bf16_t* q; int64_t q_st, q_sh;          // [B, QH, D]
+  const bf16_t* k; int64_t k_sr, k_sh;          // pool, flat rows
+  const bf16_t* v; int64_t v_sr, v_sh;
+  const bf16_t* w; int64_t w_st, w_sh;          // gates [B, QH, 3]
+  bf16_t* cmp_o; bf16_t* slc_o; bf16_t* swa_o; int64_t co_st, co_sh;  // branch outputs [B, QH, VD] (slc/swa optional)
+  bf16_t* out; int64_t o_st, o_sh;              // final output (optional)
+  float* lse_out; int64_t lse_st, lse_sh;       // compressed-branch lse (optional)
+  int32_t* topk; int64_t tk_sh, tk_st;          // [KH, B, top_n]
+  const int32_t* ctx_lens;
+  const int32_t* table; int table_stride;       // raw block tables
+  const int32_t* cmp_table; int cmp_table_stride;
+  int page_size;
+  int G, KH;
+  float scale_log2;
+  int kernel_size, stride, block_size, window, top_n, num_init, num_local, ignore_index;
+  int y_cap, nb_cap;                            // fixed_y_maxlen, fixed_num_slc_blocks
+};
+int nsa_decode_cmp_topk_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream);
+int nsa_decode_slc_swa_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream);

@@ -1,0 +1,459 @@
+// Paged-KV decode (one query token per request): two fused kernels after the pooling of the newest compressed row.
+//   decode_cmp_topk_kernel      compressed attention (o, lse) + block importance + top-n selection
+//   decode_slc_swa_kernel       selected-block attention + sliding-window attention + gated combine with the
+//                               compressed-branch output -> final o
+// Upstream runs this step as 7 launches (flash_nsa/inference/__init__.py:207-257: cmp_attn_decode stage1/2,
+// topk_decode probs/select, fused_slc_swa_attn_decode stage1/2, combine_decode).
+//
+// One workgroup of 8 waves per (request, kv head); the G <= 16 q-heads of the group are the MFMA N dimension
+// (v_mfma_f32_16x16x32_bf16, S^T = K Q^T so that softmax statistics are per-lane).  The key range is cut in units
+// of 32 keys dealt round-robin to the waves; every wave runs an online softmax over its units with the K
+// fragments and V rows of the next unit in flight (register double buffering), and the partial (m, l, o) of the
+// waves are merged through LDS.  The step is HBM-bound: every K/V row is read once per pass straight from the
+// pool through the block tables.
+#include "nsa_common.h"
+#include "nsa_api_internal.h"
+
+namespace {
+
+constexpr int DEC_WAVES = 8;
+constexpr int UK = 32;  // keys per unit
+
+// One wave's flash-attention state over units of 32 keys for the 16 heads of a kv group.
+template <int D, int VD>
+struct UnitFlash {
+  static constexpr int KC = D / 32;
+  static constexpr int VJ = (UK * (VD / 8)) / 64;
+  static constexpr int VLD = VD + NSA_LDS_PAD;
+  bf16x8 qf[KC];
+  f32x4 oacc[VD / 16];
+  float m_run, l_run;
+  float sc;
+  int l16, kq, lane;
+  bf16_t* Vs;  // wave-private [UK][VLD]
+
+  NSA_DEVICE void init(const bf16_t* qrow, float scale_log2, int lane_, bf16_t* vs) {
+    lane = lane_;
+    l16 = lane & 15;
+    kq = lane >> 4;
+    sc = scale_log2;
+    Vs = vs;
+#pragma unroll
+    for (int kc = 0; kc < KC; kc++) qf[kc] = ld_global_b128(qrow + kq * 8 + kc * 32);
+#pragma unroll
+    for (int dt = 0; dt < VD / 16; dt++) oacc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    m_run = NSA_NEG_INF;
+    l_run = 0.f;
+  }
+  // loads of the unit starting at key0; keys outside [klo, khi] are replaced by a clamped key (masked later)
+  template <class RowFn>
+  NSA_DEVICE void issue(int key0, int klo, int khi, RowFn row_of_key, const bf16_t* kbase, int64_t k_sr,
+                        const bf16_t* vbase, int64_t v_sr, bf16x8 (&kf)[2][KC], bf16x8 (&vr)[VJ]) {
+#pragma unroll
+    for (int jt = 0; jt < 2; jt++) {
+      int key = max(klo, min(key0 + jt * 16 + l16, khi));
+      const bf16_t* kp = kbase + row_of_key(key) * k_sr + kq * 8;
+#pragma unroll
+      for (int kc = 0; kc < KC; kc++) kf[jt][kc] = ld_global_b128(kp + kc * 32);
+    }
+#pragma unroll
+    for (int j = 0; j < VJ; j++) {
+      int pc = lane + j * 64;
+      int kr = pc / (VD / 8), dp = pc % (VD / 8);
+      int key = max(klo, min(key0 + kr, khi));
+      vr[j] = ld_global_b128(vbase + row_of_key(key) * v_sr + dp * 8);
+    }
+  }
+  NSA_DEVICE void compute(int key0, int klo, int khi, bf16x8 (&kf)[2][KC], bf16x8 (&vr)[VJ]) {
+    f32x4 sacc[2];
+#pragma unroll
+    for (int jt = 0; jt < 2; jt++) {
+      sacc[jt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kc = 0; kc < KC; kc++) sacc[jt] = mfma16(kf[jt][kc], qf[kc], sacc[jt]);
+    }
+#pragma unroll
+    for (int j = 0; j < VJ; j++) {
+      int pc = lane + j * 64;
+      *reinterpret_cast<bf16x8*>(&Vs[(pc / (VD / 8)) * VLD + (pc % (VD / 8)) * 8]) = vr[j];
+    }
+    if (key0 < klo || key0 + UK - 1 > khi) {  // wave-uniform: only boundary units are masked
+#pragma unroll
+      for (int jt = 0; jt < 2; jt++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          int key = key0 + jt * 16 + kq * 4 + i;
+          if (key < klo || key > khi) sacc[jt][i] = NSA_NEG_INF;
+        }
+    }
+    float tmax = fmaxf(fmaxf(fmaxf(sacc[0][0], sacc[0][1]), fmaxf(sacc[0][2], sacc[0][3])),
+                       fmaxf(fmaxf(sacc[1][0], sacc[1][1]), fmaxf(sacc[1][2], sacc[1][3])));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_old = m_run;
+    const float m_new = fmaxf(m_old, tmax);
+    const float m_safe = (m_new == NSA_NEG_INF) ? 0.f : m_new;
+    const float msc = m_safe * sc;
+    m_run = m_new;
+    float psum = 0.f;
+#pragma unroll
+    for (int jt = 0; jt < 2; jt++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        float pv = fast_exp2(__builtin_fmaf(sacc[jt][i], sc, -msc));
+        sacc[jt][i] = pv;
+        psum += pv;
+      }
+    if (__builtin_amdgcn_ballot_w64(m_new != m_old) != 0) {
+      const float alpha = fast_exp2((m_old - m_safe) * sc);
+      l_run *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < VD / 16; dt++) oacc[dt] *= alpha;
+    }
+    l_run += psum;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    bf16x8 pf = pack8(sacc[0][0], sacc[0][1], sacc[0][2], sacc[0][3], sacc[1][0], sacc[1][1], sacc[1][2], sacc[1][3]);
+    const int kb0 = kq * 4 + (l16 >> 2);
+    const int kb1 = kb0 + 16;
+#pragma unroll
+    for (int dt = 0; dt < VD / 16; dt++) {
+      const int col = dt * 16 + 4 * (l16 & 3);
+      bf16x4 v0 = lds_read_tr(&Vs[kb0 * VLD + col]);
+      bf16x4 v1 = lds_read_tr(&Vs[kb1 * VLD + col]);
+      oacc[dt] = mfma16(cat4(v0, v1), pf, oacc[dt]);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+  // pipelined loop over units u = first, first+step, ... < nu ; key0_of(u) gives the unit's first key
+  template <class KeyFn, class RowFn>
+  NSA_DEVICE void run(int first, int step, int nu, int klo, int khi, KeyFn key0_of, RowFn row_of_key,
+                      const bf16_t* kbase, int64_t k_sr, const bf16_t* vbase, int64_t v_sr) {
+    bf16x8 kfA[2][KC], kfB[2][KC], vrA[VJ], vrB[VJ];
+    int keyA = 0, keyB = 0;
+    if (first < nu) { keyA = key0_of(first); issue(keyA, klo, khi, row_of_key, kbase, k_sr, vbase, v_sr, kfA, vrA); }
+    for (int u = first; u < nu; u += 2 * step) {
+      const bool hasB = u + step < nu;
+      if (hasB) { keyB = key0_of(u + step); issue(keyB, klo, khi, row_of_key, kbase, k_sr, vbase, v_sr, kfB, vrB); }
+      compute(keyA, klo, khi, kfA, vrA);
+      if (hasB) {
+        if (u + 2 * step < nu) {
+          keyA = key0_of(u + 2 * step);
+          issue(keyA, klo, khi, row_of_key, kbase, k_sr, vbase, v_sr, kfA, vrA);
+        }
+        compute(keyB, klo, khi, kfB, vrB);
+      }
+    }
+  }
+  // wave partial -> LDS slot: m (raw units), l, o[16 heads][VD]
+  NSA_DEVICE void publish(float* pm, float* pl, float* po) {
+    float l_tot = l_run + __shfl_xor(l_run, 16, 64);
+    l_tot += __shfl_xor(l_tot, 32, 64);
+    if (kq == 0) { pm[l16] = m_run; pl[l16] = l_tot; }
+#pragma unroll
+    for (int dt = 0; dt < VD / 16; dt++)
+      *reinterpret_cast<f32x4*>(&po[l16 * VD + dt * 16 + kq * 4]) = oacc[dt];
+  }
+};
+
+// merged value of one (head, channel) from n wave partials; returns o (normalised) and optionally lse2
+NSA_DEVICE float merge_partials(const float* pm, const float* pl, const float* po, int nparts, int part_stride_ml,
+                                int part_stride_o, int head, int d, int VD, float sc, float* lse2_out) {
+  float m = NSA_NEG_INF;
+  for (int w = 0; w < nparts; w++) m = fmaxf(m, pm[w * part_stride_ml + head]);
+  if (m == NSA_NEG_INF) {
+    if (lse2_out) *lse2_out = 0.f;
+    return 0.f;
+  }
+  float l = 0.f, o = 0.f;
+  for (int w = 0; w < nparts; w++) {
+    float mw = pm[w * part_stride_ml + head];
+    float a = (mw == NSA_NEG_INF) ? 0.f : fast_exp2((mw - m) * sc);
+    l += a * pl[w * part_stride_ml + head];
+    o += a * po[w * part_stride_o + head * VD + d];
+  }
+  if (lse2_out) *lse2_out = m * sc + fast_log2(l);
+  return l > 0.f ? o / l : 0.f;
+}
+
+template <int D, int VD>
+__global__ __launch_bounds__(DEC_WAVES * 64) void decode_cmp_topk_kernel(NsaDecodeParams p) {
+  using UF = UnitFlash<D, VD>;
+  constexpr int NW = DEC_WAVES;
+  // dynamic LDS: [V staging, one slot per wave (reused for the wave's partial o)] [m][l][lse] [pg] [imp]
+  extern __shared__ __attribute__((aligned(16))) unsigned char dyn_raw[];
+  constexpr int SLOT = UK * UF::VLD;  // bf16 elements per wave slot (>= 16*VD floats)
+  static_assert(SLOT * 2 >= 16 * VD * 4, "a wave's V slot must hold its partial output");
+  bf16_t* Vs_all = reinterpret_cast<bf16_t*>(dyn_raw);
+  float* part_m = reinterpret_cast<float*>(dyn_raw + (size_t)NW * SLOT * 2);
+  float* part_l = part_m + NW * 16;
+  float* lse_s = part_l + NW * 16;
+  float* pg = lse_s + 16;
+  float* imp = pg + p.y_cap;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int b = blockIdx.x, kh = blockIdx.y;
+  const int G = p.G;
+  const int L = p.ctx_lens[b];
+  const int t = L - 1;
+  const int y = L >= p.kernel_size ? min((L - p.kernel_size) / p.stride + 1, p.y_cap) : 0;
+  const int nb = min(L > 0 ? (L - 1) / p.block_size + 1 : 0, p.nb_cap);
+  const int32_t* ctab = p.cmp_table + (int64_t)b * p.cmp_table_stride;
+  const int page = p.page_size;
+  auto row_of = [&](int key) -> int64_t { return (int64_t)ctab[key / page] * page + (key % page); };
+  const bf16_t* kbase = p.k + (int64_t)kh * p.k_sh;
+  const bf16_t* vbase = p.v + (int64_t)kh * p.v_sh;
+  const int l16 = lane & 15, kq = lane >> 4;
+  const int g = min(l16, G - 1);
+  const int head = kh * G + g;
+
+  UF uf;
+  uf.init(p.q + (int64_t)b * p.q_st + (int64_t)head * p.q_sh, p.scale_log2, lane, Vs_all + wave * UK * UF::VLD);
+  const int nu = (y + UK - 1) / UK;
+
+  // ---- phase A: compressed attention, units dealt round-robin to the waves ----
+  uf.run(wave, NW, nu, 0, y - 1, [&](int u) { return u * UK; }, row_of, kbase, p.k_sr, vbase, p.v_sr);
+  uf.publish(part_m + wave * 16, part_l + wave * 16, reinterpret_cast<float*>(Vs_all + wave * SLOT));
+  for (int i = tid; i < p.y_cap; i += NW * 64) pg[i] = 0.f;
+  __syncthreads();
+  for (int idx = tid; idx < 16 * VD; idx += NW * 64) {
+    int h = idx / VD, d = idx - h * VD;
+    float lse2;
+    float o = merge_partials(part_m, part_l, reinterpret_cast<const float*>(Vs_all), NW, 16, SLOT / 2, h, d, VD,
+                             p.scale_log2, &lse2);
+    if (h < G) {
+      p.cmp_o[(int64_t)b * p.co_st + (int64_t)(kh * G + h) * p.co_sh + d] = (bf16_t)o;
+      if (d == 0) {
+        lse_s[h] = lse2;
+        if (p.lse_out) p.lse_out[(int64_t)b * p.lse_st + (kh * G + h) * p.lse_sh] = lse2;
+      }
+    } else if (d == 0) {
+      lse_s[h] = 0.f;
+    }
+  }
+  __syncthreads();
+
+  // ---- phase B: p = exp2(s*c - lse) summed over the heads of the group, per compressed key ----
+  {
+    // S[head][key] = Q K^T : lane holds key = l16, heads kq*4 .. +3
+    float lse4[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) lse4[i] = lse_s[kq * 4 + i];
+    bf16x8 kf[2][UF::KC];
+    for (int u = wave; u < nu; u += NW) {
+      const int key0 = u * UK;
+#pragma unroll
+      for (int jt = 0; jt < 2; jt++) {
+        int key = min(key0 + jt * 16 + l16, y - 1);
+        const bf16_t* kp = kbase + row_of(key) * p.k_sr + kq * 8;
+#pragma unroll
+        for (int kc = 0; kc < UF::KC; kc++) kf[jt][kc] = ld_global_b128(kp + kc * 32);
+      }
+#pragma unroll
+      for (int jt = 0; jt < 2; jt++) {
+        f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kc = 0; kc < UF::KC; kc++) s = mfma16(uf.qf[kc], kf[jt][kc], s);
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+          if (kq * 4 + i < G) acc += fast_exp2(__builtin_fmaf(s[i], p.scale_log2, -lse4[i]));
+        acc += __shfl_xor(acc, 16, 64);
+        acc += __shfl_xor(acc, 32, 64);
+        int key = key0 + jt * 16 + l16;
+        if (kq == 0 && key < y) pg[key] = acc;
+      }
+    }
+  }
+  __syncthreads();
+  // ---- fold compressed keys into selection-block scores (ascending key order per block) ----
+  {
+    const int Bs = p.block_size, Kz = p.kernel_size, St = p.stride;
+    const int nloops = (Bs + Kz - St) / St;
+    for (int j = tid; j < p.nb_cap; j += NW * 64) {
+      float acc = 0.f;
+      if (j < nb) {
+        int i0 = (j * Bs - Kz) / St + 1;
+        int cs = St - Kz;
+        for (int r = 0; r < nloops; r++, cs += St) {
+          int i = i0 + r;
+          if (i >= 0 && i < y) {
+            int area = min(cs + Kz, Bs) - max(cs, 0);
+            acc += pg[i] * ((float)area / (float)St);
+          }
+        }
+      }
+      imp[j] = acc;
+    }
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  // ---- selection: forced initial and local blocks, then repeated arg-max (lowest index on ties) ----
+  {
+    const int nk = t >= 0 ? t / p.block_size : -1;
+    int result = p.ignore_index;
+    if (lane == 0) {
+      for (int s = 0; s < p.num_init; s++)
+        if (s < p.nb_cap) imp[s] = -1.f;
+      for (int i = 0; i < p.num_local; i++)
+        if (nk - i >= 0 && nk - i < p.nb_cap) imp[nk - i] = -1.f;
+    }
+    if (lane < p.num_init) {
+      if (lane <= nk) result = lane;
+    } else if (lane < p.num_init + p.num_local) {
+      if (lane <= nk) result = nk - (lane - p.num_init);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int nsel = min(p.top_n, nk + 1);
+    const int jmax = min(nk, p.nb_cap - 1);
+    for (int slot = p.num_init + p.num_local; slot < nsel; slot++) {
+      float best = -2.f;
+      int bj = 0x7fffffff;
+      for (int j = lane; j <= jmax; j += 64) {
+        float v = imp[j];
+        if (v > best) { best = v; bj = j; }
+      }
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {
+        float ob = __shfl_xor(best, o, 64);
+        int oj = __shfl_xor(bj, o, 64);
+        if (ob > best || (ob == best && oj < bj)) { best = ob; bj = oj; }
+      }
+      if (lane == slot) result = bj;
+      if (lane == 0 && bj <= jmax) imp[bj] = -1.f;
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    if (lane < p.top_n) p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + lane] = result;
+  }
+}
+
+template <int D, int VD>
+__global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecodeParams p) {
+  using UF = UnitFlash<D, VD>;
+  constexpr int NW = DEC_WAVES;
+  constexpr int NW_SLC = 5;  // waves on the selected blocks, the rest on the window
+  extern __shared__ __attribute__((aligned(16))) unsigned char dyn_raw[];
+  constexpr int SLOT = UK * UF::VLD;
+  static_assert(SLOT * 2 >= 16 * VD * 4, "a wave's V slot must hold its partial output");
+  bf16_t* Vs_all = reinterpret_cast<bf16_t*>(dyn_raw);
+  float* part_m = reinterpret_cast<float*>(dyn_raw + (size_t)NW * SLOT * 2);
+  float* part_l = part_m + NW * 16;
+  int* blk_s = reinterpret_cast<int*>(part_l + NW * 16);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int b = blockIdx.x, kh = blockIdx.y;
+  const int G = p.G;
+  const int L = p.ctx_lens[b];
+  const int t = L - 1;
+  const int32_t* tab = p.table + (int64_t)b * p.table_stride;
+  const int page = p.page_size;
+  auto row_of = [&](int key) -> int64_t { return (int64_t)tab[key / page] * page + (key % page); };
+  const bf16_t* kbase = p.k + (int64_t)kh * p.k_sh;
+  const bf16_t* vbase = p.v + (int64_t)kh * p.v_sh;
+  const int l16 = lane & 15;
+  const int g = min(l16, G - 1);
+  const int head = kh * G + g;
+  const int Bs = p.block_size;
+  const int nvalid = t >= 0 ? min(p.top_n, t / Bs + 1) : 0;
+  if (tid < 64) blk_s[tid] = tid < nvalid ? p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + tid] : 0;
+  __syncthreads();
+
+  UF uf;
+  uf.init(p.q + (int64_t)b * p.q_st + (int64_t)head * p.q_sh, p.scale_log2, lane, Vs_all + wave * UK * UF::VLD);
+  if (t >= 0) {
+    if (wave < NW_SLC) {
+      const int upb = Bs / UK;
+      uf.run(wave, NW_SLC, nvalid * upb, 0, t,
+             [&](int u) { int slot = u / upb; return max(blk_s[slot], 0) * Bs + (u - slot * upb) * UK; }, row_of,
+             kbase, p.k_sr, vbase, p.v_sr);
+    } else {
+      const int klo = max(0, t - p.window);
+      const int k0 = (klo / UK) * UK;
+      const int nu = (t - k0) / UK + 1;
+      uf.run(wave - NW_SLC, NW - NW_SLC, nu, klo, t, [&](int u) { return k0 + u * UK; }, row_of, kbase, p.k_sr,
+             vbase, p.v_sr);
+    }
+  }
+  uf.publish(part_m + wave * 16, part_l + wave * 16, reinterpret_cast<float*>(Vs_all + wave * SLOT));
+  __syncthreads();
+  const float* part_o = reinterpret_cast<const float*>(Vs_all);
+  for (int idx = tid; idx < 16 * VD; idx += NW * 64) {
+    int h = idx / VD, d = idx - h * VD;
+    if (h >= G) continue;
+    const int hq = kh * G + h;
+    float o_slc = merge_partials(part_m, part_l, part_o, NW_SLC, 16, SLOT / 2, h, d, VD, p.scale_log2, nullptr);
+    float o_swa = merge_partials(part_m + NW_SLC * 16, part_l + NW_SLC * 16, part_o + NW_SLC * (SLOT / 2),
+                                 NW - NW_SLC, 16, SLOT / 2, h, d, VD, p.scale_log2, nullptr);
+    // branch outputs are rounded to bf16 before the gated sum, as the three-kernel path stores them
+    o_slc = (float)(bf16_t)o_slc;
+    o_swa = (float)(bf16_t)o_swa;
+    if (p.slc_o) p.slc_o[(int64_t)b * p.co_st + (int64_t)hq * p.co_sh + d] = (bf16_t)o_slc;
+    if (p.swa_o) p.swa_o[(int64_t)b * p.co_st + (int64_t)hq * p.co_sh + d] = (bf16_t)o_swa;
+    if (p.out) {
+      const bf16_t* wp = p.w + (int64_t)b * p.w_st + (int64_t)hq * p.w_sh;
+      float s0 = 1.f / (1.f + __expf(-(float)wp[0]));
+      float s1 = 1.f / (1.f + __expf(-(float)wp[1]));
+      float s2 = 1.f / (1.f + __expf(-(float)wp[2]));
+      float o_cmp = (float)p.cmp_o[(int64_t)b * p.co_st + (int64_t)hq * p.co_sh + d];
+      p.out[(int64_t)b * p.o_st + (int64_t)hq * p.o_sh + d] = (bf16_t)(o_cmp * s0 + o_slc * s1 + o_swa * s2);
+    }
+  }
+}
+
+}  // namespace
+
+template <class K>
+static int launch_dyn(K kern, dim3 grid, size_t dyn, const NsaDecodeParams& p, hipStream_t stream, const char* name) {
+  if (dyn > 160 * 1024) {
+    nsa_set_error("%s: %zu bytes of LDS needed (fixed_y_maxlen / fixed_num_slc_blocks too large)", name, dyn);
+    return NSA_ERR_UNSUPPORTED;
+  }
+  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn);
+  if (e != hipSuccess) {
+    nsa_set_error("%s: hipFuncSetAttribute(%zu) failed: %s", name, dyn, hipGetErrorString(e));
+    return NSA_ERR_LAUNCH;
+  }
+  kern<<<grid, DEC_WAVES * 64, dyn, stream>>>(p);
+  return nsa_check_launch(name);
+}
+
+template <int D, int VD>
+static size_t slot_bytes() { return (size_t)DEC_WAVES * UK * (VD + NSA_LDS_PAD) * 2; }
+
+int nsa_decode_cmp_topk_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream) {
+  if (B <= 0) return NSA_OK;
+  dim3 grid(B, p.KH);
+  size_t extra = (size_t)(2 * DEC_WAVES * 16 + 16 + p.y_cap + p.nb_cap) * sizeof(float);
+  if (D == 128 && VD == 128)
+    return launch_dyn(decode_cmp_topk_kernel<128, 128>, grid, slot_bytes<128, 128>() + extra, p, stream,
+                      "decode_cmp_topk_kernel");
+  if (D == 64 && VD == 64)
+    return launch_dyn(decode_cmp_topk_kernel<64, 64>, grid, slot_bytes<64, 64>() + extra, p, stream,
+                      "decode_cmp_topk_kernel");
+  nsa_set_error("decode: unsupported head dims D=%d VD=%d (built: 128/128, 64/64)", D, VD);
+  return NSA_ERR_UNSUPPORTED;
+}
+
+int nsa_decode_slc_swa_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream) {
+  if (B <= 0) return NSA_OK;
+  dim3 grid(B, p.KH);
+  size_t extra = (size_t)(2 * DEC_WAVES * 16 + 64) * sizeof(float);
+  if (D == 128 && VD == 128)
+    return launch_dyn(decode_slc_swa_kernel<128, 128>, grid, slot_bytes<128, 128>() + extra, p, stream,
+                      "decode_slc_swa_kernel");
+  if (D == 64 && VD == 64)
+    return launch_dyn(decode_slc_swa_kernel<64, 64>, grid, slot_bytes<64, 64>() + extra, p, stream,
+                      "decode_slc_swa_kernel");
+  nsa_set_error("decode: unsupported head dims D=%d VD=%d (built: 128/128, 64/64)", D, VD);
+  return NSA_ERR_UNSUPPORTED;
+}

@@ -5,7 +5,8 @@ them; they write the newly completed compressed rows into the same pool (mean po
 never synchronise with the host, so the decode step can be captured in a HIP graph."""
 from .stages import (mean_pooling_prefill, kv_mean_pooling_decode, cmp_attn_prefill, cmp_attn_decode, topk_prefill,
                      topk_decode, slc_attn_prefill, fused_slc_swa_attn_decode, swa_prefill, combine_prefill,
-                     combine_decode, mean_pooling_decode, slc_attn_decode)
+                     combine_decode, mean_pooling_decode, slc_attn_decode, fused_decode_supported, decode_cmp_topk,
+                     decode_slc_swa_combine)
 
 
 def nsa_prefill(q, k, v, w, x_cu_seqlens, y_cu_seqlens, x_maxlen, y_maxlen, context_lens, block_tables,
@@ -49,6 +50,26 @@ def nsa_decode(q, k, v, w, context_lens, block_tables, cmp_slot_mapping, cmp_blo
         sm_scale = q.size(-1) ** -0.5
     kv_mean_pooling_decode(k, v, block_table=block_tables, slot_mapping=cmp_slot_mapping, context_lens=context_lens,
                            kernel_size=kernel_size, stride=stride)
+    if fused_decode_supported(q, k, v):
+        # two fused launches: (compressed attention + importance + selection), (selected + window + combine)
+        cmp_o, topk = decode_cmp_topk(q, k, v, cmp_block_tables, context_lens, fixed_y_maxlen=fixed_y_maxlen,
+                                      fixed_num_slc_blocks=fixed_num_slc_blocks, kernel_size=kernel_size,
+                                      stride=stride, block_size=block_size, top_n=top_n, num_inital=num_init_blocks,
+                                      num_local=num_local_blocks, sm_scale=sm_scale)
+        return decode_slc_swa_combine(q, k, v, w, topk, cmp_o, block_tables, context_lens, block_size=block_size,
+                                      top_n=top_n, window_size=window_size, sm_scale=sm_scale)
+    return nsa_decode_staged(q, k, v, w, context_lens, block_tables, cmp_block_tables, cmp_num_splits, slc_num_splits,
+                             fixed_y_maxlen, fixed_num_slc_blocks, kernel_size, stride, block_size, top_n,
+                             num_init_blocks, num_local_blocks, window_size, sm_scale)
+
+
+def nsa_decode_staged(q, k, v, w, context_lens, block_tables, cmp_block_tables, cmp_num_splits=0, slc_num_splits=0,
+                      fixed_y_maxlen=8192, fixed_num_slc_blocks=2048, kernel_size=32, stride=16, block_size=64,
+                      top_n=16, num_init_blocks=1, num_local_blocks=2, window_size=512, sm_scale=None):
+    """The decode step stage by stage (after pooling), through the stage functions that mirror upstream's; used when
+    a kv head has more than 16 q-heads, and by the tests as a second implementation of the fused path."""
+    if sm_scale is None:
+        sm_scale = q.size(-1) ** -0.5
     cmp_o, lse = cmp_attn_decode(q, k, v, block_tables=cmp_block_tables, context_lens=context_lens,
                                  num_splits=cmp_num_splits, kernel_size=kernel_size, stride=stride,
                                  sm_scale=sm_scale)

@@ -177,3 +177,57 @@ def combine_prefill(a, b, c, w):
 
 def combine_decode(a, b, c, w):
     return combine_fwd(a, b, c, w)
+
+
+# ------------------------------------------------------------------------------------------------ fused decode
+def fused_decode_supported(q, k, v):
+    QH, KH = q.size(1), k.size(2)
+    return QH // KH <= 16 and (q.size(-1), v.size(-1)) in ((128, 128), (64, 64))
+
+
+def decode_cmp_topk(q, k, v, cmp_block_tables, context_lens, fixed_y_maxlen=8192, fixed_num_slc_blocks=2048,
+                    kernel_size=32, stride=16, block_size=64, top_n=16, num_inital=1, num_local=2, sm_scale=None,
+                    return_lse=False):
+    """One launch: compressed attention + block importance + top-n selection for one token per request.
+    -> (cmp_o [B,QH,VD], topk [KH,B,top_n] int32[, lse [B,QH]])"""
+    check_bf16(q)
+    page, KH, D, ksr, ksh = _pool_args(k)
+    _, _, VD, vsr, vsh = _pool_args(v)
+    B, QH, _ = q.shape
+    sm_scale = q.size(-1) ** -0.5 if sm_scale is None else sm_scale
+    cmp_o = torch.empty(B, QH, VD, device=q.device, dtype=q.dtype)
+    topk = torch.empty(KH, B, top_n, device=q.device, dtype=torch.int32)
+    lse = torch.empty(B, QH, device=q.device, dtype=torch.float32) if return_lse else None
+    _lib.call("nsa_decode_cmp_topk", q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), ksr, ksh, v.data_ptr(),
+              vsr, vsh, cmp_o.data_ptr(), cmp_o.stride(0), cmp_o.stride(1), _lib.ptr(lse),
+              lse.stride(0) if return_lse else 0, lse.stride(1) if return_lse else 0, topk.data_ptr(),
+              topk.stride(0), topk.stride(1), _i32(context_lens).data_ptr(), _i32(cmp_block_tables).data_ptr(),
+              cmp_block_tables.stride(0), page, B, QH, KH, D, VD, int(fixed_y_maxlen), int(fixed_num_slc_blocks),
+              kernel_size, stride, block_size, top_n, num_inital, num_local, -1, sm_scale, _lib.stream_ptr())
+    if return_lse:
+        return cmp_o, topk, lse
+    return cmp_o, topk
+
+
+def decode_slc_swa_combine(q, k, v, w, topk, cmp_o, block_tables, context_lens, block_size=64, top_n=16,
+                           window_size=512, sm_scale=None, return_branches=False):
+    """One launch: selected-block + window attention and the gated combine -> o [B,QH,VD]
+    (with return_branches also slc_o, swa_o)."""
+    check_bf16(q)
+    page, KH, D, ksr, ksh = _pool_args(k)
+    _, _, VD, vsr, vsh = _pool_args(v)
+    B, QH, _ = q.shape
+    sm_scale = q.size(-1) ** -0.5 if sm_scale is None else sm_scale
+    out = torch.empty(B, QH, VD, device=q.device, dtype=q.dtype)
+    slc_o = torch.empty_like(out) if return_branches else None
+    swa_o = torch.empty_like(out) if return_branches else None
+    assert cmp_o.stride() == out.stride()
+    _lib.call("nsa_decode_slc_swa_combine", q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), ksr, ksh,
+              v.data_ptr(), vsr, vsh, w.data_ptr(), w.stride(0), w.stride(1), topk.data_ptr(), topk.stride(0),
+              topk.stride(1), cmp_o.data_ptr(), _lib.ptr(slc_o), _lib.ptr(swa_o), cmp_o.stride(0), cmp_o.stride(1),
+              out.data_ptr(), out.stride(0), out.stride(1), _i32(context_lens).data_ptr(),
+              _i32(block_tables).data_ptr(), block_tables.stride(0), page, B, QH, KH, D, VD, block_size, top_n,
+              window_size, sm_scale, _lib.stream_ptr())
+    if return_branches:
+        return out, slc_o, swa_o
+    return out

@@ -181,3 +181,38 @@ def test_decode_graph_replay_equals_eager(device):
     graph.replay()
     torch.cuda.synchronize()
     assert torch.equal(out, eager2)
+
+
+@pytest.mark.parametrize("QH,KH,D", [(64, 4, 128), (16, 1, 128), (12, 2, 64)])
+def test_fused_decode_matches_staged_decode(device, QH, KH, D):
+    """The two-launch fused decode against the stage-by-stage path (a second, independent set of kernels):
+    same block selection, branch outputs and final output."""
+    from flash_nsa.inference import (nsa_decode_staged, decode_cmp_topk, decode_slc_swa_combine, cmp_attn_decode,
+                                     topk_decode, fused_slc_swa_attn_decode)
+    ctx = [4096, 333, 48, 31, 1, 777, 2999, 640, 1024, 65]
+    case = build_pool(ctx, KH, D, D, page=128, seed=21)
+    prepool(case, ctx)
+    B = len(ctx)
+    d = to_dev(case, device)
+    q = randn_bf16(B, QH, D, seed=22).to(device)
+    w = randn_bf16(B, QH, 3, seed=23).to(device)
+    ctx_t = torch.tensor(ctx, dtype=torch.int32, device=device)
+    kw = dict(top_n=8, window_size=200)
+    cmp_o, topk, lse = decode_cmp_topk(q, d["k"], d["v"], d["cbt"], ctx_t, 512, 64, top_n=8, return_lse=True)
+    out, slc_o, swa_o = decode_slc_swa_combine(q, d["k"], d["v"], w, topk, cmp_o, d["bt"], ctx_t, return_branches=True,
+                                               **kw)
+    r_cmp, r_lse = cmp_attn_decode(q, d["k"], d["v"], d["cbt"], ctx_t)
+    r_topk = topk_decode(q, d["k"], r_lse, d["cbt"], ctx_t, 512, 64, top_n=8)
+    r_slc, r_swa = fused_slc_swa_attn_decode(q, d["k"], d["v"], topk, d["bt"], ctx_t, **kw)
+    assert_close(cmp_o, r_cmp, "cmp_o", atol=4e-3, rtol=1e-2)
+    assert_close(lse, r_lse, "cmp lse", atol=1e-3, rtol=1e-4)
+    nv = torch.clamp((ctx_t - 1) // 64 + 1, max=8).cpu()
+    a, r = topk.cpu(), r_topk.cpu()
+    for b in range(B):
+        for kh in range(KH):
+            assert sorted(a[kh, b, :nv[b]].tolist()) == sorted(r[kh, b, :nv[b]].tolist()), (b, kh)
+    assert_close(slc_o, r_slc, "slc_o", atol=4e-3, rtol=1e-2)
+    assert_close(swa_o, r_swa, "swa_o", atol=4e-3, rtol=1e-2)
+    ref = nsa_decode_staged(q, d["k"], d["v"], w, ctx_t, d["bt"], d["cbt"], fixed_y_maxlen=512,
+                            fixed_num_slc_blocks=64, **kw)
+    assert_close(out, ref, "decode o", atol=8e-3, rtol=1e-2)
