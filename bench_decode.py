@@ -2,9 +2,9 @@
 
 Workload (BASELINE.json configs[4]): batch 64, context lengths uniform in [4096, 32768] from seed 3, page size 256,
 block tables = slices of a random permutation of the pool, 64 q / 4 kv heads, d=128, bf16 N(0,1), top-16 of
-64-token blocks + window 512.  Algorithmic bytes per request of length L: compressed K and V rows once
-(y*KH*(D+VD)*2), compressed K again for the importance pass (y*KH*D*2), 16 selected blocks, the 513 window rows,
-q + w + o.
+64-token blocks + window 512.  Algorithmic bytes per request of length L: compressed K and V rows once (y*KH*(D+VD)*2; the second read of the
+compressed K for the importance pass is an implementation choice and is not counted), 16 selected blocks, the
+513 window rows, q + w + o.
 """
 import torch
 
@@ -48,7 +48,7 @@ def algorithmic_bytes(lens, KH=4, D=128, VD=128, QH=64, top_n=16, block=64, wind
     tot = 0
     for L in lens:
         y = max((L - 32) // 16 + 1, 0)
-        tot += y * KH * (D + VD) * 2 + y * KH * D * 2
+        tot += y * KH * (D + VD) * 2
         tot += min(top_n, (L - 1) // block + 1) * block * KH * (D + VD) * 2
         tot += min(L, window + 1) * KH * (D + VD) * 2
         tot += QH * D * 2 + QH * 3 * 2 + QH * VD * 2

@@ -196,14 +196,28 @@ int nsa_decode_cmp_topk(const void* q, int64_t q_st, int64_t q_sh, const void* k
                         int page_size, int B, int QH, int KH, int D, int VD, int fixed_y_maxlen,
                         int fixed_num_slc_blocks, int kernel_size, int stride, int block_size, int top_n,
                         int num_init, int num_local, int ignore_index, float sm_scale, void* stream);
+/* Split variant of the compressed branch for batches whose context lengths differ widely (two launches, grid
+ * B x KH x nsplit): partial attention per key-interleaved split, then merge (cmp_o, lse) + head-summed probabilities
+ * pg [B,KH,fixed_y_maxlen] fp32 of every compressed key.  Scratch (fp32): sp_m, sp_l [B,KH,nsplit,16],
+ * sp_o [B,KH,nsplit,16,VD].  The selection itself then runs in the prologue of nsa_decode_slc_swa_combine. */
+int nsa_decode_cmp_split(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr, int64_t k_sh,
+                         const void* v_cache, int64_t v_sr, int64_t v_sh, void* cmp_o, int64_t co_st, int64_t co_sh,
+                         float* lse, int64_t lse_st, int64_t lse_sh, float* pg, float* sp_m, float* sp_l, float* sp_o,
+                         int nsplit, const int32_t* context_lens, const int32_t* cmp_block_tables,
+                         int cmp_table_stride, int page_size, int B, int QH, int KH, int D, int VD,
+                         int fixed_y_maxlen, int kernel_size, int stride, float sm_scale, void* stream);
 /* Replaces flash_nsa/inference/select_attn.py:655-787 (fused_slc_swa_attn_decode) + inference/combine.py:104-127
  * (combine_decode): selected-block and window attention; slc_o / swa_o (optional, same strides as cmp_o) receive the
- * branch outputs; out (optional) = cmp_o*sig(w0) + slc_o*sig(w1) + swa_o*sig(w2). */
+ * branch outputs; out (optional) = cmp_o*sig(w0) + slc_o*sig(w1) + swa_o*sig(w2).
+ * pg == NULL: topk is an input.  pg != NULL (from nsa_decode_cmp_split): the block scores are folded from pg and
+ * the selection (inference/topk.py:433-493) runs in the kernel's prologue; topk is then an output. */
 int nsa_decode_slc_swa_combine(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr,
                                int64_t k_sh, const void* v_cache, int64_t v_sr, int64_t v_sh, const void* w,
-                               int64_t w_st, int64_t w_sh, const int32_t* topk, int64_t tk_sh, int64_t tk_st,
-                               const void* cmp_o, void* slc_o, void* swa_o, int64_t co_st, int64_t co_sh, void* out,
-                               int64_t o_st, int64_t o_sh, const int32_t* context_lens, const int32_t* block_tables,
+                               int64_t w_st, int64_t w_sh, int32_t* topk, int64_t tk_sh, int64_t tk_st,
+                               const float* pg, int fixed_y_maxlen, int fixed_num_slc_blocks, int kernel_size,
+                               int stride, int num_init, int num_local, int ignore_index, const void* cmp_o,
+                               void* slc_o, void* swa_o, int64_t co_st, int64_t co_sh, void* out, int64_t o_st,
+                               int64_t o_sh, const int32_t* context_lens, const int32_t* block_tables,
                                int table_stride, int page_size, int B, int QH, int KH, int D, int VD, int block_size,
                                int top_n, int window, float sm_scale, void* stream);
 

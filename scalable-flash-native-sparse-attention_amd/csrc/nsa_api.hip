@@ -468,11 +468,45 @@ int nsa_decode_cmp_topk(const void* q, int64_t q_st, int64_t q_sh, const void* k
   return nsa_decode_cmp_topk_launch(p, B, D, VD, (hipStream_t)stream);
 }
 
+int nsa_decode_cmp_split(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr, int64_t k_sh,
+                         const void* v_cache, int64_t v_sr, int64_t v_sh, void* cmp_o, int64_t co_st, int64_t co_sh,
+                         float* lse, int64_t lse_st, int64_t lse_sh, float* pg, float* sp_m, float* sp_l, float* sp_o,
+                         int nsplit, const int32_t* context_lens, const int32_t* cmp_block_tables,
+                         int cmp_table_stride, int page_size, int B, int QH, int KH, int D, int VD,
+                         int fixed_y_maxlen, int kernel_size, int stride, float sm_scale, void* stream) {
+  int rc = check_heads("decode_cmp_split", QH, KH, D, VD);
+  if (rc) return rc;
+  rc = check_nsa_sizes("decode_cmp_split", kernel_size, stride, 0);
+  if (rc) return rc;
+  rc = check_page("decode_cmp_split", page_size);
+  if (rc) return rc;
+  NSA_REQUIRE(QH / KH <= 16, NSA_ERR_UNSUPPORTED, "decode_cmp_split: at most 16 q-heads per kv head (got %d)", QH / KH);
+  NSA_REQUIRE(nsplit >= 1 && nsplit <= 64, NSA_ERR_BAD_ARG, "decode_cmp_split: nsplit %d must be in [1,64]", nsplit);
+  NSA_REQUIRE(fixed_y_maxlen >= 1 && fixed_y_maxlen <= 32768, NSA_ERR_BAD_ARG,
+              "decode_cmp_split: fixed_y_maxlen %d must be in [1,32768]", fixed_y_maxlen);
+  NsaDecodeParams p{};
+  p.q = (const bf16_t*)q; p.q_st = q_st; p.q_sh = q_sh;
+  p.k = (const bf16_t*)k_cache; p.k_sr = k_sr; p.k_sh = k_sh;
+  p.v = (const bf16_t*)v_cache; p.v_sr = v_sr; p.v_sh = v_sh;
+  p.cmp_o = (bf16_t*)cmp_o; p.co_st = co_st; p.co_sh = co_sh;
+  p.lse_out = lse; p.lse_st = lse_st; p.lse_sh = lse_sh;
+  p.pg = pg; p.sp_m = sp_m; p.sp_l = sp_l; p.sp_o = sp_o;
+  p.ctx_lens = context_lens;
+  p.cmp_table = cmp_block_tables; p.cmp_table_stride = cmp_table_stride; p.page_size = page_size;
+  p.G = QH / KH; p.KH = KH;
+  p.scale_log2 = sm_scale * NSA_LOG2E;
+  p.kernel_size = kernel_size; p.stride = stride;
+  p.y_cap = fixed_y_maxlen;
+  return nsa_decode_cmp_split_launch(p, B, nsplit, D, VD, (hipStream_t)stream);
+}
+
 int nsa_decode_slc_swa_combine(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr,
                                int64_t k_sh, const void* v_cache, int64_t v_sr, int64_t v_sh, const void* w,
-                               int64_t w_st, int64_t w_sh, const int32_t* topk, int64_t tk_sh, int64_t tk_st,
-                               const void* cmp_o, void* slc_o, void* swa_o, int64_t co_st, int64_t co_sh, void* out,
-                               int64_t o_st, int64_t o_sh, const int32_t* context_lens, const int32_t* block_tables,
+                               int64_t w_st, int64_t w_sh, int32_t* topk, int64_t tk_sh, int64_t tk_st,
+                               const float* pg, int fixed_y_maxlen, int fixed_num_slc_blocks, int kernel_size,
+                               int stride, int num_init, int num_local, int ignore_index, const void* cmp_o,
+                               void* slc_o, void* swa_o, int64_t co_st, int64_t co_sh, void* out, int64_t o_st,
+                               int64_t o_sh, const int32_t* context_lens, const int32_t* block_tables,
                                int table_stride, int page_size, int B, int QH, int KH, int D, int VD, int block_size,
                                int top_n, int window, float sm_scale, void* stream) {
   int rc = check_heads("decode_slc_swa_combine", QH, KH, D, VD);
@@ -486,12 +520,24 @@ int nsa_decode_slc_swa_combine(const void* q, int64_t q_st, int64_t q_sh, const 
   NSA_REQUIRE(top_n >= 1 && top_n <= 64, NSA_ERR_BAD_ARG, "decode_slc_swa_combine: top_n %d must be in [1,64]", top_n);
   NSA_REQUIRE(out == nullptr || (w != nullptr && cmp_o != nullptr), NSA_ERR_BAD_ARG,
               "decode_slc_swa_combine: the combined output needs the gates and the compressed-branch output");
+  if (pg != nullptr) {
+    rc = check_nsa_sizes("decode_slc_swa_combine", kernel_size, stride, block_size);
+    if (rc) return rc;
+    NSA_REQUIRE(num_init >= 0 && num_local >= 0 && num_init + num_local <= top_n, NSA_ERR_BAD_ARG,
+                "decode_slc_swa_combine: num_init %d + num_local %d must be <= top_n %d", num_init, num_local, top_n);
+    NSA_REQUIRE(fixed_num_slc_blocks >= 1 && fixed_num_slc_blocks <= 8192 && fixed_y_maxlen >= 1, NSA_ERR_BAD_ARG,
+                "decode_slc_swa_combine: fixed_num_slc_blocks %d must be in [1,8192]", fixed_num_slc_blocks);
+  }
   NsaDecodeParams p{};
   p.q = (const bf16_t*)q; p.q_st = q_st; p.q_sh = q_sh;
   p.k = (const bf16_t*)k_cache; p.k_sr = k_sr; p.k_sh = k_sh;
   p.v = (const bf16_t*)v_cache; p.v_sr = v_sr; p.v_sh = v_sh;
   p.w = (const bf16_t*)w; p.w_st = w_st; p.w_sh = w_sh;
-  p.topk = const_cast<int32_t*>(topk); p.tk_sh = tk_sh; p.tk_st = tk_st;
+  p.topk = topk; p.tk_sh = tk_sh; p.tk_st = tk_st;
+  p.pg = const_cast<float*>(pg);
+  p.y_cap = fixed_y_maxlen; p.nb_cap = fixed_num_slc_blocks;
+  p.kernel_size = kernel_size; p.stride = stride;
+  p.num_init = num_init; p.num_local = num_local; p.ignore_index = ignore_index;
   p.cmp_o = (bf16_t*)const_cast<void*>(cmp_o); p.slc_o = (bf16_t*)slc_o; p.swa_o = (bf16_t*)swa_o;
   p.co_st = co_st; p.co_sh = co_sh;
   p.out = (bf16_t*)out; p.o_st = o_st; p.o_sh = o_sh;

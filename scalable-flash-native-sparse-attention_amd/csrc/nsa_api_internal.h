@@ -121,6 +121,9 @@ struct NsaDecodeParams {
   float scale_log2;
   int kernel_size, stride, block_size, window, top_n, num_init, num_local, ignore_index;
   int y_cap, nb_cap;                            // fixed_y_maxlen, fixed_num_slc_blocks
+  // split compressed branch: fp32 scratch [B,KH,nsplit,16] (m, l), [B,KH,nsplit,16,VD] (o), pg [B,KH,y_cap]
+  float* sp_m; float* sp_l; float* sp_o; float* pg;
 };
 int nsa_decode_cmp_topk_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream);
 int nsa_decode_slc_swa_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream);
+int nsa_decode_cmp_split_launch(const NsaDecodeParams& p, int B, int nsplit, int D, int VD, hipStream_t stream);

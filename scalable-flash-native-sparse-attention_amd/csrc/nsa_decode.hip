@@ -192,6 +192,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_cmp_topk_kernel(NsaDeco
   float* lse_s = part_l + NW * 16;
   float* pg = lse_s + 16;
   float* imp = pg + p.y_cap;
+  int* tab_s = reinterpret_cast<int*>(imp + p.nb_cap);  // the request's compressed-row page table
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -204,7 +205,11 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_cmp_topk_kernel(NsaDeco
   const int nb = min(L > 0 ? (L - 1) / p.block_size + 1 : 0, p.nb_cap);
   const int32_t* ctab = p.cmp_table + (int64_t)b * p.cmp_table_stride;
   const int page = p.page_size;
-  auto row_of = [&](int key) -> int64_t { return (int64_t)ctab[key / page] * page + (key % page); };
+  // page-table entries go to LDS first: a table lookup in global memory in front of every gather would serialise
+  // the pipelined K/V loads behind it (memory operations of a wave retire in order)
+  for (int i = tid; i < (y + page - 1) / page; i += NW * 64) tab_s[i] = ctab[i];
+  __syncthreads();
+  auto row_of = [&](int key) -> int64_t { return (int64_t)tab_s[key / page] * page + (key % page); };
   const bf16_t* kbase = p.k + (int64_t)kh * p.k_sh;
   const bf16_t* vbase = p.v + (int64_t)kh * p.v_sh;
   const int l16 = lane & 15, kq = lane >> 4;
@@ -335,6 +340,175 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_cmp_topk_kernel(NsaDeco
   }
 }
 
+// ---- split variant of the compressed branch: requests are cut in NSPLIT key-interleaved parts so that long
+// contexts do not leave most CUs idle; partial (m, l, o) go through a small fp32 scratch in global memory.
+constexpr int SPLIT_WAVES = 4;
+
+// grid (B, KH, nsplit): compressed attention over the units u = s*4 + wave (mod 4*nsplit)
+template <int D, int VD>
+__global__ __launch_bounds__(SPLIT_WAVES * 64) void decode_cmp_partial_kernel(NsaDecodeParams p) {
+  using UF = UnitFlash<D, VD>;
+  constexpr int NW = SPLIT_WAVES;
+  constexpr int SLOT = UK * UF::VLD;
+  extern __shared__ __attribute__((aligned(16))) unsigned char dyn_raw[];
+  bf16_t* Vs_all = reinterpret_cast<bf16_t*>(dyn_raw);
+  float* part_m = reinterpret_cast<float*>(dyn_raw + (size_t)NW * SLOT * 2);
+  float* part_l = part_m + NW * 16;
+  int* tab_s = reinterpret_cast<int*>(part_l + NW * 16);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int b = blockIdx.x, kh = blockIdx.y, sp = blockIdx.z;
+  const int nsplit = gridDim.z;
+  const int G = p.G;
+  const int L = p.ctx_lens[b];
+  const int y = L >= p.kernel_size ? min((L - p.kernel_size) / p.stride + 1, p.y_cap) : 0;
+  const int32_t* ctab = p.cmp_table + (int64_t)b * p.cmp_table_stride;
+  const int page = p.page_size;
+  for (int i = tid; i < (y + page - 1) / page; i += NW * 64) tab_s[i] = ctab[i];
+  __syncthreads();
+  auto row_of = [&](int key) -> int64_t { return (int64_t)tab_s[key / page] * page + (key % page); };
+  const bf16_t* kbase = p.k + (int64_t)kh * p.k_sh;
+  const bf16_t* vbase = p.v + (int64_t)kh * p.v_sh;
+  const int l16 = lane & 15;
+  const int head = kh * G + min(l16, G - 1);
+
+  UF uf;
+  uf.init(p.q + (int64_t)b * p.q_st + (int64_t)head * p.q_sh, p.scale_log2, lane, Vs_all + wave * SLOT);
+  const int nu = (y + UK - 1) / UK;
+  uf.run(sp * NW + wave, NW * nsplit, nu, 0, y - 1, [&](int u) { return u * UK; }, row_of, kbase, p.k_sr, vbase,
+         p.v_sr);
+  uf.publish(part_m + wave * 16, part_l + wave * 16, reinterpret_cast<float*>(Vs_all + wave * SLOT));
+  __syncthreads();
+  // merge the 4 waves; store the split's un-normalised partial
+  const int64_t base = (((int64_t)b * p.KH + kh) * nsplit + sp) * 16;
+  const float* po = reinterpret_cast<const float*>(Vs_all);
+  for (int idx = tid; idx < 16 * VD; idx += NW * 64) {
+    int h = idx / VD, d = idx - h * VD;
+    float m = NSA_NEG_INF;
+    for (int w = 0; w < NW; w++) m = fmaxf(m, part_m[w * 16 + h]);
+    float l = 0.f, o = 0.f;
+    if (m != NSA_NEG_INF) {
+      for (int w = 0; w < NW; w++) {
+        float mw = part_m[w * 16 + h];
+        float a = (mw == NSA_NEG_INF) ? 0.f : fast_exp2((mw - m) * p.scale_log2);
+        l += a * part_l[w * 16 + h];
+        o += a * po[w * (SLOT / 2) + h * VD + d];
+      }
+    }
+    p.sp_o[(base + h) * VD + d] = o;
+    if (d == 0) { p.sp_m[base + h] = m; p.sp_l[base + h] = l; }
+  }
+}
+
+// grid (B, KH, nsplit): merge the splits (lse; split 0 also writes cmp_o), then the head-summed probabilities of
+// this split's compressed keys -> pg [B, KH, y_cap] fp32
+template <int D, int VD>
+__global__ __launch_bounds__(SPLIT_WAVES * 64) void decode_importance_kernel(NsaDecodeParams p) {
+  constexpr int NW = SPLIT_WAVES;
+  constexpr int KC = D / 32;
+  __shared__ float lse_s[16];
+  __shared__ float m_s[16], l_s[16];
+  extern __shared__ int tab_dyn[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int b = blockIdx.x, kh = blockIdx.y, sp = blockIdx.z;
+  const int nsplit = gridDim.z;
+  const int G = p.G;
+  const int L = p.ctx_lens[b];
+  const int y = L >= p.kernel_size ? min((L - p.kernel_size) / p.stride + 1, p.y_cap) : 0;
+  const int32_t* ctab = p.cmp_table + (int64_t)b * p.cmp_table_stride;
+  const int page = p.page_size;
+  for (int i = tid; i < (y + page - 1) / page; i += NW * 64) tab_dyn[i] = ctab[i];
+  const int64_t base = ((int64_t)b * p.KH + kh) * nsplit * 16;
+  if (tid < 16) {
+    float m = NSA_NEG_INF;
+    for (int s2 = 0; s2 < nsplit; s2++) m = fmaxf(m, p.sp_m[base + s2 * 16 + tid]);
+    float l = 0.f;
+    if (m != NSA_NEG_INF)
+      for (int s2 = 0; s2 < nsplit; s2++) {
+        float ms = p.sp_m[base + s2 * 16 + tid];
+        if (ms != NSA_NEG_INF) l += fast_exp2((ms - m) * p.scale_log2) * p.sp_l[base + s2 * 16 + tid];
+      }
+    m_s[tid] = m;
+    l_s[tid] = l;
+    float lse2 = (m != NSA_NEG_INF && l > 0.f) ? m * p.scale_log2 + fast_log2(l) : 0.f;
+    lse_s[tid] = lse2;
+    if (sp == 0 && tid < G && p.lse_out) p.lse_out[(int64_t)b * p.lse_st + (kh * G + tid) * p.lse_sh] = lse2;
+  }
+  __syncthreads();
+  if (sp == 0) {
+    for (int idx = tid; idx < G * VD; idx += NW * 64) {
+      int h = idx / VD, d = idx - h * VD;
+      float m = m_s[h], l = l_s[h], o = 0.f;
+      if (m != NSA_NEG_INF && l > 0.f) {
+        for (int s2 = 0; s2 < nsplit; s2++) {
+          float ms = p.sp_m[base + s2 * 16 + h];
+          if (ms != NSA_NEG_INF) o += fast_exp2((ms - m) * p.scale_log2) * p.sp_o[(base + s2 * 16 + h) * VD + d];
+        }
+        o /= l;
+      }
+      p.cmp_o[(int64_t)b * p.co_st + (int64_t)(kh * G + h) * p.co_sh + d] = (bf16_t)o;
+    }
+  }
+  // S[head][key] = Q K^T : lane holds key = l16, heads kq*4 .. +3
+  auto row_of = [&](int key) -> int64_t { return (int64_t)tab_dyn[key / page] * page + (key % page); };
+  const bf16_t* kbase = p.k + (int64_t)kh * p.k_sh;
+  const int l16 = lane & 15, kq = lane >> 4;
+  const int head = kh * G + min(l16, G - 1);
+  bf16x8 qf[KC];
+  {
+    const bf16_t* qp = p.q + (int64_t)b * p.q_st + (int64_t)head * p.q_sh + kq * 8;
+#pragma unroll
+    for (int kc = 0; kc < KC; kc++) qf[kc] = ld_global_b128(qp + kc * 32);
+  }
+  float lse4[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) lse4[i] = lse_s[kq * 4 + i];
+  float* pg = p.pg + ((int64_t)b * p.KH + kh) * p.y_cap;
+  const int nu = (y + UK - 1) / UK;
+  const int step = NW * nsplit;
+  bf16x8 kfA[2][KC], kfB[2][KC];
+  auto issue = [&](int u, bf16x8 (&kf)[2][KC]) {
+#pragma unroll
+    for (int jt = 0; jt < 2; jt++) {
+      int key = min(u * UK + jt * 16 + l16, y - 1);
+      const bf16_t* kp = kbase + row_of(key) * p.k_sr + kq * 8;
+#pragma unroll
+      for (int kc = 0; kc < KC; kc++) kf[jt][kc] = ld_global_b128(kp + kc * 32);
+    }
+  };
+  auto compute = [&](int u, bf16x8 (&kf)[2][KC]) {
+#pragma unroll
+    for (int jt = 0; jt < 2; jt++) {
+      f32x4 sv = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kc = 0; kc < KC; kc++) sv = mfma16(qf[kc], kf[jt][kc], sv);
+      float acc = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+        if (kq * 4 + i < G) acc += fast_exp2(__builtin_fmaf(sv[i], p.scale_log2, -lse4[i]));
+      acc += __shfl_xor(acc, 16, 64);
+      acc += __shfl_xor(acc, 32, 64);
+      int key = u * UK + jt * 16 + l16;
+      if (kq == 0 && key < y) pg[key] = acc;
+    }
+  };
+  const int first = sp * NW + wave;
+  if (first < nu) issue(first, kfA);
+  for (int u = first; u < nu; u += 2 * step) {
+    const bool hasB = u + step < nu;
+    if (hasB) issue(u + step, kfB);
+    compute(u, kfA);
+    if (hasB) {
+      if (u + 2 * step < nu) issue(u + 2 * step, kfA);
+      compute(u + step, kfB);
+    }
+  }
+}
+
 template <int D, int VD>
 __global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecodeParams p) {
   using UF = UnitFlash<D, VD>;
@@ -347,6 +521,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecod
   float* part_m = reinterpret_cast<float*>(dyn_raw + (size_t)NW * SLOT * 2);
   float* part_l = part_m + NW * 16;
   int* blk_s = reinterpret_cast<int*>(part_l + NW * 16);
+  int* tab_s = blk_s + 64;  // the request's raw page table
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -357,7 +532,8 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecod
   const int t = L - 1;
   const int32_t* tab = p.table + (int64_t)b * p.table_stride;
   const int page = p.page_size;
-  auto row_of = [&](int key) -> int64_t { return (int64_t)tab[key / page] * page + (key % page); };
+  for (int i = tid; i < (L + page - 1) / page; i += NW * 64) tab_s[i] = tab[i];
+  auto row_of = [&](int key) -> int64_t { return (int64_t)tab_s[key / page] * page + (key % page); };
   const bf16_t* kbase = p.k + (int64_t)kh * p.k_sh;
   const bf16_t* vbase = p.v + (int64_t)kh * p.v_sh;
   const int l16 = lane & 15;
@@ -365,7 +541,73 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecod
   const int head = kh * G + g;
   const int Bs = p.block_size;
   const int nvalid = t >= 0 ? min(p.top_n, t / Bs + 1) : 0;
-  if (tid < 64) blk_s[tid] = tid < nvalid ? p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + tid] : 0;
+  if (p.pg != nullptr) {
+    // selection prologue: fold the head-summed probabilities of the compressed keys into block scores (held in the
+    // not-yet-used V staging area), force the initial/local blocks, then repeated arg-max by wave 0
+    float* imp = reinterpret_cast<float*>(Vs_all);
+    const float* pg = p.pg + ((int64_t)b * p.KH + kh) * p.y_cap;
+    const int Kz = p.kernel_size, St = p.stride;
+    const int y = L >= Kz ? min((L - Kz) / St + 1, p.y_cap) : 0;
+    const int nb = min(L > 0 ? (L - 1) / Bs + 1 : 0, p.nb_cap);
+    const int nloops = (Bs + Kz - St) / St;
+    for (int j = tid; j < nb; j += NW * 64) {
+      float acc = 0.f;
+      int i0 = (j * Bs - Kz) / St + 1;
+      int cs = St - Kz;
+      for (int r = 0; r < nloops; r++, cs += St) {
+        int i = i0 + r;
+        if (i >= 0 && i < y) {
+          int area = min(cs + Kz, Bs) - max(cs, 0);
+          acc += pg[i] * ((float)area / (float)St);
+        }
+      }
+      imp[j] = acc;
+    }
+    __syncthreads();
+    if (wave == 0) {
+      const int nk = t >= 0 ? t / Bs : -1;
+      int result = p.ignore_index;
+      if (lane == 0) {
+        for (int s2 = 0; s2 < p.num_init; s2++)
+          if (s2 < nb) imp[s2] = -1.f;
+        for (int i = 0; i < p.num_local; i++)
+          if (nk - i >= 0 && nk - i < nb) imp[nk - i] = -1.f;
+      }
+      if (lane < p.num_init) {
+        if (lane <= nk) result = lane;
+      } else if (lane < p.num_init + p.num_local) {
+        if (lane <= nk) result = nk - (lane - p.num_init);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      const int nsel = min(p.top_n, nk + 1);
+      const int jmax = min(nk, nb - 1);
+      for (int slot = p.num_init + p.num_local; slot < nsel; slot++) {
+        float best = -2.f;
+        int bj = 0x7fffffff;
+        for (int j = lane; j <= jmax; j += 64) {
+          float v = imp[j];
+          if (v > best) { best = v; bj = j; }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+          float ob = __shfl_xor(best, o, 64);
+          int oj = __shfl_xor(bj, o, 64);
+          if (ob > best || (ob == best && oj < bj)) { best = ob; bj = oj; }
+        }
+        if (lane == slot) result = bj;
+        if (lane == 0 && bj <= jmax) imp[bj] = -1.f;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      }
+      blk_s[lane] = lane < nvalid ? max(result, 0) : 0;
+      if (lane < p.top_n) p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + lane] = result;
+    }
+  } else if (tid < 64) {
+    blk_s[tid] = tid < nvalid ? p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + tid] : 0;
+  }
   __syncthreads();
 
   UF uf;
@@ -433,7 +675,8 @@ static size_t slot_bytes() { return (size_t)DEC_WAVES * UK * (VD + NSA_LDS_PAD) 
 int nsa_decode_cmp_topk_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream) {
   if (B <= 0) return NSA_OK;
   dim3 grid(B, p.KH);
-  size_t extra = (size_t)(2 * DEC_WAVES * 16 + 16 + p.y_cap + p.nb_cap) * sizeof(float);
+  size_t extra = (size_t)(2 * DEC_WAVES * 16 + 16 + p.y_cap + p.nb_cap + (p.y_cap + p.page_size - 1) / p.page_size) *
+                 sizeof(float);
   if (D == 128 && VD == 128)
     return launch_dyn(decode_cmp_topk_kernel<128, 128>, grid, slot_bytes<128, 128>() + extra, p, stream,
                       "decode_cmp_topk_kernel");
@@ -447,7 +690,7 @@ int nsa_decode_cmp_topk_launch(const NsaDecodeParams& p, int B, int D, int VD, h
 int nsa_decode_slc_swa_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream) {
   if (B <= 0) return NSA_OK;
   dim3 grid(B, p.KH);
-  size_t extra = (size_t)(2 * DEC_WAVES * 16 + 64) * sizeof(float);
+  size_t extra = (size_t)(2 * DEC_WAVES * 16 + 64 + p.table_stride) * sizeof(float);
   if (D == 128 && VD == 128)
     return launch_dyn(decode_slc_swa_kernel<128, 128>, grid, slot_bytes<128, 128>() + extra, p, stream,
                       "decode_slc_swa_kernel");
@@ -456,4 +699,28 @@ int nsa_decode_slc_swa_launch(const NsaDecodeParams& p, int B, int D, int VD, hi
                       "decode_slc_swa_kernel");
   nsa_set_error("decode: unsupported head dims D=%d VD=%d (built: 128/128, 64/64)", D, VD);
   return NSA_ERR_UNSUPPORTED;
+}
+
+int nsa_decode_cmp_split_launch(const NsaDecodeParams& p, int B, int nsplit, int D, int VD, hipStream_t stream) {
+  if (B <= 0) return NSA_OK;
+  dim3 grid(B, p.KH, nsplit);
+  int ntab = (p.y_cap + p.page_size - 1) / p.page_size;
+  size_t dyn1 = (size_t)SPLIT_WAVES * UK * (VD + NSA_LDS_PAD) * 2 + (size_t)(2 * SPLIT_WAVES * 16 + ntab) * 4;
+  size_t dyn2 = (size_t)ntab * 4;
+  if (!((D == 128 && VD == 128) || (D == 64 && VD == 64))) {
+    nsa_set_error("decode: unsupported head dims D=%d VD=%d (built: 128/128, 64/64)", D, VD);
+    return NSA_ERR_UNSUPPORTED;
+  }
+  if (D == 128) {
+    decode_cmp_partial_kernel<128, 128><<<grid, SPLIT_WAVES * 64, dyn1, stream>>>(p);
+    int rc = nsa_check_launch("decode_cmp_partial_kernel");
+    if (rc) return rc;
+    decode_importance_kernel<128, 128><<<grid, SPLIT_WAVES * 64, dyn2, stream>>>(p);
+  } else {
+    decode_cmp_partial_kernel<64, 64><<<grid, SPLIT_WAVES * 64, dyn1, stream>>>(p);
+    int rc = nsa_check_launch("decode_cmp_partial_kernel");
+    if (rc) return rc;
+    decode_importance_kernel<64, 64><<<grid, SPLIT_WAVES * 64, dyn2, stream>>>(p);
+  }
+  return nsa_check_launch("decode_importance_kernel");
 }

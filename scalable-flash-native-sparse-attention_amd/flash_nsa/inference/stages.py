@@ -209,10 +209,39 @@ def decode_cmp_topk(q, k, v, cmp_block_tables, context_lens, fixed_y_maxlen=8192
     return cmp_o, topk
 
 
+def decode_cmp_split(q, k, v, cmp_block_tables, context_lens, nsplit=4, fixed_y_maxlen=8192, kernel_size=32,
+                     stride=16, sm_scale=None, return_lse=False):
+    """Compressed branch of the decode step, split over `nsplit` workgroups per (request, kv head) so that a batch
+    with very different context lengths still fills the chip.
+    -> (cmp_o [B,QH,VD], pg [B,KH,fixed_y_maxlen] fp32 head-summed probabilities[, lse [B,QH]])"""
+    check_bf16(q)
+    page, KH, D, ksr, ksh = _pool_args(k)
+    _, _, VD, vsr, vsh = _pool_args(v)
+    B, QH, _ = q.shape
+    sm_scale = q.size(-1) ** -0.5 if sm_scale is None else sm_scale
+    dev = q.device
+    cmp_o = torch.empty(B, QH, VD, device=dev, dtype=q.dtype)
+    pg = torch.empty(B, KH, int(fixed_y_maxlen), device=dev, dtype=torch.float32)
+    sp_ml = torch.empty(2, B, KH, nsplit, 16, device=dev, dtype=torch.float32)
+    sp_o = torch.empty(B, KH, nsplit, 16, VD, device=dev, dtype=torch.float32)
+    lse = torch.empty(B, QH, device=dev, dtype=torch.float32) if return_lse else None
+    _lib.call("nsa_decode_cmp_split", q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), ksr, ksh, v.data_ptr(),
+              vsr, vsh, cmp_o.data_ptr(), cmp_o.stride(0), cmp_o.stride(1), _lib.ptr(lse),
+              lse.stride(0) if return_lse else 0, lse.stride(1) if return_lse else 0, pg.data_ptr(),
+              sp_ml[0].data_ptr(), sp_ml[1].data_ptr(), sp_o.data_ptr(), nsplit, _i32(context_lens).data_ptr(),
+              _i32(cmp_block_tables).data_ptr(), cmp_block_tables.stride(0), page, B, QH, KH, D, VD,
+              int(fixed_y_maxlen), kernel_size, stride, sm_scale, _lib.stream_ptr())
+    if return_lse:
+        return cmp_o, pg, lse
+    return cmp_o, pg
+
+
 def decode_slc_swa_combine(q, k, v, w, topk, cmp_o, block_tables, context_lens, block_size=64, top_n=16,
-                           window_size=512, sm_scale=None, return_branches=False):
+                           window_size=512, sm_scale=None, return_branches=False, pg=None, fixed_num_slc_blocks=2048,
+                           kernel_size=32, stride=16, num_inital=1, num_local=2):
     """One launch: selected-block + window attention and the gated combine -> o [B,QH,VD]
-    (with return_branches also slc_o, swa_o)."""
+    (with return_branches also slc_o, swa_o).  With `pg` (from decode_cmp_split) the block selection runs in the
+    kernel's prologue and `topk` may be None; the selection is then returned as a third/fifth value."""
     check_bf16(q)
     page, KH, D, ksr, ksh = _pool_args(k)
     _, _, VD, vsr, vsh = _pool_args(v)
@@ -222,12 +251,17 @@ def decode_slc_swa_combine(q, k, v, w, topk, cmp_o, block_tables, context_lens, 
     slc_o = torch.empty_like(out) if return_branches else None
     swa_o = torch.empty_like(out) if return_branches else None
     assert cmp_o.stride() == out.stride()
+    select_here = pg is not None
+    if select_here:
+        topk = torch.empty(KH, B, top_n, device=q.device, dtype=torch.int32)
     _lib.call("nsa_decode_slc_swa_combine", q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), ksr, ksh,
               v.data_ptr(), vsr, vsh, w.data_ptr(), w.stride(0), w.stride(1), topk.data_ptr(), topk.stride(0),
-              topk.stride(1), cmp_o.data_ptr(), _lib.ptr(slc_o), _lib.ptr(swa_o), cmp_o.stride(0), cmp_o.stride(1),
-              out.data_ptr(), out.stride(0), out.stride(1), _i32(context_lens).data_ptr(),
+              topk.stride(1), _lib.ptr(pg), pg.size(-1) if select_here else 0, int(fixed_num_slc_blocks), kernel_size,
+              stride, num_inital, num_local, -1, cmp_o.data_ptr(), _lib.ptr(slc_o), _lib.ptr(swa_o), cmp_o.stride(0),
+              cmp_o.stride(1), out.data_ptr(), out.stride(0), out.stride(1), _i32(context_lens).data_ptr(),
               _i32(block_tables).data_ptr(), block_tables.stride(0), page, B, QH, KH, D, VD, block_size, top_n,
               window_size, sm_scale, _lib.stream_ptr())
-    if return_branches:
-        return out, slc_o, swa_o
-    return out
+    res = (out, slc_o, swa_o) if return_branches else (out,)
+    if select_here:
+        res = res + (topk,)
+    return res if len(res) > 1 else res[0]

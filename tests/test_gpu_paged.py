@@ -216,3 +216,17 @@ def test_fused_decode_matches_staged_decode(device, QH, KH, D):
     ref = nsa_decode_staged(q, d["k"], d["v"], w, ctx_t, d["bt"], d["cbt"], fixed_y_maxlen=512,
                             fixed_num_slc_blocks=64, **kw)
     assert_close(out, ref, "decode o", atol=8e-3, rtol=1e-2)
+    # split compressed branch + in-kernel selection (the path nsa_decode takes)
+    from flash_nsa.inference import decode_cmp_split
+    for nsplit in (1, 3, 4):
+        cmp2, pg, lse2 = decode_cmp_split(q, d["k"], d["v"], d["cbt"], ctx_t, nsplit=nsplit, fixed_y_maxlen=512,
+                                          return_lse=True)
+        assert_close(cmp2, r_cmp, f"split{nsplit} cmp_o", atol=4e-3, rtol=1e-2)
+        assert_close(lse2, r_lse, f"split{nsplit} lse", atol=1e-3, rtol=1e-4)
+        out2, topk2 = decode_slc_swa_combine(q, d["k"], d["v"], w, None, cmp2, d["bt"], ctx_t, pg=pg,
+                                             fixed_num_slc_blocks=64, **kw)
+        t2 = topk2.cpu()
+        for b in range(B):
+            for kh in range(KH):
+                assert sorted(t2[kh, b, :nv[b]].tolist()) == sorted(r[kh, b, :nv[b]].tolist()), (nsplit, b, kh)
+        assert_close(out2, ref, f"split{nsplit} decode o", atol=8e-3, rtol=1e-2)
