@@ -72,11 +72,18 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
   if (MODE == MODE_CMP) {
     kbase = p.k_cu[b];
     nkeys = p.k_cu[b + 1] - kbase;
+    // blockIdx.x enumerates only the (key tile, query chunk) pairs that have visible rows, key-tile major, so
+    // that consecutive workgroups (which the dispatcher deals round-robin to the XCDs) carry equal work
     const int nch = cdiv_i(xl, p.q_chunk_tokens);
-    const int ktile = blockIdx.x / p.grid_chunks;
-    const int ch = blockIdx.x - ktile * p.grid_chunks;
+    int rem = blockIdx.x, ktile = 0, ch = -1;
+    for (; ktile * KW < nkeys; ktile++) {
+      const int fc = min(nch, (p.stride * ktile * KW + p.kernel_size - 1) / p.q_chunk_tokens);
+      const int cnt = nch - fc;
+      if (rem < cnt) { ch = fc + rem; break; }
+      rem -= cnt;
+    }
+    if (ch < 0) return;
     key0 = ktile * KW;
-    if (key0 >= nkeys || ch >= nch) return;
     const int first = p.stride * key0 + p.kernel_size - 1;
     const int ta = max(ch * p.q_chunk_tokens, first);
     const int tb = min((ch + 1) * p.q_chunk_tokens, xl);
@@ -130,40 +137,116 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
   bf16x8 qreg[QJ], oreg[OJ];
   float lse_reg = 0.f, delta_reg = 0.f;
   int t_reg = T_INVALID;
-  auto row_of = [&](int rr, int& n, int& g) {  // group-row -> (token local to the sequence, head in group)
+  // Per-thread row bookkeeping.  A thread stages the same tile-relative rows every iteration, so when G is a power
+  // of two dividing 64 its (token index, head) pairs advance by a constant per tile and no division is needed in
+  // the loop; other group sizes recompute the pair each time.
+  const bool fastG = gshift >= 0 && G <= RT;
+  const int n_step = fastG ? (RT >> gshift) : 0;
+  const int row_last = row_end - 1;
+  auto split_row = [&](int rr, int& n, int& g) {
     if (gshift >= 0) { n = rr >> gshift; g = rr & (G - 1); }
     else { n = rr / G; g = rr - n * G; }
-    if (MODE == MODE_SLC) n = list[n];
+  };
+  int n_lastrow, g_lastrow;
+  split_row(row_last, n_lastrow, g_lastrow);
+  int qn[QJ], on[OJ], sn;                 // token index (MODE_SLC: list position) of the thread's rows, current tile
+  int64_t qoffs[QJ], ooffs[OJ];           // head + channel offsets (elements)
+  int sg;
+#pragma unroll
+  for (int j = 0; j < QJ; j++) {
+    int pc = tid + j * NT, g;
+    split_row(row_begin + pc / QP, qn[j], g);
+    qoffs[j] = (int64_t)(kh * G + g) * p.q_sh + (pc % QP) * 8;
+  }
+#pragma unroll
+  for (int j = 0; j < OJ; j++) {
+    int pc = tid + j * NT, g;
+    split_row(row_begin + pc / OP, on[j], g);
+    ooffs[j] = (int64_t)(kh * G + g) * p.do_sh + (pc % OP) * 8;
+  }
+  split_row(row_begin + (tid & (RT - 1)), sn, sg);
+  const int64_t qoff_last = (int64_t)(kh * G + g_lastrow) * p.q_sh;
+  const int64_t ooff_last = (int64_t)(kh * G + g_lastrow) * p.do_sh;
+  // (token index or list position, head+channel offset) of tile-relative row `rowrel` for the tile starting at rt0
+  auto locate = [&](int rt0, int rowrel, int n_inc, int64_t off_inc, int64_t off_last, int chan, int64_t hstride,
+                    int& n, int64_t& off) {
+    if (!fastG) {
+      int g;
+      split_row(min(rt0 + rowrel, row_last), n, g);
+      off = (int64_t)(kh * G + g) * hstride + chan;
+    } else if (rt0 + rowrel > row_last) {
+      n = n_lastrow;
+      off = off_last + chan;
+    } else {
+      n = n_inc;
+      off = off_inc;
+    }
+  };
+  // MODE_SLC: tokens of the NEXT tile to load, fetched from the inverse-index list one tile ahead of their use so
+  // that the dependent (list -> row) lookups never stall the pipeline
+  int tq[QJ], to[OJ], tsn = 0;
+  auto fetch_tokens = [&](int rt0) {
+    if (MODE != MODE_SLC) return;
+#pragma unroll
+    for (int j = 0; j < QJ; j++) {
+      int pc = tid + j * NT, n;
+      int64_t off;
+      locate(rt0, pc / QP, qn[j], 0, 0, 0, 0, n, off);
+      tq[j] = list[n];
+    }
+    if (QP != OP) {
+#pragma unroll
+      for (int j = 0; j < OJ; j++) {
+        int pc = tid + j * NT, n;
+        int64_t off;
+        locate(rt0, pc / OP, on[j], 0, 0, 0, 0, n, off);
+        to[j] = list[n];
+      }
+    }
+    if (tid < RT) {
+      int n;
+      int64_t off;
+      locate(rt0, tid, sn, 0, 0, 0, 0, n, off);
+      tsn = list[n];
+    }
   };
   auto gload = [&](int rt0) {
 #pragma unroll
     for (int j = 0; j < QJ; j++) {
-      int pc = tid + j * NT;
-      int rr = min(rt0 + pc / QP, row_end - 1), dp = pc % QP;
-      int n, g;
-      row_of(rr, n, g);
-      qreg[j] = ld_global_b128(p.q + (int64_t)(x0 + n) * p.q_st + (int64_t)(kh * G + g) * p.q_sh + dp * 8);
+      int pc = tid + j * NT, n;
+      int64_t off;
+      locate(rt0, pc / QP, qn[j], qoffs[j], qoff_last, (pc % QP) * 8, p.q_sh, n, off);
+      if (MODE == MODE_SLC) n = tq[j];
+      qreg[j] = ld_global_b128(p.q + (int64_t)(x0 + n) * p.q_st + off);
     }
 #pragma unroll
     for (int j = 0; j < OJ; j++) {
-      int pc = tid + j * NT;
-      int rr = min(rt0 + pc / OP, row_end - 1), dp = pc % OP;
-      int n, g;
-      row_of(rr, n, g);
-      oreg[j] = ld_global_b128(p.dO + (int64_t)(x0 + n) * p.do_st + (int64_t)(kh * G + g) * p.do_sh + dp * 8);
+      int pc = tid + j * NT, n;
+      int64_t off;
+      locate(rt0, pc / OP, on[j], ooffs[j], ooff_last, (pc % OP) * 8, p.do_sh, n, off);
+      if (MODE == MODE_SLC) n = (QP == OP) ? tq[j] : to[j];
+      oreg[j] = ld_global_b128(p.dO + (int64_t)(x0 + n) * p.do_st + off);
     }
     if (tid < RT) {
-      int rr = rt0 + tid;
-      bool ok = rr < row_end;
-      int n, g;
-      row_of(ok ? rr : row_end - 1, n, g);
-      int64_t tok = x0 + n;
-      int head = kh * G + g;
-      lse_reg = p.lse[tok * p.lse_st + (int64_t)head * p.lse_sh];
-      delta_reg = p.delta[tok * p.delta_st + (int64_t)head * p.delta_sh];
+      const bool ok = rt0 + tid <= row_last;
+      int n;
+      int64_t hoff;
+      locate(rt0, tid, sn, (int64_t)(kh * G + sg), (int64_t)(kh * G + g_lastrow), 0, 1, n, hoff);
+      if (MODE == MODE_SLC) n = tsn;
+      const int64_t tok = x0 + n;
+      lse_reg = p.lse[tok * p.lse_st + hoff * p.lse_sh];
+      delta_reg = p.delta[tok * p.delta_st + hoff * p.delta_sh];
       t_reg = ok ? n : T_INVALID;
     }
+    // advance the bookkeeping to the next tile, then start fetching that tile's tokens
+#pragma unroll
+    for (int j = 0; j < QJ; j++) qn[j] += n_step;
+#pragma unroll
+    for (int j = 0; j < OJ; j++) on[j] += n_step;
+    sn += n_step;
+    if (rt0 + RT < row_end) fetch_tokens(rt0 + RT);
   };
+  fetch_tokens(row_begin);
   gload(row_begin);
 
   for (int rt0 = row_begin; rt0 < row_end; rt0 += RT) {
@@ -313,8 +396,14 @@ int launch(const NsaBwdTileParams& p0, int mode, int B, int max_q_len, int max_k
   NsaBwdTileParams p = p0;
   if (mode == MODE_CMP) {
     if (B <= 0 || max_k_len <= 0) return NSA_OK;
-    p.grid_chunks = cdiv_i(max_q_len, p.q_chunk_tokens);
-    dim3 grid(cdiv_i(max_k_len, 128) * p.grid_chunks, B, p.KH);
+    const int nch = cdiv_i(max_q_len, p.q_chunk_tokens);
+    int total = 0;
+    for (int kt = 0; kt * 128 < max_k_len; kt++)
+      total += nch - (nch < (p.stride * kt * 128 + p.kernel_size - 1) / p.q_chunk_tokens
+                          ? nch
+                          : (p.stride * kt * 128 + p.kernel_size - 1) / p.q_chunk_tokens);
+    if (total <= 0) return NSA_OK;
+    dim3 grid(total, B, p.KH);
     bwd_dkdv_kernel<D, VD, MODE_CMP, 4><<<grid, 256, 0, stream>>>(p);
   } else if (mode == MODE_SWA) {
     if (B <= 0 || max_k_len <= 0) return NSA_OK;

@@ -45,7 +45,7 @@ def slc_topk_indices(q, k, lse, sm_scale=None, return_slc_prob=False, align=True
 
 
 @torch.no_grad()
-def get_bind_from_find(topk, helper=NSAHelper, chunk_tokens=256):
+def get_bind_from_find(topk, helper=NSAHelper, chunk_tokens=1024):
     """Inverse of the selection: for every (kv head, selection block) the ascending list of query tokens that
     selected it.  Returns a dict with the CSR (csr_off [KH,nblk+1], csr_tok [KH*T*top_n]), the work-item prefix
     (item_off [KH,nblk+1]) and the static bound on the number of work items per kv head."""
