@@ -324,12 +324,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_cmp_topk_kernel(NsaDeco
         float v = imp[j];
         if (v > best) { best = v; bj = j; }
       }
-#pragma unroll
-      for (int o = 32; o > 0; o >>= 1) {
-        float ob = __shfl_xor(best, o, 64);
-        int oj = __shfl_xor(bj, o, 64);
-        if (ob > best || (ob == best && oj < bj)) { best = ob; bj = oj; }
-      }
+      bj = wave_argmax_lowest(best, bj, bj != 0x7fffffff);
       if (lane == slot) result = bj;
       if (lane == 0 && bj <= jmax) imp[bj] = -1.f;
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -590,12 +585,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecod
           float v = imp[j];
           if (v > best) { best = v; bj = j; }
         }
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) {
-          float ob = __shfl_xor(best, o, 64);
-          int oj = __shfl_xor(bj, o, 64);
-          if (ob > best || (ob == best && oj < bj)) { best = ob; bj = oj; }
-        }
+        bj = wave_argmax_lowest(best, bj, bj != 0x7fffffff);
         if (lane == slot) result = bj;
         if (lane == 0 && bj <= jmax) imp[bj] = -1.f;
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

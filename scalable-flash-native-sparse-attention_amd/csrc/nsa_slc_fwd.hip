@@ -19,11 +19,15 @@ __global__ __launch_bounds__(256, 2) void slc_fwd_kernel(NsaSlcParams p) {
   constexpr int UK = 32;                      // keys per unit
   constexpr int KC = D / 32;                  // K fragments per 16-key tile
   constexpr int VJ = (UK * (VD / 8)) / 64;    // 16-byte V loads per lane and unit
+  constexpr int KJ = (UK * (D / 8)) / 64;     // 16-byte K loads per lane and unit
+  constexpr int KLD = D + NSA_LDS_PAD;
   __shared__ __attribute__((aligned(16))) bf16_t Vs_all[4 * UK * VLD];
+  __shared__ __attribute__((aligned(16))) bf16_t Ks_all[4 * UK * KLD];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   bf16_t* Vs = Vs_all + wave * UK * VLD;
+  bf16_t* Ks = Ks_all + wave * UK * KLD;
   const int l16 = lane & 15;
   const int kq = lane >> 4;
   const int b = blockIdx.y;
@@ -65,40 +69,71 @@ __global__ __launch_bounds__(256, 2) void slc_fwd_kernel(NsaSlcParams p) {
   float m_run = NSA_NEG_INF, l_run = 0.f;
   const float sc = p.scale_log2;
 
-  // first key of unit u (negative block ids -- ignore values -- are clamped; such units are fully masked)
+  // first key of unit u; wave-uniform.  Units that start past the last attendable key (second half of the current
+  // block) and ignore values (negative ids) are reported as -1 and skipped.
   auto unit_key0 = [&](int u) {
     int slot = u / upb;
-    int blk = __shfl(my_blk, slot, 64);
-    return blk * Bs + (u - slot * upb) * UK;
+    int blk = __builtin_amdgcn_readfirstlane(__shfl(my_blk, slot, 64));
+    int key0 = blk * Bs + (u - slot * upb) * UK;
+    return (blk < 0 || key0 > key_last) ? -1 : key0;
   };
-  auto row_of_key = [&](int key) -> int64_t {  // flat K/V row of an absolute key position
-    if (PAGED) return (int64_t)table[key / p.page_size] * p.page_size + (key % p.page_size);
-    return (int64_t)x0 + key;
-  };
-  auto issue = [&](int key0, bf16x8 (&kf)[2][KC], bf16x8 (&vr)[VJ]) {
-    // out-of-range keys are replaced by the last attendable key; their scores are masked
+  // per-lane element offsets inside a unit are the same for every unit: the loads are (uniform base) + offset
+  // K and V rows are fetched as whole 16-byte-per-lane coalesced rows (every cache line is requested once and used
+  // completely) and go through wave-private LDS; the MFMA fragments are read from there
+  int64_t koff[KJ], voff[VJ];
 #pragma unroll
-    for (int jt = 0; jt < 2; jt++) {
-      int key = max(0, min(key0 + jt * 16 + l16, key_last));
-      const bf16_t* kp = p.k + row_of_key(key) * p.k_sr + (int64_t)kh * p.k_sh + kq * 8;
+  for (int j = 0; j < KJ; j++) {
+    int pc = lane + j * 64;
+    koff[j] = (int64_t)(pc / (D / 8)) * p.k_sr + (pc % (D / 8)) * 8;
+  }
 #pragma unroll
-      for (int kc = 0; kc < KC; kc++) kf[jt][kc] = ld_global_b128(kp + kc * 32);
+  for (int j = 0; j < VJ; j++) {
+    int pc = lane + j * 64;
+    voff[j] = (int64_t)(pc / (VD / 8)) * p.v_sr + (pc % (VD / 8)) * 8;
+  }
+  auto issue = [&](int key0, bf16x8 (&kf)[KJ], bf16x8 (&vr)[VJ]) {
+    if (key0 < 0) return;
+    int64_t row0;  // flat row of the unit's first key (a unit never straddles a page)
+    if (PAGED) row0 = (int64_t)__builtin_amdgcn_readfirstlane(table[key0 / p.page_size]) * p.page_size + (key0 % p.page_size);
+    else row0 = (int64_t)x0 + key0;
+    const bf16_t* kb = p.k + row0 * p.k_sr + (int64_t)kh * p.k_sh;
+    const bf16_t* vb = p.v + row0 * p.v_sr + (int64_t)kh * p.v_sh;
+    const int kmax = key_last - key0;  // >= 0
+    if (kmax >= UK - 1) {
+#pragma unroll
+      for (int j = 0; j < KJ; j++) kf[j] = ld_global_b128(kb + koff[j]);
+#pragma unroll
+      for (int j = 0; j < VJ; j++) vr[j] = ld_global_b128(vb + voff[j]);
+    } else {  // the unit holding the causal boundary: rows past it are replaced by the boundary row (masked later)
+#pragma unroll
+      for (int j = 0; j < KJ; j++) {
+        int pc = lane + j * 64;
+        kf[j] = ld_global_b128(kb + (int64_t)min(pc / (D / 8), kmax) * p.k_sr + (pc % (D / 8)) * 8);
+      }
+#pragma unroll
+      for (int j = 0; j < VJ; j++) {
+        int pc = lane + j * 64;
+        vr[j] = ld_global_b128(vb + (int64_t)min(pc / (VD / 8), kmax) * p.v_sr + (pc % (VD / 8)) * 8);
+      }
     }
+  };
+  auto compute = [&](int key0, bf16x8 (&kf)[KJ], bf16x8 (&vr)[VJ]) {
+    if (key0 < 0) return;
 #pragma unroll
-    for (int j = 0; j < VJ; j++) {
+    for (int j = 0; j < KJ; j++) {
       int pc = lane + j * 64;
-      int kr = pc / (VD / 8), dp = pc % (VD / 8);
-      int key = max(0, min(key0 + kr, key_last));
-      vr[j] = ld_global_b128(p.v + row_of_key(key) * p.v_sr + (int64_t)kh * p.v_sh + dp * 8);
+      *reinterpret_cast<bf16x8*>(&Ks[(pc / (D / 8)) * KLD + (pc % (D / 8)) * 8]) = kf[j];
     }
-  };
-  auto compute = [&](int key0, bf16x8 (&kf)[2][KC], bf16x8 (&vr)[VJ]) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     f32x4 sacc[2];
 #pragma unroll
     for (int jt = 0; jt < 2; jt++) {
       sacc[jt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const bf16_t* kp = &Ks[(jt * 16 + l16) * KLD + kq * 8];
 #pragma unroll
-      for (int kc = 0; kc < KC; kc++) sacc[jt] = mfma16(kf[jt][kc], qf[kc], sacc[jt]);
+      for (int kc = 0; kc < KC; kc++) sacc[jt] = mfma16(*reinterpret_cast<const bf16x8*>(kp + kc * 32), qf[kc], sacc[jt]);
     }
     // V rows -> wave-private LDS (previous unit's transpose reads are complete: LDS ops of a wave are in order)
 #pragma unroll
@@ -106,14 +141,14 @@ __global__ __launch_bounds__(256, 2) void slc_fwd_kernel(NsaSlcParams p) {
       int pc = lane + j * 64;
       *reinterpret_cast<bf16x8*>(&Vs[(pc / (VD / 8)) * VLD + (pc % (VD / 8)) * 8]) = vr[j];
     }
-    const int kmax = key_last - key0;  // last usable key offset inside this unit (may be negative)
-    if (key0 < 0 || kmax < UK - 1) {   // wave-uniform: only the unit holding the causal boundary is masked
+    const int kmax = key_last - key0;  // last usable key offset inside this unit
+    if (kmax < UK - 1) {               // wave-uniform: only the unit holding the causal boundary is masked
 #pragma unroll
       for (int jt = 0; jt < 2; jt++)
 #pragma unroll
         for (int i = 0; i < 4; i++) {
           int ko = jt * 16 + kq * 4 + i;
-          if (key0 < 0 || ko > kmax) sacc[jt][i] = NSA_NEG_INF;
+          if (ko > kmax) sacc[jt][i] = NSA_NEG_INF;
         }
     }
     float tmax = fmaxf(fmaxf(fmaxf(sacc[0][0], sacc[0][1]), fmaxf(sacc[0][2], sacc[0][3])),
@@ -159,7 +194,7 @@ __global__ __launch_bounds__(256, 2) void slc_fwd_kernel(NsaSlcParams p) {
     __builtin_amdgcn_wave_barrier();
   };
 
-  bf16x8 kfA[2][KC], kfB[2][KC], vrA[VJ], vrB[VJ];
+  bf16x8 kfA[KJ], kfB[KJ], vrA[VJ], vrB[VJ];
   int keyA = 0, keyB = 0;
   if (nu > 0) { keyA = unit_key0(0); issue(keyA, kfA, vrA); }
   for (int u = 0; u < nu; u += 2) {

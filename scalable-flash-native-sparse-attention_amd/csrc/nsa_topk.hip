@@ -229,12 +229,7 @@ __global__ __launch_bounds__(256) void topk_kernel(NsaTopkParams p) {
         float v = imp[j];
         if (v > best) { best = v; bj = j; }
       }
-#pragma unroll
-      for (int o = 32; o > 0; o >>= 1) {
-        float ob = __shfl_xor(best, o, 64);
-        int oj = __shfl_xor(bj, o, 64);
-        if (ob > best || (ob == best && oj < bj)) { best = ob; bj = oj; }
-      }
+      bj = wave_argmax_lowest(best, bj, bj != 0x7fffffff);
       if (lane == slot) result = bj;
       if (lane == 0 && bj <= jmax) imp[bj] = -1.f;
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
