@@ -11,7 +11,7 @@ namespace {
 constexpr int MODE_CMP = 0;
 constexpr int MODE_SWA = 1;
 
-template <int D, int VD, int MODE, int MINB>
+template <int D, int VD, int MODE, int MINB, bool DO_LDS>
 __global__ __launch_bounds__(256, MINB) void bwd_dq_tile_kernel(NsaBwdTileParams p) {
   constexpr int ROWS_W = 32;
   constexpr int ROWS_WG = 4 * ROWS_W;
@@ -20,6 +20,9 @@ __global__ __launch_bounds__(256, MINB) void bwd_dq_tile_kernel(NsaBwdTileParams
   constexpr int VLD = VD + NSA_LDS_PAD;
   __shared__ __attribute__((aligned(16))) bf16_t Ks[KT * KLD];
   __shared__ __attribute__((aligned(16))) bf16_t Vs[KT * VLD];
+  // with DO_LDS the dO fragments of a wave's 32 rows live in a wave-private LDS region instead of 32 registers,
+  // which brings the kernel under 256 registers (two workgroups per CU)
+  __shared__ __attribute__((aligned(16))) bf16_t dOs[DO_LDS ? 4 * 32 * VLD : 8];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -53,14 +56,18 @@ __global__ __launch_bounds__(256, MINB) void bwd_dq_tile_kernel(NsaBwdTileParams
   const int64_t tok = x0 + n;
   const int head = kh * G + g;
 
-  bf16x8 qf[D / 16], dof[VD / 16];
+  bf16x8 qf[D / 16], dof[DO_LDS ? 1 : VD / 16];
   {
     const bf16_t* qp = p.q + tok * p.q_st + (int64_t)head * p.q_sh + hl * 8;
 #pragma unroll
     for (int kc = 0; kc < D / 16; kc++) qf[kc] = ld_global_b128(qp + kc * 16);
     const bf16_t* dp = p.dO + tok * p.do_st + (int64_t)head * p.do_sh + hl * 8;
 #pragma unroll
-    for (int kc = 0; kc < VD / 16; kc++) dof[kc] = ld_global_b128(dp + kc * 16);
+    for (int kc = 0; kc < VD / 16; kc++) {
+      bf16x8 t8 = ld_global_b128(dp + kc * 16);
+      if (DO_LDS) *reinterpret_cast<bf16x8*>(&dOs[(wave * 32 + l32) * VLD + hl * 8 + kc * 16]) = t8;
+      else dof[kc] = t8;
+    }
   }
   const float lse = p.lse[tok * p.lse_st + (int64_t)head * p.lse_sh];
   const float delta = p.delta[tok * p.delta_st + (int64_t)head * p.delta_sh];
@@ -152,8 +159,9 @@ __global__ __launch_bounds__(256, MINB) void bwd_dq_tile_kernel(NsaBwdTileParams
       const bf16_t* vp1 = vp0 + 32 * VLD;
 #pragma unroll
       for (int kc = 0; kc < VD / 16; kc++) {
-        pacc[0] = mfma32(*reinterpret_cast<const bf16x8*>(vp0 + kc * 16), dof[kc], pacc[0]);
-        pacc[1] = mfma32(*reinterpret_cast<const bf16x8*>(vp1 + kc * 16), dof[kc], pacc[1]);
+        bf16x8 df = DO_LDS ? *reinterpret_cast<const bf16x8*>(&dOs[(wave * 32 + l32) * VLD + hl * 8 + kc * 16]) : dof[kc];
+        pacc[0] = mfma32(*reinterpret_cast<const bf16x8*>(vp0 + kc * 16), df, pacc[0]);
+        pacc[1] = mfma32(*reinterpret_cast<const bf16x8*>(vp1 + kc * 16), df, pacc[1]);
       }
     }
     const float lsc = lse;
@@ -218,12 +226,12 @@ template <int MODE>
 int dispatch(const NsaBwdTileParams& p, int B, int max_q_len, int D, int VD, hipStream_t stream) {
   if (B <= 0 || max_q_len <= 0) return NSA_OK;
   dim3 grid(cdiv_i(max_q_len * p.G, 128), B, p.KH);
-  static const int minb = nsa_tuning_knob("NSA_DQ_MINB", 1);
+  static const int minb = nsa_tuning_knob("NSA_DQ_MINB", 2);
   if (D == 128 && VD == 128) {
-    if (minb == 2) bwd_dq_tile_kernel<128, 128, MODE, 2><<<grid, 256, 0, stream>>>(p);
-    else bwd_dq_tile_kernel<128, 128, MODE, 1><<<grid, 256, 0, stream>>>(p);
-  } else if (D == 64 && VD == 64) bwd_dq_tile_kernel<64, 64, MODE, 2><<<grid, 256, 0, stream>>>(p);
-  else if (D == 192 && VD == 128) bwd_dq_tile_kernel<192, 128, MODE, 1><<<grid, 256, 0, stream>>>(p);
+    if (minb == 2) bwd_dq_tile_kernel<128, 128, MODE, 2, true><<<grid, 256, 0, stream>>>(p);
+    else bwd_dq_tile_kernel<128, 128, MODE, 1, false><<<grid, 256, 0, stream>>>(p);
+  } else if (D == 64 && VD == 64) bwd_dq_tile_kernel<64, 64, MODE, 2, false><<<grid, 256, 0, stream>>>(p);
+  else if (D == 192 && VD == 128) bwd_dq_tile_kernel<192, 128, MODE, 1, false><<<grid, 256, 0, stream>>>(p);
   else {
     nsa_set_error("attention dq: unsupported head dims D=%d VD=%d", D, VD);
     return NSA_ERR_UNSUPPORTED;

@@ -9,13 +9,21 @@
 namespace {
 
 template <int D, int VD>
-__global__ __launch_bounds__(256) void slc_dq_kernel(NsaSlcBwdDqParams p) {
+__global__ __launch_bounds__(256, 2) void slc_dq_kernel(NsaSlcBwdDqParams p) {
+  // Work unit = 32 keys.  The K and V rows of unit u+1 are fetched (coalesced 16-byte-per-lane row loads) into
+  // registers while unit u is computed out of wave-private LDS.
+  constexpr int UK = 32;
   constexpr int KLD = D + NSA_LDS_PAD;
-  __shared__ __attribute__((aligned(16))) bf16_t Ks_all[4 * 64 * KLD];
+  constexpr int VLD = VD + NSA_LDS_PAD;
+  constexpr int KC = D / 32, VC = VD / 32;
+  constexpr int KJ = (UK * (D / 8)) / 64, VJ = (UK * (VD / 8)) / 64;
+  __shared__ __attribute__((aligned(16))) bf16_t Ks_all[4 * UK * KLD];
+  __shared__ __attribute__((aligned(16))) bf16_t Vs_all[4 * UK * VLD];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
-  bf16_t* Ks = Ks_all + wave * 64 * KLD;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  bf16_t* Ks = Ks_all + wave * UK * KLD;
+  bf16_t* Vs = Vs_all + wave * UK * VLD;
   const int l16 = lane & 15;
   const int kq = lane >> 4;
   const int b = blockIdx.y;
@@ -31,20 +39,23 @@ __global__ __launch_bounds__(256) void slc_dq_kernel(NsaSlcBwdDqParams p) {
   const int64_t tok = x0 + n;
   const int Bs = p.block_size;
   const int nvalid = min(p.top_n, t / Bs + 1);
+  const int upb = Bs / UK;
+  const int nu = nvalid * upb;
+  const int key_last = min(xl - 1, t);
 
   int g = hc * 16 + l16;
   const bool head_ok = g < p.G;
   if (!head_ok) g = p.G - 1;
   const int head = kh * p.G + g;
 
-  bf16x8 qf[D / 32], dof[VD / 32];
+  bf16x8 qf[KC], dof[VC];
   {
     const bf16_t* qp = p.q + tok * p.q_st + (int64_t)head * p.q_sh + kq * 8;
 #pragma unroll
-    for (int kc = 0; kc < D / 32; kc++) qf[kc] = ld_global_b128(qp + kc * 32);
+    for (int kc = 0; kc < KC; kc++) qf[kc] = ld_global_b128(qp + kc * 32);
     const bf16_t* dp = p.dO + tok * p.do_st + (int64_t)head * p.do_sh + kq * 8;
 #pragma unroll
-    for (int kc = 0; kc < VD / 32; kc++) dof[kc] = ld_global_b128(dp + kc * 32);
+    for (int kc = 0; kc < VC; kc++) dof[kc] = ld_global_b128(dp + kc * 32);
   }
   const float lse = p.lse[tok * p.lse_st + (int64_t)head * p.lse_sh];
   const float delta = p.delta[tok * p.delta_st + (int64_t)head * p.delta_sh];
@@ -55,78 +66,116 @@ __global__ __launch_bounds__(256) void slc_dq_kernel(NsaSlcBwdDqParams p) {
 #pragma unroll
   for (int dt = 0; dt < D / 16; dt++) dqacc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   const float sc = p.scale_log2;
-  const int subs = Bs / 64;
 
-  for (int slot = 0; slot < nvalid; slot++) {
-    const int blk = __shfl(my_blk, slot, 64);
-    for (int sub = 0; sub < subs; sub++) {
-      const int key0 = blk * Bs + sub * 64;
-      if (key0 > t || key0 < 0) continue;
-      const int64_t row0 = (int64_t)x0 + key0;
-      const int kmax = min(xl - 1, t) - key0;
-
-      // K tile -> registers -> wave-private LDS
-      bf16x8 kreg[D / 8];
+  auto unit_key0 = [&](int u) {  // wave-uniform; -1: nothing to attend in this unit
+    int slot = u / upb;
+    int blk = __builtin_amdgcn_readfirstlane(__shfl(my_blk, slot, 64));
+    int key0 = blk * Bs + (u - slot * upb) * UK;
+    return (blk < 0 || key0 > key_last) ? -1 : key0;
+  };
+  int64_t koff[KJ], voff[VJ];
 #pragma unroll
-      for (int j = 0; j < (D / 8); j++) {
+  for (int j = 0; j < KJ; j++) {
+    int pc = lane + j * 64;
+    koff[j] = (int64_t)(pc / (D / 8)) * p.k_sr + (pc % (D / 8)) * 8;
+  }
+#pragma unroll
+  for (int j = 0; j < VJ; j++) {
+    int pc = lane + j * 64;
+    voff[j] = (int64_t)(pc / (VD / 8)) * p.v_sr + (pc % (VD / 8)) * 8;
+  }
+  auto issue = [&](int key0, bf16x8 (&kr)[KJ], bf16x8 (&vr)[VJ]) {
+    if (key0 < 0) return;
+    const int64_t row0 = (int64_t)x0 + key0;
+    const bf16_t* kb = p.k + row0 * p.k_sr + (int64_t)kh * p.k_sh;
+    const bf16_t* vb = p.v + row0 * p.v_sr + (int64_t)kh * p.v_sh;
+    const int kmax = key_last - key0;
+    if (kmax >= UK - 1) {
+#pragma unroll
+      for (int j = 0; j < KJ; j++) kr[j] = ld_global_b128(kb + koff[j]);
+#pragma unroll
+      for (int j = 0; j < VJ; j++) vr[j] = ld_global_b128(vb + voff[j]);
+    } else {  // causal boundary unit: rows past the boundary are replaced by the boundary row (masked later)
+#pragma unroll
+      for (int j = 0; j < KJ; j++) {
         int pc = lane + j * 64;
-        int kr = pc / (D / 8), dp = pc - kr * (D / 8);
-        int krc = min(kr, kmax);
-        kreg[j] = ld_global_b128(p.k + (row0 + krc) * p.k_sr + (int64_t)kh * p.k_sh + dp * 8);
-      }
-      // dP^T = V dO^T with V fragments from global
-      f32x4 pacc[4];
-#pragma unroll
-      for (int jt = 0; jt < 4; jt++) {
-        pacc[jt] = f32x4{0.f, 0.f, 0.f, 0.f};
-        int kr = min(jt * 16 + l16, kmax);
-        const bf16_t* vp = p.v + (row0 + kr) * p.v_sr + (int64_t)kh * p.v_sh + kq * 8;
-#pragma unroll
-        for (int kc = 0; kc < VD / 32; kc++) pacc[jt] = mfma16(ld_global_b128(vp + kc * 32), dof[kc], pacc[jt]);
+        kr[j] = ld_global_b128(kb + (int64_t)min(pc / (D / 8), kmax) * p.k_sr + (pc % (D / 8)) * 8);
       }
 #pragma unroll
-      for (int j = 0; j < (D / 8); j++) {
+      for (int j = 0; j < VJ; j++) {
         int pc = lane + j * 64;
-        int kr = pc / (D / 8), dp = pc - kr * (D / 8);
-        *reinterpret_cast<bf16x8*>(&Ks[kr * KLD + dp * 8]) = kreg[j];
+        vr[j] = ld_global_b128(vb + (int64_t)min(pc / (VD / 8), kmax) * p.v_sr + (pc % (VD / 8)) * 8);
       }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+  };
+  auto compute = [&](int key0, bf16x8 (&kr)[KJ], bf16x8 (&vr)[VJ]) {
+    if (key0 < 0) return;
+#pragma unroll
+    for (int j = 0; j < KJ; j++) {
+      int pc = lane + j * 64;
+      *reinterpret_cast<bf16x8*>(&Ks[(pc / (D / 8)) * KLD + (pc % (D / 8)) * 8]) = kr[j];
+    }
+#pragma unroll
+    for (int j = 0; j < VJ; j++) {
+      int pc = lane + j * 64;
+      *reinterpret_cast<bf16x8*>(&Vs[(pc / (VD / 8)) * VLD + (pc % (VD / 8)) * 8]) = vr[j];
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    f32x4 sacc[2], pacc[2];
+#pragma unroll
+    for (int jt = 0; jt < 2; jt++) {
+      sacc[jt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      pacc[jt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const bf16_t* kp = &Ks[(jt * 16 + l16) * KLD + kq * 8];
+#pragma unroll
+      for (int kc = 0; kc < KC; kc++)
+        sacc[jt] = mfma16(*reinterpret_cast<const bf16x8*>(kp + kc * 32), qf[kc], sacc[jt]);
+      const bf16_t* vp = &Vs[(jt * 16 + l16) * VLD + kq * 8];
+#pragma unroll
+      for (int kc = 0; kc < VC; kc++)
+        pacc[jt] = mfma16(*reinterpret_cast<const bf16x8*>(vp + kc * 32), dof[kc], pacc[jt]);
+    }
+    const int kmax = key_last - key0;
+#pragma unroll
+    for (int jt = 0; jt < 2; jt++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) sacc[jt][i] = fast_exp2(__builtin_fmaf(sacc[jt][i], sc, -lse));
+    if (kmax < UK - 1) {  // wave-uniform
+#pragma unroll
+      for (int jt = 0; jt < 2; jt++)
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+          if (jt * 16 + kq * 4 + i > kmax) sacc[jt][i] = 0.f;
+    }
+#pragma unroll
+    for (int jt = 0; jt < 2; jt++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) sacc[jt][i] *= (pacc[jt][i] - delta);
+    bf16x8 df = pack8(sacc[0][0], sacc[0][1], sacc[0][2], sacc[0][3], sacc[1][0], sacc[1][1], sacc[1][2], sacc[1][3]);
+    const int kb0 = kq * 4 + (l16 >> 2);
+    const int kb1 = kb0 + 16;
+#pragma unroll
+    for (int dt = 0; dt < D / 16; dt++) {
+      const int col = dt * 16 + 4 * (l16 & 3);
+      bf16x4 a0 = lds_read_tr(&Ks[kb0 * KLD + col]);
+      bf16x4 a1 = lds_read_tr(&Ks[kb1 * KLD + col]);
+      dqacc[dt] = mfma16(cat4(a0, a1), df, dqacc[dt]);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  };
 
-      f32x4 sacc[4];
-#pragma unroll
-      for (int jt = 0; jt < 4; jt++) {
-        sacc[jt] = f32x4{0.f, 0.f, 0.f, 0.f};
-        const bf16_t* kp = &Ks[(jt * 16 + l16) * KLD + kq * 8];
-#pragma unroll
-        for (int kc = 0; kc < D / 32; kc++)
-          sacc[jt] = mfma16(*reinterpret_cast<const bf16x8*>(kp + kc * 32), qf[kc], sacc[jt]);
-      }
-#pragma unroll
-      for (int jt = 0; jt < 4; jt++)
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-          int ko = jt * 16 + kq * 4 + i;
-          float pv = ko <= kmax ? fast_exp2(sacc[jt][i] * sc - lse) : 0.f;
-          sacc[jt][i] = pv * (pacc[jt][i] - delta);
-        }
-#pragma unroll
-      for (int c = 0; c < 2; c++) {
-        bf16x8 df = pack8(sacc[2 * c][0], sacc[2 * c][1], sacc[2 * c][2], sacc[2 * c][3], sacc[2 * c + 1][0],
-                          sacc[2 * c + 1][1], sacc[2 * c + 1][2], sacc[2 * c + 1][3]);
-        const int kb0 = (2 * c) * 16 + kq * 4 + (l16 >> 2);
-        const int kb1 = kb0 + 16;
-#pragma unroll
-        for (int dt = 0; dt < D / 16; dt++) {
-          const int col = dt * 16 + 4 * (l16 & 3);
-          bf16x4 a0 = lds_read_tr(&Ks[kb0 * KLD + col]);
-          bf16x4 a1 = lds_read_tr(&Ks[kb1 * KLD + col]);
-          dqacc[dt] = mfma16(cat4(a0, a1), df, dqacc[dt]);
-        }
-      }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
+  bf16x8 krA[KJ], krB[KJ], vrA[VJ], vrB[VJ];
+  int keyA = 0, keyB = 0;
+  if (nu > 0) { keyA = unit_key0(0); issue(keyA, krA, vrA); }
+  for (int u = 0; u < nu; u += 2) {
+    if (u + 1 < nu) { keyB = unit_key0(u + 1); issue(keyB, krB, vrB); }
+    compute(keyA, krA, vrA);
+    if (u + 1 < nu) {
+      if (u + 2 < nu) { keyA = unit_key0(u + 2); issue(keyA, krA, vrA); }
+      compute(keyB, krB, vrB);
     }
   }
 
