@@ -204,3 +204,33 @@ def test_nsa_core_fwd_bwd(device, core, lens, QH, KH, D, methods):
         assert_close(wk.grad, wkr.grad, "dWk", atol=5e-2, rtol=2e-2, row_scale=True)
     if wv is not None:
         assert_close(wv.grad, wvr.grad, "dWv", atol=5e-2, rtol=2e-2, row_scale=True)
+
+
+def test_nsa_core_qk192_v128(device):
+    """Dqk = 192, Dv = 128 (the head shape upstream's inference notebook exercises), forward + backward."""
+    from flash_nsa import NSAConfig, NSACore
+    from flash_nsa.ops.compress_kv import mean_pooling_fwd
+    from flash_nsa.ops.compress_attn import cmp_attn_fwd
+    from flash_nsa.ops.topk import slc_topk_indices
+    lens, QH, KH, D, VD = [700, 333], 8, 2, 192, 128
+    cu = make_cu(lens)
+    T = int(cu[-1])
+    q, k, v, w = make_qkvw(T, QH, KH, D, VD, seed=80)
+    do = randn_bf16(T, QH, VD, seed=85)
+    cfg = NSAConfig(qk_head_dim=D, v_head_dim=VD, num_heads=QH, num_kv_heads=KH, top_n=6, window_size=100)
+    mod = NSACore(cfg)
+    qd, kd, vd, wd = [t.to(device).requires_grad_() for t in (q, k, v, w)]
+    out = mod(qd, kd, vd, wd, cu.to(device))
+    out.backward(do.to(device))
+    with torch.no_grad():
+        ck, cv = mean_pooling_fwd(kd.detach()), mean_pooling_fwd(vd.detach())
+        _, lse = cmp_attn_fwd(qd.detach(), ck, cv)
+        topk, _ = slc_topk_indices(qd.detach(), ck, lse)
+    qr, kr, vr, wr = leaf(q), leaf(k), leaf(v), leaf(w)
+    ro = O.nsa_forward(qr, kr, vr, wr, cu, O.OracleConfig(top_n=6, window_size=100), topk=topk.cpu())
+    ro.backward(do.float())
+    assert_close(out, ro, "o")
+    assert_close(qd.grad, qr.grad, "dq")
+    assert_close(kd.grad, kr.grad, "dk", row_scale=True)
+    assert_close(vd.grad, vr.grad, "dv", row_scale=True)
+    assert_close(wd.grad, wr.grad, "dw", atol=5e-2)

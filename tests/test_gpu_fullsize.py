@@ -1,0 +1,166 @@
+"""Full-size runs of the benchmark configurations, checked through properties that do not need the (dense, CPU)
+oracle at that size:
+  * causality / prefix consistency: the first rows of a long run equal a run on the prefix alone;
+  * packing invariance: a packed variable-length batch equals its sequences run one by one;
+  * decode: the fused decode step equals the stage-by-stage path and a single-request prefill of the last token;
+  * a slice of the full-size run (first tokens, where the oracle is affordable) against the oracle."""
+import pytest
+import torch
+
+from oracle import nsa_oracle as O
+from gpu_util import assert_close, make_cu
+
+pytestmark = pytest.mark.gpu
+
+
+def dev_randn(shape, seed, device):
+    g = torch.Generator(device=device).manual_seed(seed)
+    return torch.randn(*shape, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+
+
+def test_c2_prefix_consistency_and_oracle_slice(device):
+    """T = 65536, 64q/4kv heads, d = 128 (benchmark configuration): forward + backward run; the first 4096 rows of the
+    forward equal a 4096-token run (causality), and the first 1024 rows of kv group 0 match the oracle."""
+    from flash_nsa import NSAConfig, NSACore
+    T, QH, KH, D, P = 65536, 64, 4, 128, 4096
+    q, k, v, w = [dev_randn(s, i, device) for i, s in enumerate([(T, QH, D), (T, KH, D), (T, KH, D), (T, QH, 3)])]
+    core = NSACore(NSAConfig(head_dim=D, num_heads=QH, num_kv_heads=KH))
+    qg = q.clone().requires_grad_()
+    cu = torch.tensor([0, T], dtype=torch.int32, device=device)
+    out = core(qg, k, v, w, cu)
+    out.backward(dev_randn((T, QH, D), 9, device))
+    assert torch.isfinite(out).all() and torch.isfinite(qg.grad).all()
+    with torch.no_grad():
+        short = core(q[:P].contiguous(), k[:P].contiguous(), v[:P].contiguous(), w[:P].contiguous(),
+                     torch.tensor([0, P], dtype=torch.int32, device=device))
+    assert torch.equal(out[:P], short), "rows of the prefix changed when later tokens were appended"
+    # oracle on a slice: first 1024 tokens, the 16 q-heads of kv head 0, device's own block selection
+    n = 1024
+    from flash_nsa import NSAHelper
+    from flash_nsa.ops.compress_kv import mean_pooling_fwd
+    from flash_nsa.ops.compress_attn import cmp_attn_fwd
+    from flash_nsa.ops.topk import slc_topk_indices
+    cun = torch.tensor([0, n], dtype=torch.int32, device=device)
+    qs, ks, vs, ws = q[:n, :16].contiguous(), k[:n, :1].contiguous(), v[:n, :1].contiguous(), w[:n, :16].contiguous()
+    with torch.no_grad():
+        core16 = NSACore(NSAConfig(head_dim=D, num_heads=16, num_kv_heads=1))
+        o16 = core16(qs, ks, vs, ws, cun)
+        ck, cv = mean_pooling_fwd(ks), mean_pooling_fwd(vs)
+        _, lse = cmp_attn_fwd(qs, ck, cv)
+        topk, _ = slc_topk_indices(qs, ck, lse)
+    assert torch.equal(o16, out[:n, :16]), "a kv group computed alone differs from the same group inside 4 groups"
+    ref = O.nsa_forward(qs.float().cpu(), ks.float().cpu(), vs.float().cpu(), ws.float().cpu(), [0, n],
+                        topk=topk.cpu(), round_dtype=torch.bfloat16)
+    assert_close(o16, ref, "o (slice of the 64K run)")
+
+
+def test_c3_packed_batch_equals_single_sequences(device):
+    """8 sequences with lengths uniform in [4096, 8192] (seed 1), forward + backward: packed == one by one."""
+    from flash_nsa import NSAConfig, NSACore
+    g = torch.Generator().manual_seed(1)
+    lens = torch.randint(4096, 8193, (8,), generator=g).tolist()
+    cu = make_cu(lens)
+    T, QH, KH, D = int(cu[-1]), 64, 4, 128
+    q, k, v, w, do = [dev_randn(s, 10 + i, device) for i, s in
+                      enumerate([(T, QH, D), (T, KH, D), (T, KH, D), (T, QH, 3), (T, QH, D)])]
+    core = NSACore(NSAConfig(head_dim=D, num_heads=QH, num_kv_heads=KH))
+
+    def run(qq, kk, vv, ww, dd, cuu):
+        ts = [t.clone().requires_grad_() for t in (qq, kk, vv, ww)]
+        o = core(*ts, cuu.to(device))
+        o.backward(dd)
+        return [o.detach()] + [t.grad for t in ts]
+
+    packed = run(q, k, v, w, do, cu)
+    for b in (0, 3, 7):
+        a, e = int(cu[b]), int(cu[b + 1])
+        single = run(q[a:e], k[a:e], v[a:e], w[a:e], do[a:e], make_cu([e - a]))
+        assert torch.equal(packed[0][a:e], single[0]), f"sequence {b}: forward differs"
+        assert torch.equal(packed[1][a:e], single[1]), f"sequence {b}: dq differs"
+        # dk/dv are accumulated with fp32 atomics in a data-dependent order: equal up to fp32 summation order
+        assert_close(packed[2][a:e], single[2], f"sequence {b}: dk", atol=2e-3, rtol=2e-3, row_scale=True)
+        assert_close(packed[3][a:e], single[3], f"sequence {b}: dv", atol=2e-3, rtol=2e-3, row_scale=True)
+        assert_close(packed[4][a:e], single[4], f"sequence {b}: dw", atol=1e-6, rtol=0)
+
+
+def test_c5_decode_full_batch(device):
+    """Batch 64, contexts uniform in [4096, 32768], page 256, random page permutation (benchmark configuration):
+    fused decode == stage-by-stage decode; one request re-checked as a one-token paged prefill; graph replay."""
+    import sys, os
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    import bench_decode as bd
+    from flash_nsa import nsa_decode, nsa_prefill
+    from flash_nsa.inference import nsa_decode_staged, mean_pooling_prefill
+    c = bd.build_case(device)
+    page = c["page"]
+    ycu = torch.zeros(65, dtype=torch.int32)
+    ycu[1:] = torch.cumsum(torch.tensor(c["ys"]), 0)
+    slots_all = torch.cat([(c["cbt"][b].cpu()[torch.arange(y) // page].to(torch.int64) * page + torch.arange(y) % page)
+                           for b, y in enumerate(c["ys"])]).to(torch.int32).to(device)
+    for cache in (c["k"], c["v"]):
+        mean_pooling_prefill(cache, ycu.to(device), max(c["ys"]), c["bt"], slots_all)
+    kw = dict(fixed_y_maxlen=2048, fixed_num_slc_blocks=512)
+    fused = nsa_decode(c["q"], c["k"], c["v"], c["w"], c["ctx"], c["bt"], c["slots"], c["cbt"], **kw)
+    staged = nsa_decode_staged(c["q"], c["k"], c["v"], c["w"], c["ctx"], c["bt"], c["cbt"], **kw)
+    assert torch.isfinite(fused).all()
+    assert_close(fused, staged, "fused vs staged decode", atol=8e-3, rtol=1e-2)
+    split = nsa_decode(c["q"], c["k"], c["v"], c["w"], c["ctx"], c["bt"], c["slots"], c["cbt"], cmp_num_splits=4, **kw)
+    assert_close(split, staged, "split vs staged decode", atol=8e-3, rtol=1e-2)
+    # request 5 as a single-token prefill through nsa_prefill (all compressed rows already pooled: slots -1)
+    b = 5
+    L, y = c["lens"][b], c["ys"][b]
+    o1 = nsa_prefill(c["q"][b:b + 1], c["k"], c["v"], c["w"][b:b + 1], torch.tensor([0, 1], dtype=torch.int32, device=device),
+                     torch.tensor([0, y], dtype=torch.int32, device=device), 1, y, c["ctx"][b:b + 1], c["bt"][b:b + 1],
+                     torch.full((y,), -1, dtype=torch.int32, device=device), c["cbt"][b:b + 1], **kw)
+    assert_close(fused[b:b + 1], o1, "decode vs one-token prefill", atol=8e-3, rtol=1e-2)
+
+
+def test_c4_chunked_prefill_full_size(device):
+    """16 requests, cached prefix uniform in [0, 16384] + a new chunk of 2048 tokens, page 256, random page
+    permutation (benchmark configuration): the chunk's output equals the training forward on the gathered
+    contiguous sequence (rows of the chunk), and the pooled rows equal the contiguous pooling bit for bit."""
+    from flash_nsa import NSAConfig, NSACore, nsa_prefill, NSAHelper
+    from flash_nsa.inference import mean_pooling_prefill
+    from flash_nsa.ops.compress_kv import mean_pooling_fwd
+    from paged_util import build_pool, prefill_slot_mapping
+    QH, KH, D, page, chunk = 64, 4, 128, 256, 2048
+    g = torch.Generator().manual_seed(2)
+    cached = torch.randint(0, 16385, (16,), generator=g).tolist()
+    ctx = [c + chunk for c in cached]
+    case = build_pool(ctx, KH, D, D, page=page, seed=2)
+    d = {k_: (v_.to(device) if isinstance(v_, torch.Tensor) else v_) for k_, v_ in case.items()}
+    # an earlier step pooled the rows that lie inside the cached prefix
+    pre = dict(case)
+    pre["ctx"] = cached
+    pre["ys"] = [max((L - 32) // 16 + 1, 0) for L in cached]
+    slots0, ycu0 = prefill_slot_mapping(pre, [0] * 16)
+    cached_t = torch.tensor(cached, dtype=torch.int32, device=device)
+    if int(ycu0[-1]) > 0:
+        for cache in (d["k"], d["v"]):
+            mean_pooling_prefill(cache, ycu0.to(device), max(pre["ys"]), d["bt"], slots0.to(device))
+    slots, ycu = prefill_slot_mapping(case, cached)
+    xcu = make_cu([chunk] * 16)
+    t = 16 * chunk
+    q, w = dev_randn((t, QH, D), 31, device), dev_randn((t, QH, 3), 32, device)
+    ctx_t = torch.tensor(ctx, dtype=torch.int32, device=device)
+    o = nsa_prefill(q, d["k"], d["v"], w, xcu.to(device), ycu.to(device), chunk, max(case["ys"]), ctx_t, d["bt"],
+                    slots.to(device), d["cbt"], fixed_y_maxlen=2048, fixed_num_slc_blocks=512)
+    assert torch.isfinite(o).all()
+    core = NSACore(NSAConfig(head_dim=D, num_heads=QH, num_kv_heads=KH))
+    kc, vc = d["k"].cpu(), d["v"].cpu()
+    for b in (0, 7, 15):
+        L = ctx[b]
+        ks = O.gather_rows(kc, case["bt"][b], L).to(device)
+        vs = O.gather_rows(vc, case["bt"][b], L).to(device)
+        qf = dev_randn((L, QH, D), 40 + b, device)
+        wf = dev_randn((L, QH, 3), 50 + b, device)
+        qf[-chunk:] = q[b * chunk:(b + 1) * chunk]
+        wf[-chunk:] = w[b * chunk:(b + 1) * chunk]
+        cu1 = torch.tensor([0, L], dtype=torch.int32, device=device)
+        with torch.no_grad():
+            full = core(qf, ks, vs, wf, cu1)
+            ck = mean_pooling_fwd(ks)
+        assert_close(o[b * chunk:(b + 1) * chunk], full[-chunk:], f"request {b}: chunk vs contiguous forward",
+                     atol=4e-3, rtol=1e-2)
+        pooled = O.gather_rows(kc * 0 + d["k"].cpu(), case["cbt"][b], case["ys"][b])
+        assert torch.equal(pooled, ck.cpu()), f"request {b}: pooled rows differ from contiguous pooling"
