@@ -82,6 +82,18 @@ NSA_DEVICE bf16x8 cat4(bf16x4 a, bf16x4 b) {
   return __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
+// exchange between the two 32-lane halves of a wave on the VALU (v_permlane32_swap), no LDS crossbar round trip
+NSA_DEVICE float xhalf_max(float v) {
+  uint32_t b = __builtin_bit_cast(uint32_t, v);
+  auto r = __builtin_amdgcn_permlane32_swap(b, b, false, false);
+  return fmaxf(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1]));
+}
+NSA_DEVICE float xhalf_sum(float v) {
+  uint32_t b = __builtin_bit_cast(uint32_t, v);
+  auto r = __builtin_amdgcn_permlane32_swap(b, b, false, false);
+  return __builtin_bit_cast(float, (uint32_t)r[0]) + __builtin_bit_cast(float, (uint32_t)r[1]);
+}
+
 NSA_DEVICE float wave_max(float v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));

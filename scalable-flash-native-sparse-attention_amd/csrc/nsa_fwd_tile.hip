@@ -172,7 +172,7 @@ __global__ __launch_bounds__(256, MINB) void fwd_tile_kernel(NsaFwdTileParams p)
     for (int nt = 0; nt < 2; nt++)
 #pragma unroll
       for (int i = 0; i < 16; i++) tmax = fmaxf(tmax, sacc[nt][i]);
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    tmax = xhalf_max(tmax);
     const float m_old = m_run[rs];
     const float m_new = fmaxf(m_old, tmax);
     const float m_safe = (m_new == NSA_NEG_INF) ? 0.f : m_new;
@@ -250,7 +250,7 @@ __global__ __launch_bounds__(256, MINB) void fwd_tile_kernel(NsaFwdTileParams p)
   // ---- epilogue ----
 #pragma unroll
   for (int rs = 0; rs < RS; rs++) {
-    float l_tot = l_run[rs] + __shfl_xor(l_run[rs], 32, 64);
+    float l_tot = xhalf_sum(l_run[rs]);
     if (!valid[rs]) continue;
     float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     bf16_t* op = p.o + tok[rs] * p.o_st + (int64_t)head[rs] * p.o_sh;
