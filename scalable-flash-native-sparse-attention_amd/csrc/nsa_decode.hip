@@ -20,24 +20,38 @@ constexpr int DEC_WAVES = 8;
 constexpr int UK = 32;  // keys per unit
 
 // One wave's flash-attention state over units of 32 keys for the 16 heads of a kv group.
+// K and V rows of a unit are fetched as whole rows (16 lanes x 16 bytes per row: every cache line is requested once
+// and used completely), held in registers while the previous unit is computed, and pass through one wave-private
+// LDS slot: first the K rows (read back as MFMA A fragments), then the V rows (read back transposed).
+// With KEEP the un-normalised probabilities exp2((s - m_unit) * c) of every unit are kept in LDS as fp16 together
+// with the m_unit they refer to, so that the importance pass needs no second pass over the keys.
 template <int D, int VD>
 struct UnitFlash {
   static constexpr int KC = D / 32;
+  static constexpr int KJ = (UK * (D / 8)) / 64;
   static constexpr int VJ = (UK * (VD / 8)) / 64;
+  static constexpr int KLD = D + NSA_LDS_PAD;
   static constexpr int VLD = VD + NSA_LDS_PAD;
+  static constexpr int SLOT = UK * (KLD > VLD ? KLD : VLD);  // bf16 elements of a wave's staging slot
   bf16x8 qf[KC];
   f32x4 oacc[VD / 16];
   float m_run, l_run;
   float sc;
   int l16, kq, lane;
-  bf16_t* Vs;  // wave-private [UK][VLD]
+  bf16_t* Ss;          // wave-private staging slot
+  _Float16* keep_p;    // [16][keep_ld] or null
+  float* keep_m;       // [units][16]
+  int keep_ld;
 
-  NSA_DEVICE void init(const bf16_t* qrow, float scale_log2, int lane_, bf16_t* vs) {
+  NSA_DEVICE void init(const bf16_t* qrow, float scale_log2, int lane_, bf16_t* slot) {
     lane = lane_;
     l16 = lane & 15;
     kq = lane >> 4;
     sc = scale_log2;
-    Vs = vs;
+    Ss = slot;
+    keep_p = nullptr;
+    keep_m = nullptr;
+    keep_ld = 0;
 #pragma unroll
     for (int kc = 0; kc < KC; kc++) qf[kc] = ld_global_b128(qrow + kq * 8 + kc * 32);
 #pragma unroll
@@ -45,37 +59,55 @@ struct UnitFlash {
     m_run = NSA_NEG_INF;
     l_run = 0.f;
   }
-  // loads of the unit starting at key0; keys outside [klo, khi] are replaced by a clamped key (masked later)
-  template <class RowFn>
-  NSA_DEVICE void issue(int key0, int klo, int khi, RowFn row_of_key, const bf16_t* kbase, int64_t k_sr,
-                        const bf16_t* vbase, int64_t v_sr, bf16x8 (&kf)[2][KC], bf16x8 (&vr)[VJ]) {
+  // loads of the unit starting at key0 (wave-uniform); keys outside [klo, khi] are replaced by a clamped key
+  // (masked later).  A unit spans at most two pages: the page of its first usable key is looked up once.
+  NSA_DEVICE void issue(int key0, int klo, int khi, const int* tab_s, int page, const bf16_t* kbase, int64_t k_sr,
+                        const bf16_t* vbase, int64_t v_sr, bf16x8 (&kf)[KJ], bf16x8 (&vr)[VJ]) {
+    const int ks = __builtin_amdgcn_readfirstlane(max(klo, min(key0, khi)));
+    const int pi = ks / page;
+    const int rem0 = ks - pi * page;
+    const int64_t base0 = (int64_t)tab_s[pi] * page;
+    const int64_t base1 = (rem0 + UK > page && (int64_t)(pi + 1) * page <= khi) ? (int64_t)tab_s[pi + 1] * page - page : base0;
 #pragma unroll
-    for (int jt = 0; jt < 2; jt++) {
-      int key = max(klo, min(key0 + jt * 16 + l16, khi));
-      const bf16_t* kp = kbase + row_of_key(key) * k_sr + kq * 8;
-#pragma unroll
-      for (int kc = 0; kc < KC; kc++) kf[jt][kc] = ld_global_b128(kp + kc * 32);
+    for (int j = 0; j < KJ; j++) {
+      int pc = lane + j * 64;
+      int r = rem0 + max(klo, min(key0 + pc / (D / 8), khi)) - ks;
+      int64_t row = (r >= page ? base1 : base0) + r;
+      kf[j] = ld_global_b128(kbase + row * k_sr + (pc % (D / 8)) * 8);
     }
 #pragma unroll
     for (int j = 0; j < VJ; j++) {
       int pc = lane + j * 64;
-      int kr = pc / (VD / 8), dp = pc % (VD / 8);
-      int key = max(klo, min(key0 + kr, khi));
-      vr[j] = ld_global_b128(vbase + row_of_key(key) * v_sr + dp * 8);
+      int r = rem0 + max(klo, min(key0 + pc / (VD / 8), khi)) - ks;
+      int64_t row = (r >= page ? base1 : base0) + r;
+      vr[j] = ld_global_b128(vbase + row * v_sr + (pc % (VD / 8)) * 8);
     }
   }
-  NSA_DEVICE void compute(int key0, int klo, int khi, bf16x8 (&kf)[2][KC], bf16x8 (&vr)[VJ]) {
+  NSA_DEVICE void compute(int key0, int klo, int khi, bf16x8 (&kf)[KJ], bf16x8 (&vr)[VJ]) {
+#pragma unroll
+    for (int j = 0; j < KJ; j++) {
+      int pc = lane + j * 64;
+      *reinterpret_cast<bf16x8*>(&Ss[(pc / (D / 8)) * KLD + (pc % (D / 8)) * 8]) = kf[j];
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     f32x4 sacc[2];
 #pragma unroll
     for (int jt = 0; jt < 2; jt++) {
       sacc[jt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const bf16_t* kp = &Ss[(jt * 16 + l16) * KLD + kq * 8];
 #pragma unroll
-      for (int kc = 0; kc < KC; kc++) sacc[jt] = mfma16(kf[jt][kc], qf[kc], sacc[jt]);
+      for (int kc = 0; kc < KC; kc++)
+        sacc[jt] = mfma16(*reinterpret_cast<const bf16x8*>(kp + kc * 32), qf[kc], sacc[jt]);
     }
+    // the K fragments are consumed (LDS operations of a wave complete in order): the slot now takes the V rows
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int j = 0; j < VJ; j++) {
       int pc = lane + j * 64;
-      *reinterpret_cast<bf16x8*>(&Vs[(pc / (VD / 8)) * VLD + (pc % (VD / 8)) * 8]) = vr[j];
+      *reinterpret_cast<bf16x8*>(&Ss[(pc / (VD / 8)) * VLD + (pc % (VD / 8)) * 8]) = vr[j];
     }
     if (key0 < klo || key0 + UK - 1 > khi) {  // wave-uniform: only boundary units are masked
 #pragma unroll
@@ -89,7 +121,7 @@ struct UnitFlash {
     float tmax = fmaxf(fmaxf(fmaxf(sacc[0][0], sacc[0][1]), fmaxf(sacc[0][2], sacc[0][3])),
                        fmaxf(fmaxf(sacc[1][0], sacc[1][1]), fmaxf(sacc[1][2], sacc[1][3])));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    tmax = xhalf_max(tmax);
     const float m_old = m_run;
     const float m_new = fmaxf(m_old, tmax);
     const float m_safe = (m_new == NSA_NEG_INF) ? 0.f : m_new;
@@ -104,6 +136,15 @@ struct UnitFlash {
         sacc[jt][i] = pv;
         psum += pv;
       }
+    if (keep_p != nullptr) {
+      typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+      for (int jt = 0; jt < 2; jt++) {
+        h4 hv = {(_Float16)sacc[jt][0], (_Float16)sacc[jt][1], (_Float16)sacc[jt][2], (_Float16)sacc[jt][3]};
+        *reinterpret_cast<h4*>(&keep_p[l16 * keep_ld + key0 + jt * 16 + kq * 4]) = hv;
+      }
+      if (kq == 0) keep_m[(key0 / UK) * 16 + l16] = m_safe;
+    }
     if (__builtin_amdgcn_ballot_w64(m_new != m_old) != 0) {
       const float alpha = fast_exp2((m_old - m_safe) * sc);
       l_run *= alpha;
@@ -120,28 +161,28 @@ struct UnitFlash {
 #pragma unroll
     for (int dt = 0; dt < VD / 16; dt++) {
       const int col = dt * 16 + 4 * (l16 & 3);
-      bf16x4 v0 = lds_read_tr(&Vs[kb0 * VLD + col]);
-      bf16x4 v1 = lds_read_tr(&Vs[kb1 * VLD + col]);
+      bf16x4 v0 = lds_read_tr(&Ss[kb0 * VLD + col]);
+      bf16x4 v1 = lds_read_tr(&Ss[kb1 * VLD + col]);
       oacc[dt] = mfma16(cat4(v0, v1), pf, oacc[dt]);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
   }
   // pipelined loop over units u = first, first+step, ... < nu ; key0_of(u) gives the unit's first key
-  template <class KeyFn, class RowFn>
-  NSA_DEVICE void run(int first, int step, int nu, int klo, int khi, KeyFn key0_of, RowFn row_of_key,
+  template <class KeyFn>
+  NSA_DEVICE void run(int first, int step, int nu, int klo, int khi, KeyFn key0_of, const int* tab_s, int page,
                       const bf16_t* kbase, int64_t k_sr, const bf16_t* vbase, int64_t v_sr) {
-    bf16x8 kfA[2][KC], kfB[2][KC], vrA[VJ], vrB[VJ];
+    bf16x8 kfA[KJ], kfB[KJ], vrA[VJ], vrB[VJ];
     int keyA = 0, keyB = 0;
-    if (first < nu) { keyA = key0_of(first); issue(keyA, klo, khi, row_of_key, kbase, k_sr, vbase, v_sr, kfA, vrA); }
+    if (first < nu) { keyA = key0_of(first); issue(keyA, klo, khi, tab_s, page, kbase, k_sr, vbase, v_sr, kfA, vrA); }
     for (int u = first; u < nu; u += 2 * step) {
       const bool hasB = u + step < nu;
-      if (hasB) { keyB = key0_of(u + step); issue(keyB, klo, khi, row_of_key, kbase, k_sr, vbase, v_sr, kfB, vrB); }
+      if (hasB) { keyB = key0_of(u + step); issue(keyB, klo, khi, tab_s, page, kbase, k_sr, vbase, v_sr, kfB, vrB); }
       compute(keyA, klo, khi, kfA, vrA);
       if (hasB) {
         if (u + 2 * step < nu) {
           keyA = key0_of(u + 2 * step);
-          issue(keyA, klo, khi, row_of_key, kbase, k_sr, vbase, v_sr, kfA, vrA);
+          issue(keyA, klo, khi, tab_s, page, kbase, k_sr, vbase, v_sr, kfA, vrA);
         }
         compute(keyB, klo, khi, kfB, vrB);
       }
@@ -150,7 +191,7 @@ struct UnitFlash {
   // wave partial -> LDS slot: m (raw units), l, o[16 heads][VD]
   NSA_DEVICE void publish(float* pm, float* pl, float* po) {
     float l_tot = l_run + __shfl_xor(l_run, 16, 64);
-    l_tot += __shfl_xor(l_tot, 32, 64);
+    l_tot = xhalf_sum(l_tot);
     if (kq == 0) { pm[l16] = m_run; pl[l16] = l_tot; }
 #pragma unroll
     for (int dt = 0; dt < VD / 16; dt++)
@@ -178,21 +219,29 @@ NSA_DEVICE float merge_partials(const float* pm, const float* pl, const float* p
   return l > 0.f ? o / l : 0.f;
 }
 
-template <int D, int VD>
+template <int D, int VD, bool KEEP>
 __global__ __launch_bounds__(DEC_WAVES * 64) void decode_cmp_topk_kernel(NsaDecodeParams p) {
   using UF = UnitFlash<D, VD>;
   constexpr int NW = DEC_WAVES;
-  // dynamic LDS: [V staging, one slot per wave (reused for the wave's partial o)] [m][l][lse] [pg] [imp]
+  // dynamic LDS: [staging slot per wave (reused for the wave's partial o, then for pg)] [m][l][lse] [imp] [table]
+  //              KEEP: [un-normalised p, fp16 [16][keep_ld]] [m of every unit [units][16]]
+  //              else: [pg]
   extern __shared__ __attribute__((aligned(16))) unsigned char dyn_raw[];
-  constexpr int SLOT = UK * UF::VLD;  // bf16 elements per wave slot (>= 16*VD floats)
-  static_assert(SLOT * 2 >= 16 * VD * 4, "a wave's V slot must hold its partial output");
+  constexpr int SLOT = UF::SLOT;
+  static_assert(SLOT * 2 >= 16 * VD * 4, "a wave's slot must hold its partial output");
   bf16_t* Vs_all = reinterpret_cast<bf16_t*>(dyn_raw);
   float* part_m = reinterpret_cast<float*>(dyn_raw + (size_t)NW * SLOT * 2);
   float* part_l = part_m + NW * 16;
   float* lse_s = part_l + NW * 16;
-  float* pg = lse_s + 16;
-  float* imp = pg + p.y_cap;
+  float* imp = lse_s + 16;
   int* tab_s = reinterpret_cast<int*>(imp + p.nb_cap);  // the request's compressed-row page table
+  const int ntab = (p.y_cap + p.page_size - 1) / p.page_size;
+  const int n_units_cap = (p.y_cap + UK - 1) / UK;
+  const int keep_ld = n_units_cap * UK + 8;  // +8 halves: the 16 head rows start in different banks
+  float* after_tab = reinterpret_cast<float*>(tab_s + ((ntab + 3) & ~3));
+  float* keep_m = after_tab;                                               // KEEP
+  _Float16* keep_p = reinterpret_cast<_Float16*>(keep_m + n_units_cap * 16);  // KEEP
+  float* pg = KEEP ? reinterpret_cast<float*>(dyn_raw) : after_tab;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -209,7 +258,6 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_cmp_topk_kernel(NsaDeco
   // the pipelined K/V loads behind it (memory operations of a wave retire in order)
   for (int i = tid; i < (y + page - 1) / page; i += NW * 64) tab_s[i] = ctab[i];
   __syncthreads();
-  auto row_of = [&](int key) -> int64_t { return (int64_t)tab_s[key / page] * page + (key % page); };
   const bf16_t* kbase = p.k + (int64_t)kh * p.k_sh;
   const bf16_t* vbase = p.v + (int64_t)kh * p.v_sh;
   const int l16 = lane & 15, kq = lane >> 4;
@@ -217,13 +265,17 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_cmp_topk_kernel(NsaDeco
   const int head = kh * G + g;
 
   UF uf;
-  uf.init(p.q + (int64_t)b * p.q_st + (int64_t)head * p.q_sh, p.scale_log2, lane, Vs_all + wave * UK * UF::VLD);
+  uf.init(p.q + (int64_t)b * p.q_st + (int64_t)head * p.q_sh, p.scale_log2, lane, Vs_all + wave * SLOT);
+  if (KEEP) {
+    uf.keep_p = keep_p;
+    uf.keep_m = keep_m;
+    uf.keep_ld = keep_ld;
+  }
   const int nu = (y + UK - 1) / UK;
 
   // ---- phase A: compressed attention, units dealt round-robin to the waves ----
-  uf.run(wave, NW, nu, 0, y - 1, [&](int u) { return u * UK; }, row_of, kbase, p.k_sr, vbase, p.v_sr);
+  uf.run(wave, NW, nu, 0, y - 1, [&](int u) { return u * UK; }, tab_s, page, kbase, p.k_sr, vbase, p.v_sr);
   uf.publish(part_m + wave * 16, part_l + wave * 16, reinterpret_cast<float*>(Vs_all + wave * SLOT));
-  for (int i = tid; i < p.y_cap; i += NW * 64) pg[i] = 0.f;
   __syncthreads();
   for (int idx = tid; idx < 16 * VD; idx += NW * 64) {
     int h = idx / VD, d = idx - h * VD;
@@ -243,8 +295,23 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_cmp_topk_kernel(NsaDeco
   __syncthreads();
 
   // ---- phase B: p = exp2(s*c - lse) summed over the heads of the group, per compressed key ----
-  {
-    // S[head][key] = Q K^T : lane holds key = l16, heads kq*4 .. +3
+  if (KEEP) {
+    // p = kept exp2((s - m_unit)*c) * exp2(m_unit*c - lse): turn the m table into these factors, then one thread per key
+    for (int i = tid; i < nu * 16; i += NW * 64) {
+      int h = i & 15;
+      keep_m[i] = h < G ? fast_exp2(__builtin_fmaf(keep_m[i], p.scale_log2, -lse_s[h])) : 0.f;
+    }
+    __syncthreads();
+    for (int key = tid; key < y; key += NW * 64) {
+      const float* fac = keep_m + (key / UK) * 16;
+      float acc = 0.f;
+#pragma unroll
+      for (int h = 0; h < 16; h++) acc += (float)keep_p[h * keep_ld + key] * fac[h];
+      pg[key] = acc;
+    }
+  } else {
+    // second pass over the compressed keys: S[head][key] = Q K^T, lane holds key = l16, heads kq*4 .. +3
+    auto row_of = [&](int key) -> int64_t { return (int64_t)tab_s[key / page] * page + (key % page); };
     float lse4[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) lse4[i] = lse_s[kq * 4 + i];
@@ -344,7 +411,7 @@ template <int D, int VD>
 __global__ __launch_bounds__(SPLIT_WAVES * 64) void decode_cmp_partial_kernel(NsaDecodeParams p) {
   using UF = UnitFlash<D, VD>;
   constexpr int NW = SPLIT_WAVES;
-  constexpr int SLOT = UK * UF::VLD;
+  constexpr int SLOT = UF::SLOT;
   extern __shared__ __attribute__((aligned(16))) unsigned char dyn_raw[];
   bf16_t* Vs_all = reinterpret_cast<bf16_t*>(dyn_raw);
   float* part_m = reinterpret_cast<float*>(dyn_raw + (size_t)NW * SLOT * 2);
@@ -363,7 +430,6 @@ __global__ __launch_bounds__(SPLIT_WAVES * 64) void decode_cmp_partial_kernel(Ns
   const int page = p.page_size;
   for (int i = tid; i < (y + page - 1) / page; i += NW * 64) tab_s[i] = ctab[i];
   __syncthreads();
-  auto row_of = [&](int key) -> int64_t { return (int64_t)tab_s[key / page] * page + (key % page); };
   const bf16_t* kbase = p.k + (int64_t)kh * p.k_sh;
   const bf16_t* vbase = p.v + (int64_t)kh * p.v_sh;
   const int l16 = lane & 15;
@@ -372,8 +438,8 @@ __global__ __launch_bounds__(SPLIT_WAVES * 64) void decode_cmp_partial_kernel(Ns
   UF uf;
   uf.init(p.q + (int64_t)b * p.q_st + (int64_t)head * p.q_sh, p.scale_log2, lane, Vs_all + wave * SLOT);
   const int nu = (y + UK - 1) / UK;
-  uf.run(sp * NW + wave, NW * nsplit, nu, 0, y - 1, [&](int u) { return u * UK; }, row_of, kbase, p.k_sr, vbase,
-         p.v_sr);
+  uf.run(sp * NW + wave, NW * nsplit, nu, 0, y - 1, [&](int u) { return u * UK; }, tab_s, page, kbase, p.k_sr,
+         vbase, p.v_sr);
   uf.publish(part_m + wave * 16, part_l + wave * 16, reinterpret_cast<float*>(Vs_all + wave * SLOT));
   __syncthreads();
   // merge the 4 waves; store the split's un-normalised partial
@@ -510,8 +576,8 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecod
   constexpr int NW = DEC_WAVES;
   constexpr int NW_SLC = 5;  // waves on the selected blocks, the rest on the window
   extern __shared__ __attribute__((aligned(16))) unsigned char dyn_raw[];
-  constexpr int SLOT = UK * UF::VLD;
-  static_assert(SLOT * 2 >= 16 * VD * 4, "a wave's V slot must hold its partial output");
+  constexpr int SLOT = UF::SLOT;
+  static_assert(SLOT * 2 >= 16 * VD * 4, "a wave's slot must hold its partial output");
   bf16_t* Vs_all = reinterpret_cast<bf16_t*>(dyn_raw);
   float* part_m = reinterpret_cast<float*>(dyn_raw + (size_t)NW * SLOT * 2);
   float* part_l = part_m + NW * 16;
@@ -528,7 +594,6 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecod
   const int32_t* tab = p.table + (int64_t)b * p.table_stride;
   const int page = p.page_size;
   for (int i = tid; i < (L + page - 1) / page; i += NW * 64) tab_s[i] = tab[i];
-  auto row_of = [&](int key) -> int64_t { return (int64_t)tab_s[key / page] * page + (key % page); };
   const bf16_t* kbase = p.k + (int64_t)kh * p.k_sh;
   const bf16_t* vbase = p.v + (int64_t)kh * p.v_sh;
   const int l16 = lane & 15;
@@ -601,18 +666,18 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecod
   __syncthreads();
 
   UF uf;
-  uf.init(p.q + (int64_t)b * p.q_st + (int64_t)head * p.q_sh, p.scale_log2, lane, Vs_all + wave * UK * UF::VLD);
+  uf.init(p.q + (int64_t)b * p.q_st + (int64_t)head * p.q_sh, p.scale_log2, lane, Vs_all + wave * SLOT);
   if (t >= 0) {
     if (wave < NW_SLC) {
       const int upb = Bs / UK;
       uf.run(wave, NW_SLC, nvalid * upb, 0, t,
-             [&](int u) { int slot = u / upb; return max(blk_s[slot], 0) * Bs + (u - slot * upb) * UK; }, row_of,
+             [&](int u) { int slot = u / upb; return max(blk_s[slot], 0) * Bs + (u - slot * upb) * UK; }, tab_s, page,
              kbase, p.k_sr, vbase, p.v_sr);
     } else {
       const int klo = max(0, t - p.window);
       const int k0 = (klo / UK) * UK;
       const int nu = (t - k0) / UK + 1;
-      uf.run(wave - NW_SLC, NW - NW_SLC, nu, klo, t, [&](int u) { return k0 + u * UK; }, row_of, kbase, p.k_sr,
+      uf.run(wave - NW_SLC, NW - NW_SLC, nu, klo, t, [&](int u) { return k0 + u * UK; }, tab_s, page, kbase, p.k_sr,
              vbase, p.v_sr);
     }
   }
@@ -660,19 +725,33 @@ static int launch_dyn(K kern, dim3 grid, size_t dyn, const NsaDecodeParams& p, h
 }
 
 template <int D, int VD>
-static size_t slot_bytes() { return (size_t)DEC_WAVES * UK * (VD + NSA_LDS_PAD) * 2; }
+static size_t slot_bytes() { return (size_t)DEC_WAVES * UnitFlash<D, VD>::SLOT * 2; }
+
+// LDS of the fused compressed-attention + selection kernel; `keep` adds the fp16 probabilities of every compressed
+// key and the per-unit maxima (no second pass over the keys) and drops the separate pg array
+static size_t cmp_topk_lds(size_t slots, const NsaDecodeParams& p, bool keep) {
+  const size_t ntab = (size_t)(p.y_cap + p.page_size - 1) / p.page_size;
+  const size_t units = (size_t)(p.y_cap + UK - 1) / UK;
+  size_t n = slots + (size_t)(2 * DEC_WAVES * 16 + 16 + p.nb_cap + ((ntab + 3) & ~(size_t)3)) * sizeof(float);
+  if (keep) n += units * 16 * sizeof(float) + 16 * (units * UK + 8) * sizeof(_Float16);
+  else n += (size_t)p.y_cap * sizeof(float);
+  return n;
+}
+
+template <int D, int VD>
+static int launch_cmp_topk(const NsaDecodeParams& p, dim3 grid, hipStream_t stream) {
+  const size_t keep_bytes = cmp_topk_lds(slot_bytes<D, VD>(), p, true);
+  if (keep_bytes <= 160 * 1024)
+    return launch_dyn(decode_cmp_topk_kernel<D, VD, true>, grid, keep_bytes, p, stream, "decode_cmp_topk_kernel");
+  return launch_dyn(decode_cmp_topk_kernel<D, VD, false>, grid, cmp_topk_lds(slot_bytes<D, VD>(), p, false), p, stream,
+                    "decode_cmp_topk_kernel");
+}
 
 int nsa_decode_cmp_topk_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream) {
   if (B <= 0) return NSA_OK;
   dim3 grid(B, p.KH);
-  size_t extra = (size_t)(2 * DEC_WAVES * 16 + 16 + p.y_cap + p.nb_cap + (p.y_cap + p.page_size - 1) / p.page_size) *
-                 sizeof(float);
-  if (D == 128 && VD == 128)
-    return launch_dyn(decode_cmp_topk_kernel<128, 128>, grid, slot_bytes<128, 128>() + extra, p, stream,
-                      "decode_cmp_topk_kernel");
-  if (D == 64 && VD == 64)
-    return launch_dyn(decode_cmp_topk_kernel<64, 64>, grid, slot_bytes<64, 64>() + extra, p, stream,
-                      "decode_cmp_topk_kernel");
+  if (D == 128 && VD == 128) return launch_cmp_topk<128, 128>(p, grid, stream);
+  if (D == 64 && VD == 64) return launch_cmp_topk<64, 64>(p, grid, stream);
   nsa_set_error("decode: unsupported head dims D=%d VD=%d (built: 128/128, 64/64)", D, VD);
   return NSA_ERR_UNSUPPORTED;
 }
@@ -695,7 +774,8 @@ int nsa_decode_cmp_split_launch(const NsaDecodeParams& p, int B, int nsplit, int
   if (B <= 0) return NSA_OK;
   dim3 grid(B, p.KH, nsplit);
   int ntab = (p.y_cap + p.page_size - 1) / p.page_size;
-  size_t dyn1 = (size_t)SPLIT_WAVES * UK * (VD + NSA_LDS_PAD) * 2 + (size_t)(2 * SPLIT_WAVES * 16 + ntab) * 4;
+  size_t dyn1 = (size_t)SPLIT_WAVES * (D == 128 ? UnitFlash<128, 128>::SLOT : UnitFlash<64, 64>::SLOT) * 2 +
+                (size_t)(2 * SPLIT_WAVES * 16 + ntab) * 4;
   size_t dyn2 = (size_t)ntab * 4;
   if (!((D == 128 && VD == 128) || (D == 64 && VD == 64))) {
     nsa_set_error("decode: unsupported head dims D=%d VD=%d (built: 128/128, 64/64)", D, VD);

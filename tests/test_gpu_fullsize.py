@@ -77,10 +77,31 @@ def test_c3_packed_batch_equals_single_sequences(device):
         single = run(q[a:e], k[a:e], v[a:e], w[a:e], do[a:e], make_cu([e - a]))
         assert torch.equal(packed[0][a:e], single[0]), f"sequence {b}: forward differs"
         assert torch.equal(packed[1][a:e], single[1]), f"sequence {b}: dq differs"
-        # dk/dv are accumulated with fp32 atomics in a data-dependent order: equal up to fp32 summation order
-        assert_close(packed[2][a:e], single[2], f"sequence {b}: dk", atol=2e-3, rtol=2e-3, row_scale=True)
-        assert_close(packed[3][a:e], single[3], f"sequence {b}: dv", atol=2e-3, rtol=2e-3, row_scale=True)
+        # dk/dv are accumulated with fp32 atomics in a data-dependent order: equal up to fp32 summation order, i.e. one bf16 ulp (2^-7 relative) after the final rounding
+        assert_close(packed[2][a:e], single[2], f"sequence {b}: dk", atol=2e-3, rtol=8e-3, row_scale=True)
+        assert_close(packed[3][a:e], single[3], f"sequence {b}: dv", atol=2e-3, rtol=8e-3, row_scale=True)
         assert_close(packed[4][a:e], single[4], f"sequence {b}: dw", atol=1e-6, rtol=0)
+
+
+def _decode_block_scores(c, kh, b, device, G=16, D=128, block=64, kernel=32, stride=16):
+    """fp64 selection-block scores of one (request, kv head) of the decode benchmark case: softmax over the
+    compressed keys, summed over the q-heads of the group, folded by the overlap of every compressed key with the
+    block (flash_nsa/ops/topk.py:101-118 upstream)."""
+    page, L, y = c["page"], c["lens"][b], c["ys"][b]
+    i = torch.arange(y, device=device)
+    rows = c["cbt"][b][i // page].long() * page + i % page
+    kc = c["k"].view(-1, c["k"].shape[-2], D)[rows, kh].double()
+    qg = c["q"][b, kh * G:(kh + 1) * G].double()
+    p = torch.softmax(qg @ kc.t() * D ** -0.5, -1).sum(0)
+    nb = (L - 1) // block + 1
+    imp = torch.zeros(nb, dtype=torch.float64, device=device)
+    for j in range(nb):
+        i0, cs = (j * block - kernel) // stride + 1, stride - kernel
+        for r in range((block + kernel - stride) // stride):
+            if 0 <= i0 + r < y:
+                imp[j] += p[i0 + r] * (min(cs + kernel, block) - max(cs, 0)) / stride
+            cs += stride
+    return imp
 
 
 def test_c5_decode_full_batch(device):
@@ -103,7 +124,26 @@ def test_c5_decode_full_batch(device):
     fused = nsa_decode(c["q"], c["k"], c["v"], c["w"], c["ctx"], c["bt"], c["slots"], c["cbt"], **kw)
     staged = nsa_decode_staged(c["q"], c["k"], c["v"], c["w"], c["ctx"], c["bt"], c["cbt"], **kw)
     assert torch.isfinite(fused).all()
-    assert_close(fused, staged, "fused vs staged decode", atol=8e-3, rtol=1e-2)
+    # The fused kernel keeps the probabilities of the compressed keys as fp16 between its two phases, the staged
+    # path recomputes them in fp32: the selections may differ where two block scores tie.  Such rows are checked
+    # to be ties (fp64 scores closer than 1e-3) and left out of the output comparison.
+    from flash_nsa.inference import decode_cmp_topk, cmp_attn_decode, topk_decode
+    _, tk_f = decode_cmp_topk(c["q"], c["k"], c["v"], c["cbt"], c["ctx"], 2048, 512)
+    _, lse = cmp_attn_decode(c["q"], c["k"], c["v"], block_tables=c["cbt"], context_lens=c["ctx"])
+    tk_s = topk_decode(c["q"], c["k"], lse, fixed_y_maxlen=2048, fixed_num_slc_blocks=512, block_tables=c["cbt"],
+                       context_lens=c["ctx"])
+    differ = (tk_f.sort(-1).values != tk_s.sort(-1).values).any(-1)         # [KH, B]
+    assert int(differ.sum()) <= 8, f"{int(differ.sum())} of {differ.numel()} selections differ"
+    for kh, b in differ.nonzero().tolist():
+        imp = _decode_block_scores(c, kh, b, device)
+        only_f = sorted(set(tk_f[kh, b].tolist()) - set(tk_s[kh, b].tolist()))
+        only_s = sorted(set(tk_s[kh, b].tolist()) - set(tk_f[kh, b].tolist()))
+        assert len(only_f) == len(only_s)
+        lo = min(float(imp[j]) for j in only_f + only_s)
+        hi = max(float(imp[j]) for j in only_f + only_s)
+        assert hi - lo < 1e-3, f"selection of request {b}, kv head {kh} differs beyond a tie: {only_f} vs {only_s}"
+    keep = (~differ).t().repeat_interleave(16, dim=1)                       # [B, QH]
+    assert_close(fused[keep], staged[keep], "fused vs staged decode", atol=8e-3, rtol=1e-2)
     split = nsa_decode(c["q"], c["k"], c["v"], c["w"], c["ctx"], c["bt"], c["slots"], c["cbt"], cmp_num_splits=4, **kw)
     assert_close(split, staged, "split vs staged decode", atol=8e-3, rtol=1e-2)
     # request 5 as a single-token prefill through nsa_prefill (all compressed rows already pooled: slots -1)
