@@ -549,4 +549,56 @@ int nsa_decode_slc_swa_combine(const void* q, int64_t q_st, int64_t q_sh, const 
   return nsa_decode_slc_swa_launch(p, B, D, VD, (hipStream_t)stream);
 }
 
+int nsa_decode_fused_fits(int D, int VD, int fixed_y_maxlen, int fixed_num_slc_blocks, int table_stride,
+                          int page_size) {
+  if (fixed_y_maxlen < 1 || fixed_num_slc_blocks < 1 || table_stride < 1 || page_size < 1) return 0;
+  NsaDecodeParams p{};
+  p.y_cap = fixed_y_maxlen; p.nb_cap = fixed_num_slc_blocks; p.table_stride = table_stride; p.page_size = page_size;
+  return nsa_decode_fused_lds_bytes(p, D, VD) > 0 ? 1 : 0;
+}
+
+int nsa_decode_fused(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr, int64_t k_sh,
+                     const void* v_cache, int64_t v_sr, int64_t v_sh, const void* w, int64_t w_st, int64_t w_sh,
+                     void* out, int64_t o_st, int64_t o_sh, void* cmp_o, void* slc_o, void* swa_o, int64_t co_st,
+                     int64_t co_sh, float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk, int64_t tk_sh,
+                     int64_t tk_st, const int32_t* context_lens, const int32_t* block_tables, int table_stride,
+                     const int32_t* cmp_block_tables, int cmp_table_stride, int page_size, int B, int QH, int KH,
+                     int D, int VD, int fixed_y_maxlen, int fixed_num_slc_blocks, int kernel_size, int stride,
+                     int block_size, int top_n, int num_init, int num_local, int ignore_index, int window,
+                     float sm_scale, void* stream) {
+  int rc = check_heads("decode_fused", QH, KH, D, VD);
+  if (rc) return rc;
+  rc = check_nsa_sizes("decode_fused", kernel_size, stride, block_size);
+  if (rc) return rc;
+  rc = check_page("decode_fused", page_size);
+  if (rc) return rc;
+  NSA_REQUIRE(QH / KH <= 16, NSA_ERR_UNSUPPORTED, "decode_fused: at most 16 q-heads per kv head (got %d)", QH / KH);
+  NSA_REQUIRE(block_size % 32 == 0, NSA_ERR_UNSUPPORTED, "decode_fused: block_size %d must be a multiple of 32",
+              block_size);
+  NSA_REQUIRE(top_n >= 1 && top_n <= 64 && num_init >= 0 && num_local >= 0 && num_init + num_local <= top_n,
+              NSA_ERR_BAD_ARG, "decode_fused: bad top_n/num_init/num_local %d/%d/%d", top_n, num_init, num_local);
+  NSA_REQUIRE(fixed_y_maxlen >= 1 && fixed_num_slc_blocks >= 1 && table_stride >= 1 && cmp_table_stride >= 1,
+              NSA_ERR_BAD_ARG, "decode_fused: fixed_y_maxlen, fixed_num_slc_blocks and the table widths must be positive");
+  NSA_REQUIRE(out != nullptr && w != nullptr, NSA_ERR_BAD_ARG, "decode_fused: out and w are required");
+  NSA_REQUIRE(window >= 0, NSA_ERR_BAD_ARG, "decode_fused: window %d must be >= 0", window);
+  NsaDecodeParams p{};
+  p.q = (const bf16_t*)q; p.q_st = q_st; p.q_sh = q_sh;
+  p.k = (const bf16_t*)k_cache; p.k_sr = k_sr; p.k_sh = k_sh;
+  p.v = (const bf16_t*)v_cache; p.v_sr = v_sr; p.v_sh = v_sh;
+  p.w = (const bf16_t*)w; p.w_st = w_st; p.w_sh = w_sh;
+  p.out = (bf16_t*)out; p.o_st = o_st; p.o_sh = o_sh;
+  p.cmp_o = (bf16_t*)cmp_o; p.slc_o = (bf16_t*)slc_o; p.swa_o = (bf16_t*)swa_o; p.co_st = co_st; p.co_sh = co_sh;
+  p.lse_out = lse; p.lse_st = lse_st; p.lse_sh = lse_sh;
+  p.topk = topk; p.tk_sh = tk_sh; p.tk_st = tk_st;
+  p.ctx_lens = context_lens;
+  p.table = block_tables; p.table_stride = table_stride;
+  p.cmp_table = cmp_block_tables; p.cmp_table_stride = cmp_table_stride; p.page_size = page_size;
+  p.G = QH / KH; p.KH = KH;
+  p.scale_log2 = sm_scale * NSA_LOG2E;
+  p.kernel_size = kernel_size; p.stride = stride; p.block_size = block_size; p.window = window;
+  p.top_n = top_n; p.num_init = num_init; p.num_local = num_local; p.ignore_index = ignore_index;
+  p.y_cap = fixed_y_maxlen; p.nb_cap = fixed_num_slc_blocks;
+  return nsa_decode_fused_launch(p, B, D, VD, (hipStream_t)stream);
+}
+
 }  // extern "C"

@@ -126,4 +126,6 @@ struct NsaDecodeParams {
 };
 int nsa_decode_cmp_topk_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream);
 int nsa_decode_slc_swa_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream);
+int nsa_decode_fused_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream);
+int nsa_decode_fused_lds_bytes(const NsaDecodeParams& p, int D, int VD);  // 0: does not fit
 int nsa_decode_cmp_split_launch(const NsaDecodeParams& p, int B, int nsplit, int D, int VD, hipStream_t stream);

@@ -59,6 +59,14 @@ struct UnitFlash {
     m_run = NSA_NEG_INF;
     l_run = 0.f;
   }
+  // start another branch with the same q fragments
+  NSA_DEVICE void reset() {
+#pragma unroll
+    for (int dt = 0; dt < VD / 16; dt++) oacc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    m_run = NSA_NEG_INF;
+    l_run = 0.f;
+    keep_p = nullptr;
+  }
   // loads of the unit starting at key0 (wave-uniform); keys outside [klo, khi] are replaced by a clamped key
   // (masked later).  A unit spans at most two pages: the page of its first usable key is looked up once.
   NSA_DEVICE void issue(int key0, int klo, int khi, const int* tab_s, int page, const bf16_t* kbase, int64_t k_sr,
@@ -219,6 +227,67 @@ NSA_DEVICE float merge_partials(const float* pm, const float* pl, const float* p
   return l > 0.f ? o / l : 0.f;
 }
 
+// head-summed probabilities of the compressed keys -> scores of the selection blocks (ascending key order per
+// block); all threads of the workgroup
+NSA_DEVICE void fold_block_scores(const float* pg, float* imp, int y, int nb, int nb_cap, const NsaDecodeParams& p,
+                                  int tid, int nthreads) {
+  const int Bs = p.block_size, Kz = p.kernel_size, St = p.stride;
+  const int nloops = (Bs + Kz - St) / St;
+  for (int j = tid; j < nb_cap; j += nthreads) {
+    float acc = 0.f;
+    if (j < nb) {
+      int i0 = (j * Bs - Kz) / St + 1;
+      int cs = St - Kz;
+      for (int r = 0; r < nloops; r++, cs += St) {
+        int i = i0 + r;
+        if (i >= 0 && i < y) {
+          int area = min(cs + Kz, Bs) - max(cs, 0);
+          acc += pg[i] * ((float)area / (float)St);
+        }
+      }
+    }
+    imp[j] = acc;
+  }
+}
+
+// one wave: forced initial and local blocks, then repeated arg-max over imp[0 .. min(t/block, nb_cap-1)] (lowest
+// index on ties; taken scores are overwritten with -1).  Returns the block of slot `lane`.
+NSA_DEVICE int select_blocks_wave(float* imp, int t, int nb_cap, const NsaDecodeParams& p, int lane) {
+  const int nk = t >= 0 ? t / p.block_size : -1;
+  int result = p.ignore_index;
+  if (lane == 0) {
+    for (int s = 0; s < p.num_init; s++)
+      if (s < nb_cap) imp[s] = -1.f;
+    for (int i = 0; i < p.num_local; i++)
+      if (nk - i >= 0 && nk - i < nb_cap) imp[nk - i] = -1.f;
+  }
+  if (lane < p.num_init) {
+    if (lane <= nk) result = lane;
+  } else if (lane < p.num_init + p.num_local) {
+    if (lane <= nk) result = nk - (lane - p.num_init);
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const int nsel = min(p.top_n, nk + 1);
+  const int jmax = min(nk, nb_cap - 1);
+  for (int slot = p.num_init + p.num_local; slot < nsel; slot++) {
+    float best = -2.f;
+    int bj = 0x7fffffff;
+    for (int j = lane; j <= jmax; j += 64) {
+      float v = imp[j];
+      if (v > best) { best = v; bj = j; }
+    }
+    bj = wave_argmax_lowest(best, bj, bj != 0x7fffffff);
+    if (lane == slot) result = bj;
+    if (lane == 0 && bj <= jmax) imp[bj] = -1.f;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+  return result;
+}
+
 template <int D, int VD, bool KEEP>
 __global__ __launch_bounds__(DEC_WAVES * 64) void decode_cmp_topk_kernel(NsaDecodeParams p) {
   using UF = UnitFlash<D, VD>;
@@ -342,64 +411,11 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_cmp_topk_kernel(NsaDeco
     }
   }
   __syncthreads();
-  // ---- fold compressed keys into selection-block scores (ascending key order per block) ----
-  {
-    const int Bs = p.block_size, Kz = p.kernel_size, St = p.stride;
-    const int nloops = (Bs + Kz - St) / St;
-    for (int j = tid; j < p.nb_cap; j += NW * 64) {
-      float acc = 0.f;
-      if (j < nb) {
-        int i0 = (j * Bs - Kz) / St + 1;
-        int cs = St - Kz;
-        for (int r = 0; r < nloops; r++, cs += St) {
-          int i = i0 + r;
-          if (i >= 0 && i < y) {
-            int area = min(cs + Kz, Bs) - max(cs, 0);
-            acc += pg[i] * ((float)area / (float)St);
-          }
-        }
-      }
-      imp[j] = acc;
-    }
-  }
+  fold_block_scores(pg, imp, y, nb, p.nb_cap, p, tid, NW * 64);
   __syncthreads();
   if (wave != 0) return;
-  // ---- selection: forced initial and local blocks, then repeated arg-max (lowest index on ties) ----
-  {
-    const int nk = t >= 0 ? t / p.block_size : -1;
-    int result = p.ignore_index;
-    if (lane == 0) {
-      for (int s = 0; s < p.num_init; s++)
-        if (s < p.nb_cap) imp[s] = -1.f;
-      for (int i = 0; i < p.num_local; i++)
-        if (nk - i >= 0 && nk - i < p.nb_cap) imp[nk - i] = -1.f;
-    }
-    if (lane < p.num_init) {
-      if (lane <= nk) result = lane;
-    } else if (lane < p.num_init + p.num_local) {
-      if (lane <= nk) result = nk - (lane - p.num_init);
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const int nsel = min(p.top_n, nk + 1);
-    const int jmax = min(nk, p.nb_cap - 1);
-    for (int slot = p.num_init + p.num_local; slot < nsel; slot++) {
-      float best = -2.f;
-      int bj = 0x7fffffff;
-      for (int j = lane; j <= jmax; j += 64) {
-        float v = imp[j];
-        if (v > best) { best = v; bj = j; }
-      }
-      bj = wave_argmax_lowest(best, bj, bj != 0x7fffffff);
-      if (lane == slot) result = bj;
-      if (lane == 0 && bj <= jmax) imp[bj] = -1.f;
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    }
-    if (lane < p.top_n) p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + lane] = result;
-  }
+  const int result = select_blocks_wave(imp, t, p.nb_cap, p, lane);
+  if (lane < p.top_n) p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + lane] = result;
 }
 
 // ---- split variant of the compressed branch: requests are cut in NSPLIT key-interleaved parts so that long
@@ -606,57 +622,12 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecod
     // not-yet-used V staging area), force the initial/local blocks, then repeated arg-max by wave 0
     float* imp = reinterpret_cast<float*>(Vs_all);
     const float* pg = p.pg + ((int64_t)b * p.KH + kh) * p.y_cap;
-    const int Kz = p.kernel_size, St = p.stride;
-    const int y = L >= Kz ? min((L - Kz) / St + 1, p.y_cap) : 0;
+    const int y = L >= p.kernel_size ? min((L - p.kernel_size) / p.stride + 1, p.y_cap) : 0;
     const int nb = min(L > 0 ? (L - 1) / Bs + 1 : 0, p.nb_cap);
-    const int nloops = (Bs + Kz - St) / St;
-    for (int j = tid; j < nb; j += NW * 64) {
-      float acc = 0.f;
-      int i0 = (j * Bs - Kz) / St + 1;
-      int cs = St - Kz;
-      for (int r = 0; r < nloops; r++, cs += St) {
-        int i = i0 + r;
-        if (i >= 0 && i < y) {
-          int area = min(cs + Kz, Bs) - max(cs, 0);
-          acc += pg[i] * ((float)area / (float)St);
-        }
-      }
-      imp[j] = acc;
-    }
+    fold_block_scores(pg, imp, y, nb, nb, p, tid, NW * 64);
     __syncthreads();
     if (wave == 0) {
-      const int nk = t >= 0 ? t / Bs : -1;
-      int result = p.ignore_index;
-      if (lane == 0) {
-        for (int s2 = 0; s2 < p.num_init; s2++)
-          if (s2 < nb) imp[s2] = -1.f;
-        for (int i = 0; i < p.num_local; i++)
-          if (nk - i >= 0 && nk - i < nb) imp[nk - i] = -1.f;
-      }
-      if (lane < p.num_init) {
-        if (lane <= nk) result = lane;
-      } else if (lane < p.num_init + p.num_local) {
-        if (lane <= nk) result = nk - (lane - p.num_init);
-      }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      const int nsel = min(p.top_n, nk + 1);
-      const int jmax = min(nk, nb - 1);
-      for (int slot = p.num_init + p.num_local; slot < nsel; slot++) {
-        float best = -2.f;
-        int bj = 0x7fffffff;
-        for (int j = lane; j <= jmax; j += 64) {
-          float v = imp[j];
-          if (v > best) { best = v; bj = j; }
-        }
-        bj = wave_argmax_lowest(best, bj, bj != 0x7fffffff);
-        if (lane == slot) result = bj;
-        if (lane == 0 && bj <= jmax) imp[bj] = -1.f;
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      }
+      const int result = select_blocks_wave(imp, t, nb, p, lane);
       blk_s[lane] = lane < nvalid ? max(result, 0) : 0;
       if (lane < p.top_n) p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + lane] = result;
     }
@@ -704,6 +675,159 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecod
       float o_cmp = (float)p.cmp_o[(int64_t)b * p.co_st + (int64_t)hq * p.co_sh + d];
       p.out[(int64_t)b * p.o_st + (int64_t)hq * p.o_sh + d] = (bf16_t)(o_cmp * s0 + o_slc * s1 + o_swa * s2);
     }
+  }
+}
+
+// ---- the whole decode step of one (request, kv head) in one workgroup ------------------------------------------
+// compressed attention -> block scores -> [wave 0: selection | waves 1..7: window attention] -> selected-block
+// attention -> gated combine.  Nothing but the final output (and, on request, topk / the branch outputs) goes
+// back to global memory; the compressed-branch output stays in registers, the window partials in the LDS region
+// that held the fp16 probabilities.
+template <int D, int VD>
+__global__ __launch_bounds__(DEC_WAVES * 64) void decode_fused_kernel(NsaDecodeParams p) {
+  using UF = UnitFlash<D, VD>;
+  constexpr int NW = DEC_WAVES;
+  constexpr int SLOT = UF::SLOT;
+  constexpr int NTHREADS = NW * 64;
+  constexpr int OPT = 16 * VD / NTHREADS;  // merged output values per thread
+  static_assert(SLOT * 2 >= 16 * VD * 4, "a wave's slot must hold its partial output");
+  static_assert((16 * VD) % NTHREADS == 0, "output values must divide over the threads");
+  extern __shared__ __attribute__((aligned(16))) unsigned char dyn_raw[];
+  bf16_t* slots = reinterpret_cast<bf16_t*>(dyn_raw);
+  float* part_m = reinterpret_cast<float*>(dyn_raw + (size_t)NW * SLOT * 2);
+  float* part_l = part_m + NW * 16;
+  float* swa_m = part_l + NW * 16;
+  float* swa_l = swa_m + NW * 16;
+  float* lse_s = swa_l + NW * 16;
+  float* imp = lse_s + 16;
+  int* blk_s = reinterpret_cast<int*>(imp + ((p.nb_cap + 3) & ~3));
+  int* ctab_s = blk_s + 64;
+  const int ntab_c = (p.y_cap + p.page_size - 1) / p.page_size;
+  int* tab_s = ctab_s + ((ntab_c + 3) & ~3);
+  const int n_units_cap = (p.y_cap + UK - 1) / UK;
+  const int keep_ld = n_units_cap * UK + 8;
+  float* keep_m = reinterpret_cast<float*>(tab_s + ((p.table_stride + 3) & ~3));
+  _Float16* keep_p = reinterpret_cast<_Float16*>(keep_m + n_units_cap * 16);
+  float* swa_o = reinterpret_cast<float*>(keep_p);  // [NW-1][16][VD], after the probabilities are consumed
+  float* pg = reinterpret_cast<float*>(dyn_raw);    // over the staging slots, between the phases
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int b = blockIdx.x, kh = blockIdx.y;
+  const int G = p.G;
+  const int L = p.ctx_lens[b];
+  const int t = L - 1;
+  const int y = L >= p.kernel_size ? min((L - p.kernel_size) / p.stride + 1, p.y_cap) : 0;
+  const int Bs = p.block_size;
+  const int nb = min(L > 0 ? (L - 1) / Bs + 1 : 0, p.nb_cap);
+  const int page = p.page_size;
+  {
+    const int32_t* ctab = p.cmp_table + (int64_t)b * p.cmp_table_stride;
+    const int32_t* tab = p.table + (int64_t)b * p.table_stride;
+    const int nc = (y + page - 1) / page, nr = min((L + page - 1) / page, p.table_stride);
+    for (int i = tid; i < nc + nr; i += NTHREADS) {
+      if (i < nc) ctab_s[i] = ctab[i];
+      else tab_s[i - nc] = tab[i - nc];
+    }
+  }
+  __syncthreads();
+  const bf16_t* kbase = p.k + (int64_t)kh * p.k_sh;
+  const bf16_t* vbase = p.v + (int64_t)kh * p.v_sh;
+  const int l16 = lane & 15;
+  const int head = kh * G + min(l16, G - 1);
+
+  UF uf;
+  uf.init(p.q + (int64_t)b * p.q_st + (int64_t)head * p.q_sh, p.scale_log2, lane, slots + wave * SLOT);
+  uf.keep_p = keep_p;
+  uf.keep_m = keep_m;
+  uf.keep_ld = keep_ld;
+  const int nu = (y + UK - 1) / UK;
+
+  // ---- compressed attention, units dealt round-robin to the waves ----
+  uf.run(wave, NW, nu, 0, y - 1, [&](int u) { return u * UK; }, ctab_s, page, kbase, p.k_sr, vbase, p.v_sr);
+  uf.publish(part_m + wave * 16, part_l + wave * 16, reinterpret_cast<float*>(slots + wave * SLOT));
+  __syncthreads();
+  float o_cmp[OPT];
+#pragma unroll
+  for (int r = 0; r < OPT; r++) {
+    const int idx = tid + r * NTHREADS;
+    const int h = idx / VD, d = idx - h * VD;
+    float lse2;
+    float o = merge_partials(part_m, part_l, reinterpret_cast<const float*>(slots), NW, 16, SLOT / 2, h, d, VD,
+                             p.scale_log2, &lse2);
+    o_cmp[r] = (float)(bf16_t)o;  // the staged path stores the branch output as bf16 before the gated sum
+    if (d == 0) lse_s[h] = h < G ? lse2 : 0.f;
+    if (h < G) {
+      if (p.cmp_o) p.cmp_o[(int64_t)b * p.co_st + (int64_t)(kh * G + h) * p.co_sh + d] = (bf16_t)o;
+      if (d == 0 && p.lse_out) p.lse_out[(int64_t)b * p.lse_st + (kh * G + h) * p.lse_sh] = lse2;
+    }
+  }
+  __syncthreads();
+  // ---- probabilities p = kept exp2((s - m_unit)*c) * exp2(m_unit*c - lse), summed over the heads ----
+  for (int i = tid; i < nu * 16; i += NTHREADS) {
+    int h = i & 15;
+    keep_m[i] = h < G ? fast_exp2(__builtin_fmaf(keep_m[i], p.scale_log2, -lse_s[h])) : 0.f;
+  }
+  __syncthreads();
+  for (int key = tid; key < y; key += NTHREADS) {
+    const float* fac = keep_m + (key / UK) * 16;
+    float acc = 0.f;
+#pragma unroll
+    for (int h = 0; h < 16; h++) acc += (float)keep_p[h * keep_ld + key] * fac[h];
+    pg[key] = acc;
+  }
+  __syncthreads();
+  fold_block_scores(pg, imp, y, nb, p.nb_cap, p, tid, NTHREADS);
+  __syncthreads();
+
+  // ---- wave 0 selects the blocks while the other waves run the window ----
+  const int nvalid = t >= 0 ? min(p.top_n, t / Bs + 1) : 0;
+  uf.reset();
+  if (wave == 0) {
+    const int result = select_blocks_wave(imp, t, p.nb_cap, p, lane);
+    blk_s[lane] = lane < nvalid ? max(result, 0) : 0;
+    if (p.topk && lane < p.top_n) p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + lane] = result;
+  } else {
+    if (t >= 0) {
+      const int klo = max(0, t - p.window);
+      const int k0 = (klo / UK) * UK;
+      const int nuw = (t - k0) / UK + 1;
+      uf.run(wave - 1, NW - 1, nuw, klo, t, [&](int u) { return k0 + u * UK; }, tab_s, page, kbase, p.k_sr, vbase,
+             p.v_sr);
+    }
+    uf.publish(swa_m + wave * 16, swa_l + wave * 16, swa_o + (wave - 1) * 16 * VD);
+  }
+  __syncthreads();
+
+  // ---- selected blocks, all waves ----
+  uf.reset();
+  if (t >= 0) {
+    const int upb = Bs / UK;
+    uf.run(wave, NW, nvalid * upb, 0, t,
+           [&](int u) { int slot = u / upb; return blk_s[slot] * Bs + (u - slot * upb) * UK; }, tab_s, page, kbase,
+           p.k_sr, vbase, p.v_sr);
+  }
+  uf.publish(part_m + wave * 16, part_l + wave * 16, reinterpret_cast<float*>(slots + wave * SLOT));
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < OPT; r++) {
+    const int idx = tid + r * NTHREADS;
+    const int h = idx / VD, d = idx - h * VD;
+    if (h >= G) continue;
+    const int hq = kh * G + h;
+    float o_slc = merge_partials(part_m, part_l, reinterpret_cast<const float*>(slots), NW, 16, SLOT / 2, h, d, VD,
+                                 p.scale_log2, nullptr);
+    float o_swa = merge_partials(swa_m + 16, swa_l + 16, swa_o, NW - 1, 16, 16 * VD, h, d, VD, p.scale_log2, nullptr);
+    o_slc = (float)(bf16_t)o_slc;
+    o_swa = (float)(bf16_t)o_swa;
+    if (p.slc_o) p.slc_o[(int64_t)b * p.co_st + (int64_t)hq * p.co_sh + d] = (bf16_t)o_slc;
+    if (p.swa_o) p.swa_o[(int64_t)b * p.co_st + (int64_t)hq * p.co_sh + d] = (bf16_t)o_swa;
+    const bf16_t* wp = p.w + (int64_t)b * p.w_st + (int64_t)hq * p.w_sh;
+    float s0 = 1.f / (1.f + __expf(-(float)wp[0]));
+    float s1 = 1.f / (1.f + __expf(-(float)wp[1]));
+    float s2 = 1.f / (1.f + __expf(-(float)wp[2]));
+    p.out[(int64_t)b * p.o_st + (int64_t)hq * p.o_sh + d] = (bf16_t)(o_cmp[r] * s0 + o_slc * s1 + o_swa * s2);
   }
 }
 
@@ -793,4 +917,40 @@ int nsa_decode_cmp_split_launch(const NsaDecodeParams& p, int B, int nsplit, int
     decode_importance_kernel<64, 64><<<grid, SPLIT_WAVES * 64, dyn2, stream>>>(p);
   }
   return nsa_check_launch("decode_importance_kernel");
+}
+
+// LDS of the one-launch decode kernel; 0 when it does not fit (the caller then takes the two-launch path)
+template <int D, int VD>
+static size_t fused_lds(const NsaDecodeParams& p) {
+  const size_t ntab_c = (size_t)(p.y_cap + p.page_size - 1) / p.page_size;
+  const size_t units = (size_t)(p.y_cap + UK - 1) / UK;
+  size_t region = 16 * (units * UK + 8) * sizeof(_Float16);
+  const size_t swa_part = (size_t)(DEC_WAVES - 1) * 16 * VD * sizeof(float);
+  if (region < swa_part) region = swa_part;
+  region = (region + 15) & ~(size_t)15;
+  size_t n = slot_bytes<D, VD>() +
+             (size_t)(4 * DEC_WAVES * 16 + 16 + (((size_t)p.nb_cap + 3) & ~(size_t)3) + 64 + ((ntab_c + 3) & ~(size_t)3) +
+                      (((size_t)p.table_stride + 3) & ~(size_t)3) + units * 16) * sizeof(float) + region;
+  if ((size_t)p.y_cap * sizeof(float) > slot_bytes<D, VD>()) return 0;
+  return n <= 160 * 1024 ? n : 0;
+}
+
+int nsa_decode_fused_lds_bytes(const NsaDecodeParams& p, int D, int VD) {
+  if (D == 128 && VD == 128) return (int)fused_lds<128, 128>(p);
+  if (D == 64 && VD == 64) return (int)fused_lds<64, 64>(p);
+  return 0;
+}
+
+int nsa_decode_fused_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream) {
+  if (B <= 0) return NSA_OK;
+  dim3 grid(B, p.KH);
+  const int dyn = nsa_decode_fused_lds_bytes(p, D, VD);
+  if (dyn == 0) {
+    nsa_set_error("decode_fused: head dims %d/%d or fixed_y_maxlen %d / fixed_num_slc_blocks %d / table width %d do "
+                  "not fit the one-launch kernel (160 KB of LDS); use the two-launch path", D, VD, p.y_cap, p.nb_cap,
+                  p.table_stride);
+    return NSA_ERR_UNSUPPORTED;
+  }
+  if (D == 128) return launch_dyn(decode_fused_kernel<128, 128>, grid, (size_t)dyn, p, stream, "decode_fused_kernel");
+  return launch_dyn(decode_fused_kernel<64, 64>, grid, (size_t)dyn, p, stream, "decode_fused_kernel");
 }

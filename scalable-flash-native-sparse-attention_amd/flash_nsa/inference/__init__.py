@@ -6,7 +6,7 @@ never synchronise with the host, so the decode step can be captured in a HIP gra
 from .stages import (mean_pooling_prefill, kv_mean_pooling_decode, cmp_attn_prefill, cmp_attn_decode, topk_prefill,
                      topk_decode, slc_attn_prefill, fused_slc_swa_attn_decode, swa_prefill, combine_prefill,
                      combine_decode, mean_pooling_decode, slc_attn_decode, fused_decode_supported, decode_cmp_topk,
-                     decode_slc_swa_combine, decode_cmp_split)
+                     decode_slc_swa_combine, decode_cmp_split, decode_one_launch, decode_one_launch_fits)
 
 
 def nsa_prefill(q, k, v, w, x_cu_seqlens, y_cu_seqlens, x_maxlen, y_maxlen, context_lens, block_tables,
@@ -51,6 +51,12 @@ def nsa_decode(q, k, v, w, context_lens, block_tables, cmp_slot_mapping, cmp_blo
     kv_mean_pooling_decode(k, v, block_table=block_tables, slot_mapping=cmp_slot_mapping, context_lens=context_lens,
                            kernel_size=kernel_size, stride=stride)
     if fused_decode_supported(q, k, v):
+        if cmp_num_splits <= 1 and decode_one_launch_fits(q, k, v, block_tables, fixed_y_maxlen, fixed_num_slc_blocks):
+            return decode_one_launch(q, k, v, w, block_tables, cmp_block_tables, context_lens,
+                                     fixed_y_maxlen=fixed_y_maxlen, fixed_num_slc_blocks=fixed_num_slc_blocks,
+                                     kernel_size=kernel_size, stride=stride, block_size=block_size, top_n=top_n,
+                                     num_inital=num_init_blocks, num_local=num_local_blocks,
+                                     window_size=window_size, sm_scale=sm_scale)
         if cmp_num_splits <= 1:
             # two fused launches: (compressed attention + importance + selection), (selected + window + combine)
             cmp_o, topk = decode_cmp_topk(q, k, v, cmp_block_tables, context_lens, fixed_y_maxlen=fixed_y_maxlen,

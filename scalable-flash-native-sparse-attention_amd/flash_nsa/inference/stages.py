@@ -185,6 +185,43 @@ def fused_decode_supported(q, k, v):
     return QH // KH <= 16 and (q.size(-1), v.size(-1)) in ((128, 128), (64, 64))
 
 
+def decode_one_launch_fits(q, k, v, block_tables, fixed_y_maxlen, fixed_num_slc_blocks):
+    """True when the whole decode step fits the one-launch kernel (its LDS holds per-request tables and the
+    probabilities of fixed_y_maxlen compressed keys)."""
+    return bool(_lib.value("nsa_decode_fused_fits", q.size(-1), v.size(-1), int(fixed_y_maxlen),
+                           int(fixed_num_slc_blocks), int(block_tables.stride(0)), int(k.size(1))))
+
+
+def decode_one_launch(q, k, v, w, block_tables, cmp_block_tables, context_lens, fixed_y_maxlen=8192,
+                      fixed_num_slc_blocks=2048, kernel_size=32, stride=16, block_size=64, top_n=16, num_inital=1,
+                      num_local=2, window_size=512, sm_scale=None, return_parts=False):
+    """The decode step after pooling in one launch (one workgroup per request and kv head): compressed attention,
+    block scores, selection, window and selected-block attention, gated combine -> o [B,QH,VD]
+    (return_parts: also cmp_o, slc_o, swa_o, topk [KH,B,top_n], lse [B,QH])."""
+    check_bf16(q)
+    page, KH, D, ksr, ksh = _pool_args(k)
+    _, _, VD, vsr, vsh = _pool_args(v)
+    B, QH, _ = q.shape
+    sm_scale = q.size(-1) ** -0.5 if sm_scale is None else sm_scale
+    dev = q.device
+    out = torch.empty(B, QH, VD, device=dev, dtype=q.dtype)
+    parts = [torch.empty_like(out) for _ in range(3)] if return_parts else [None] * 3
+    topk = torch.empty(KH, B, top_n, device=dev, dtype=torch.int32) if return_parts else None
+    lse = torch.empty(B, QH, device=dev, dtype=torch.float32) if return_parts else None
+    _lib.call("nsa_decode_fused", q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), ksr, ksh, v.data_ptr(), vsr,
+              vsh, w.data_ptr(), w.stride(0), w.stride(1), out.data_ptr(), out.stride(0), out.stride(1),
+              _lib.ptr(parts[0]), _lib.ptr(parts[1]), _lib.ptr(parts[2]), out.stride(0), out.stride(1),
+              _lib.ptr(lse), lse.stride(0) if return_parts else 0, lse.stride(1) if return_parts else 0,
+              _lib.ptr(topk), topk.stride(0) if return_parts else 0, topk.stride(1) if return_parts else 0,
+              _i32(context_lens).data_ptr(), _i32(block_tables).data_ptr(), block_tables.stride(0),
+              _i32(cmp_block_tables).data_ptr(), cmp_block_tables.stride(0), page, B, QH, KH, D, VD,
+              int(fixed_y_maxlen), int(fixed_num_slc_blocks), kernel_size, stride, block_size, top_n, num_inital,
+              num_local, -1, window_size, sm_scale, _lib.stream_ptr())
+    if return_parts:
+        return out, parts[0], parts[1], parts[2], topk, lse
+    return out
+
+
 def decode_cmp_topk(q, k, v, cmp_block_tables, context_lens, fixed_y_maxlen=8192, fixed_num_slc_blocks=2048,
                     kernel_size=32, stride=16, block_size=64, top_n=16, num_inital=1, num_local=2, sm_scale=None,
                     return_lse=False):

@@ -230,3 +230,39 @@ def test_fused_decode_matches_staged_decode(device, QH, KH, D):
             for kh in range(KH):
                 assert sorted(t2[kh, b, :nv[b]].tolist()) == sorted(r[kh, b, :nv[b]].tolist()), (nsplit, b, kh)
         assert_close(out2, ref, f"split{nsplit} decode o", atol=8e-3, rtol=1e-2)
+
+
+@pytest.mark.parametrize("QH,KH,D", [(64, 4, 128), (16, 1, 128), (12, 2, 64)])
+def test_one_launch_decode_matches_two_launch_and_staged(device, QH, KH, D):
+    """The one-launch decode kernel (what nsa_decode runs when its tables fit in LDS) against the two-launch path
+    and the stage-by-stage kernels: branch outputs, lse, selection and the final output."""
+    from flash_nsa.inference import (nsa_decode_staged, decode_cmp_topk, decode_slc_swa_combine, decode_one_launch,
+                                     decode_one_launch_fits)
+    ctx = [4096, 333, 48, 31, 1, 777, 2999, 640, 1024, 65, 0, 513, 514]
+    case = build_pool([max(c, 1) for c in ctx], KH, D, D, page=128, seed=31)
+    prepool(case, [max(c, 1) for c in ctx])
+    B = len(ctx)
+    d = to_dev(case, device)
+    q = randn_bf16(B, QH, D, seed=32).to(device)
+    w = randn_bf16(B, QH, 3, seed=33).to(device)
+    ctx_t = torch.tensor(ctx, dtype=torch.int32, device=device)
+    assert decode_one_launch_fits(q, d["k"], d["v"], d["bt"], 512, 64)
+    assert not decode_one_launch_fits(q, d["k"], d["v"], d["bt"], 8192, 2048)
+    kw = dict(top_n=8, window_size=200)
+    out, cmp_o, slc_o, swa_o, topk, lse = decode_one_launch(q, d["k"], d["v"], w, d["bt"], d["cbt"], ctx_t, 512, 64,
+                                                            return_parts=True, **kw)
+    r_cmp, r_topk, r_lse = decode_cmp_topk(q, d["k"], d["v"], d["cbt"], ctx_t, 512, 64, top_n=8, return_lse=True)
+    r_out, r_slc, r_swa = decode_slc_swa_combine(q, d["k"], d["v"], w, r_topk, r_cmp, d["bt"], ctx_t,
+                                                 return_branches=True, **kw)
+    live = ctx_t > 0
+    assert torch.equal(cmp_o[live], r_cmp[live]) and torch.equal(lse[live], r_lse[live])
+    assert torch.equal(topk[:, live], r_topk[:, live])
+    assert_close(slc_o[live], r_slc[live], "slc_o", atol=4e-3, rtol=1e-2)
+    assert_close(swa_o[live], r_swa[live], "swa_o", atol=4e-3, rtol=1e-2)
+    assert_close(out[live], r_out[live], "o", atol=8e-3, rtol=1e-2)
+    assert float(out[~live].abs().max()) == 0.0, "a padded request (context 0) must give zeros"
+    ref = nsa_decode_staged(q[live], d["k"], d["v"], w[live], ctx_t[live], d["bt"][live], d["cbt"][live],
+                            fixed_y_maxlen=512, fixed_num_slc_blocks=64, **kw)
+    assert_close(out[live], ref, "o vs staged", atol=8e-3, rtol=1e-2)
+    out2 = decode_one_launch(q, d["k"], d["v"], w, d["bt"], d["cbt"], ctx_t, 512, 64, **kw)
+    assert torch.equal(out, out2), "optional outputs must not change the result"
