@@ -221,10 +221,13 @@ int nsa_decode_slc_swa_combine(const void* q, int64_t q_st, int64_t q_sh, const 
                                int table_stride, int page_size, int B, int QH, int KH, int D, int VD, int block_size,
                                int top_n, int window, float sm_scale, void* stream);
 
-/* The whole decode step after nsa_paged_pool_decode in ONE launch (one workgroup per request and kv head):
+/* The whole decode step in ONE launch (one workgroup per request and kv head):
  * replaces flash_nsa/inference/__init__.py:207-257 (cmp_attn_decode, topk_decode, fused_slc_swa_attn_decode,
  * combine_decode).  out [B,QH,VD] is required; cmp_o / slc_o / swa_o (shared strides co_st, co_sh), lse and topk
- * are optional outputs (NULL to skip).  Needs fixed_y_maxlen / fixed_num_slc_blocks / table_stride small enough for
+ * are optional outputs (NULL to skip).  cmp_slot_mapping [B] (optional): when given, the kernel also pools the
+ * compressed K and V row that the newest token completes (flat pool row, -1: none), i.e. it includes
+ * nsa_paged_pool_decode (flash_nsa/inference/compress_kv.py:253-287) and the step is a single launch.
+ * Needs fixed_y_maxlen / fixed_num_slc_blocks / table_stride small enough for
  * 160 KB of LDS (nsa_decode_fused_fits returns 1; e.g. contexts up to 32K tokens at kernel 32 / stride 16);
  * otherwise use nsa_decode_cmp_topk + nsa_decode_slc_swa_combine. */
 int nsa_decode_fused_fits(int D, int VD, int fixed_y_maxlen, int fixed_num_slc_blocks, int table_stride,
@@ -234,7 +237,8 @@ int nsa_decode_fused(const void* q, int64_t q_st, int64_t q_sh, const void* k_ca
                      void* out, int64_t o_st, int64_t o_sh, void* cmp_o, void* slc_o, void* swa_o, int64_t co_st,
                      int64_t co_sh, float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk, int64_t tk_sh,
                      int64_t tk_st, const int32_t* context_lens, const int32_t* block_tables, int table_stride,
-                     const int32_t* cmp_block_tables, int cmp_table_stride, int page_size, int B, int QH, int KH,
+                     const int32_t* cmp_block_tables, int cmp_table_stride,
+                     const int32_t* cmp_slot_mapping, int page_size, int B, int QH, int KH,
                      int D, int VD, int fixed_y_maxlen, int fixed_num_slc_blocks, int kernel_size, int stride,
                      int block_size, int top_n, int num_init, int num_local, int ignore_index, int window,
                      float sm_scale, void* stream);

@@ -562,7 +562,8 @@ int nsa_decode_fused(const void* q, int64_t q_st, int64_t q_sh, const void* k_ca
                      void* out, int64_t o_st, int64_t o_sh, void* cmp_o, void* slc_o, void* swa_o, int64_t co_st,
                      int64_t co_sh, float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk, int64_t tk_sh,
                      int64_t tk_st, const int32_t* context_lens, const int32_t* block_tables, int table_stride,
-                     const int32_t* cmp_block_tables, int cmp_table_stride, int page_size, int B, int QH, int KH,
+                     const int32_t* cmp_block_tables, int cmp_table_stride,
+                     const int32_t* cmp_slot_mapping, int page_size, int B, int QH, int KH,
                      int D, int VD, int fixed_y_maxlen, int fixed_num_slc_blocks, int kernel_size, int stride,
                      int block_size, int top_n, int num_init, int num_local, int ignore_index, int window,
                      float sm_scale, void* stream) {
@@ -593,6 +594,7 @@ int nsa_decode_fused(const void* q, int64_t q_st, int64_t q_sh, const void* k_ca
   p.ctx_lens = context_lens;
   p.table = block_tables; p.table_stride = table_stride;
   p.cmp_table = cmp_block_tables; p.cmp_table_stride = cmp_table_stride; p.page_size = page_size;
+  p.cmp_slots = cmp_slot_mapping;
   p.G = QH / KH; p.KH = KH;
   p.scale_log2 = sm_scale * NSA_LOG2E;
   p.kernel_size = kernel_size; p.stride = stride; p.block_size = block_size; p.window = window;

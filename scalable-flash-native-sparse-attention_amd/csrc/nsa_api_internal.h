@@ -116,6 +116,7 @@ struct NsaDecodeParams {
   const int32_t* ctx_lens;
   const int32_t* table; int table_stride;       // raw block tables
   const int32_t* cmp_table; int cmp_table_stride;
+  const int32_t* cmp_slots;                     // one-launch kernel: flat row of the compressed row completed now (-1: none), or null
   int page_size;
   int G, KH;
   float scale_log2;

@@ -730,6 +730,30 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_fused_kernel(NsaDecodeP
       if (i < nc) ctab_s[i] = ctab[i];
       else tab_s[i - nc] = tab[i - nc];
     }
+    // the compressed row that the newest token completes: mean of the last kernel_size raw rows of this kv head,
+    // summed in row order in fp32 like nsa_paged_pool_decode (flash_nsa/inference/compress_kv.py:253-287 upstream);
+    // wave 0 pools K, wave 1 pools V.  The row is written to the pool and read back below as the last key.
+    const int slot = p.cmp_slots != nullptr ? p.cmp_slots[b] : -1;
+    if (slot >= 0 && L >= p.kernel_size && wave < 2) {
+      bf16_t* cache = const_cast<bf16_t*>(wave == 0 ? p.k : p.v);
+      const int64_t c_sr = wave == 0 ? p.k_sr : p.v_sr, c_sh = wave == 0 ? p.k_sh : p.v_sh;
+      const int C = (wave == 0 ? D : VD) / 8;
+      if (lane < C) {
+        const int st = ((L - p.kernel_size) / p.stride) * p.stride;
+        float a[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (int r = 0; r < p.kernel_size; r++) {
+          const int n = st + r;
+          const int64_t row = (int64_t)tab[n / page] * page + (n % page);
+          bf16x8 x = ld_global_b128(cache + row * c_sr + (int64_t)kh * c_sh + lane * 8);
+#pragma unroll
+          for (int e = 0; e < 8; e++) a[e] += (float)x[e];
+        }
+        const float inv = 1.f / (float)p.kernel_size;
+        *reinterpret_cast<bf16x8*>(cache + (int64_t)slot * c_sr + (int64_t)kh * c_sh + lane * 8) =
+            pack8(a[0] * inv, a[1] * inv, a[2] * inv, a[3] * inv, a[4] * inv, a[5] * inv, a[6] * inv, a[7] * inv);
+      }
+      __threadfence();
+    }
   }
   __syncthreads();
   const bf16_t* kbase = p.k + (int64_t)kh * p.k_sh;

@@ -48,15 +48,18 @@ def nsa_decode(q, k, v, w, context_lens, block_tables, cmp_slot_mapping, cmp_blo
     assert k.size(1) % 64 == 0, "page size must be a multiple of 64"
     if sm_scale is None:
         sm_scale = q.size(-1) ** -0.5
+    one_launch = (fused_decode_supported(q, k, v) and cmp_num_splits <= 1 and
+                  decode_one_launch_fits(q, k, v, block_tables, fixed_y_maxlen, fixed_num_slc_blocks))
+    if one_launch:
+        # pooling of the newest compressed row included
+        return decode_one_launch(q, k, v, w, block_tables, cmp_block_tables, context_lens,
+                                 fixed_y_maxlen=fixed_y_maxlen, fixed_num_slc_blocks=fixed_num_slc_blocks,
+                                 kernel_size=kernel_size, stride=stride, block_size=block_size, top_n=top_n,
+                                 num_inital=num_init_blocks, num_local=num_local_blocks, window_size=window_size,
+                                 sm_scale=sm_scale, cmp_slot_mapping=cmp_slot_mapping)
     kv_mean_pooling_decode(k, v, block_table=block_tables, slot_mapping=cmp_slot_mapping, context_lens=context_lens,
                            kernel_size=kernel_size, stride=stride)
     if fused_decode_supported(q, k, v):
-        if cmp_num_splits <= 1 and decode_one_launch_fits(q, k, v, block_tables, fixed_y_maxlen, fixed_num_slc_blocks):
-            return decode_one_launch(q, k, v, w, block_tables, cmp_block_tables, context_lens,
-                                     fixed_y_maxlen=fixed_y_maxlen, fixed_num_slc_blocks=fixed_num_slc_blocks,
-                                     kernel_size=kernel_size, stride=stride, block_size=block_size, top_n=top_n,
-                                     num_inital=num_init_blocks, num_local=num_local_blocks,
-                                     window_size=window_size, sm_scale=sm_scale)
         if cmp_num_splits <= 1:
             # two fused launches: (compressed attention + importance + selection), (selected + window + combine)
             cmp_o, topk = decode_cmp_topk(q, k, v, cmp_block_tables, context_lens, fixed_y_maxlen=fixed_y_maxlen,

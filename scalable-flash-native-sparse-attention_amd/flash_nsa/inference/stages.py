@@ -194,10 +194,12 @@ def decode_one_launch_fits(q, k, v, block_tables, fixed_y_maxlen, fixed_num_slc_
 
 def decode_one_launch(q, k, v, w, block_tables, cmp_block_tables, context_lens, fixed_y_maxlen=8192,
                       fixed_num_slc_blocks=2048, kernel_size=32, stride=16, block_size=64, top_n=16, num_inital=1,
-                      num_local=2, window_size=512, sm_scale=None, return_parts=False):
-    """The decode step after pooling in one launch (one workgroup per request and kv head): compressed attention,
+                      num_local=2, window_size=512, sm_scale=None, return_parts=False, cmp_slot_mapping=None):
+    """The decode step in one launch (one workgroup per request and kv head): compressed attention,
     block scores, selection, window and selected-block attention, gated combine -> o [B,QH,VD]
-    (return_parts: also cmp_o, slc_o, swa_o, topk [KH,B,top_n], lse [B,QH])."""
+    (return_parts: also cmp_o, slc_o, swa_o, topk [KH,B,top_n], lse [B,QH]).  With cmp_slot_mapping [B] the kernel
+    first pools the compressed K/V row completed by the newest token (what kv_mean_pooling_decode does); without it
+    the caller has pooled already."""
     check_bf16(q)
     page, KH, D, ksr, ksh = _pool_args(k)
     _, _, VD, vsr, vsh = _pool_args(v)
@@ -214,7 +216,8 @@ def decode_one_launch(q, k, v, w, block_tables, cmp_block_tables, context_lens, 
               _lib.ptr(lse), lse.stride(0) if return_parts else 0, lse.stride(1) if return_parts else 0,
               _lib.ptr(topk), topk.stride(0) if return_parts else 0, topk.stride(1) if return_parts else 0,
               _i32(context_lens).data_ptr(), _i32(block_tables).data_ptr(), block_tables.stride(0),
-              _i32(cmp_block_tables).data_ptr(), cmp_block_tables.stride(0), page, B, QH, KH, D, VD,
+              _i32(cmp_block_tables).data_ptr(), cmp_block_tables.stride(0),
+              None if cmp_slot_mapping is None else _i32(cmp_slot_mapping).data_ptr(), page, B, QH, KH, D, VD,
               int(fixed_y_maxlen), int(fixed_num_slc_blocks), kernel_size, stride, block_size, top_n, num_inital,
               num_local, -1, window_size, sm_scale, _lib.stream_ptr())
     if return_parts:

@@ -266,3 +266,26 @@ def test_one_launch_decode_matches_two_launch_and_staged(device, QH, KH, D):
     assert_close(out[live], ref, "o vs staged", atol=8e-3, rtol=1e-2)
     out2 = decode_one_launch(q, d["k"], d["v"], w, d["bt"], d["cbt"], ctx_t, 512, 64, **kw)
     assert torch.equal(out, out2), "optional outputs must not change the result"
+
+
+def test_one_launch_decode_pools_the_new_row_itself(device):
+    """nsa_decode's one-launch kernel with a slot mapping == pooling kernel followed by the same kernel without:
+    the pools end bit-identical and so do the outputs."""
+    from flash_nsa.inference import decode_one_launch, kv_mean_pooling_decode
+    QH, KH, D = 64, 4, 128
+    ctx = [1024, 48, 32, 31, 2001, 656, 645, 4099]       # four of them complete a compressed row at this step
+    case = build_pool(ctx, KH, D, D, page=128, seed=41)
+    prepool(case, [L - 1 for L in ctx])
+    slots = decode_slot_mapping(case)
+    assert int((slots >= 0).sum()) == 4
+    B = len(ctx)
+    q, w = randn_bf16(B, QH, D, seed=42).to(device), randn_bf16(B, QH, 3, seed=43).to(device)
+    ctx_t = torch.tensor(ctx, dtype=torch.int32, device=device)
+    d1, d2 = to_dev(case, device), to_dev(case, device)
+    d2["k"], d2["v"] = d2["k"].clone(), d2["v"].clone()
+    kv_mean_pooling_decode(d1["k"], d1["v"], block_table=d1["bt"], slot_mapping=slots.to(device), context_lens=ctx_t)
+    o1 = decode_one_launch(q, d1["k"], d1["v"], w, d1["bt"], d1["cbt"], ctx_t, 512, 64)
+    o2 = decode_one_launch(q, d2["k"], d2["v"], w, d2["bt"], d2["cbt"], ctx_t, 512, 64,
+                           cmp_slot_mapping=slots.to(device))
+    assert torch.equal(d1["k"], d2["k"]) and torch.equal(d1["v"], d2["v"])
+    assert torch.equal(o1, o2)
