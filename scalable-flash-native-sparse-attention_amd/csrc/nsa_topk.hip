@@ -27,27 +27,106 @@ struct SlotMap {
   }
 };
 
+// Picks the blocks of one token from its score row imp[0 .. nb_max) (one wave): forced initial and local blocks
+// first, then repeated arg-max (lowest index on ties).  Returns the block of slot `lane`.
+// With REGS the candidates of a lane (blocks lane, lane+64, ...) sit in 16 registers (nb_max <= 1024) and only the
+// winner's lane rescans; otherwise every round rescans the LDS row.
+template <bool REGS>
+NSA_DEVICE int select_row(float* imp, int t, int nb_max, const NsaTopkParams& p, int lane) {
+  const int nk = t / p.block_size;
+  const int jmax = min(nk, nb_max - 1);
+  const int nsel = min(p.top_n, nk + 1);
+  int result = p.ignore_index;
+  if (lane < p.num_init) {
+    if (lane <= nk) result = lane;
+  } else if (lane < p.num_init + p.num_local) {
+    if (lane <= nk) result = nk - (lane - p.num_init);
+  }
+  if (REGS) {
+    float v[16];
+#pragma unroll
+    for (int k = 0; k < 16; k++) {
+      const int j = lane + 64 * k;
+      float x = j <= jmax ? imp[min(j, nb_max - 1)] : -3.f;
+      if (j <= jmax && (j < p.num_init || j > nk - p.num_local)) x = -1.f;
+      v[k] = x;
+    }
+    float best = -2.f;
+    int bj = 0x7fffffff;
+#pragma unroll
+    for (int k = 0; k < 16; k++)
+      if (v[k] > best) { best = v[k]; bj = lane + 64 * k; }
+    for (int slot = p.num_init + p.num_local; slot < nsel; slot++) {
+      const int w = wave_argmax_lowest(best, bj, bj != 0x7fffffff);
+      if (lane == slot) result = w;
+      const bool mine = (w & 63) == lane && w <= jmax;
+      const int kk = w >> 6;
+      best = -2.f;
+      bj = 0x7fffffff;
+#pragma unroll
+      for (int k = 0; k < 16; k++) {
+        if (mine && k == kk) v[k] = -1.f;
+        if (v[k] > best) { best = v[k]; bj = lane + 64 * k; }
+      }
+    }
+    return result;
+  }
+  if (lane == 0) {
+    for (int s = 0; s < p.num_init; s++)
+      if (s < nb_max) imp[s] = -1.f;
+    for (int i = 0; i < p.num_local; i++)
+      if (nk - i >= 0 && nk - i < nb_max) imp[nk - i] = -1.f;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  for (int slot = p.num_init + p.num_local; slot < nsel; slot++) {
+    float best = -2.f;
+    int bj = 0x7fffffff;
+    for (int j = lane; j <= jmax; j += 64) {
+      float x = imp[j];
+      if (x > best) { best = x; bj = j; }
+    }
+    bj = wave_argmax_lowest(best, bj, bj != 0x7fffffff);
+    if (lane == slot) result = bj;
+    if (lane == 0 && bj <= jmax) imp[bj] = -1.f;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+  return result;
+}
+
+// Workgroup = 4 waves on the same 64 (token, head) rows (two MFMA row blocks); the compressed keys are cut in units
+// of 32 that are dealt to the waves (wave w takes unit 4*tile + w of every 128-key tile).  A wave stages the rows of
+// its unit in a private LDS slot (coalesced whole-row loads, one tile ahead through registers), reads each K
+// fragment once and uses it for both row blocks; the head-summed probabilities go to a double-buffered LDS tile,
+// and after the one barrier per tile all threads fold that tile into the block scores in ascending key order.
 template <int D, int GP, bool PAGED>
-__global__ __launch_bounds__(256) void topk_kernel(NsaTopkParams p) {
-  constexpr int KT = 64;
+__global__ __launch_bounds__(256, 2) void topk_kernel(NsaTopkParams p) {
+  constexpr int UK = 32;            // keys per unit
+  constexpr int KT = 4 * UK;        // keys per tile
+  constexpr int RB = 2;             // 32-row blocks per workgroup
   constexpr int KLD = D + NSA_LDS_PAD;
-  constexpr int TPW = 32 / GP;  // tokens per wave
-  constexpr int TWG = 4 * TPW;  // tokens per workgroup
-  constexpr int PLD = KT + 1;
+  constexpr int TPB = 32 / GP;      // tokens per row block
+  constexpr int TWG = RB * TPB;     // tokens per workgroup
+  constexpr int PLD = KT + 4;
+  constexpr int KP = D / 8;
+  constexpr int KJ = (UK * KP) / 64;
   using SM = SlotMap<GP>;
-  __shared__ __attribute__((aligned(16))) bf16_t Ks[KT * KLD];
-  __shared__ float Pst[4 * TPW * PLD];
+  __shared__ __attribute__((aligned(16))) bf16_t Ks_all[4 * UK * KLD];
+  __shared__ float Pst[2 * TWG * PLD];
   extern __shared__ float imp_all[];  // [TWG][nb_max]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31;
   const int hl = lane >> 5;
   const int b = blockIdx.y;
   const int kh = blockIdx.z;
   const int G = p.G;
-  const int n_hc = (G + 31) / 32;
+  const int n_hc = GP < 32 ? 1 : (G + 31) / 32;  // chunks of 32 q-heads (more than one only for G > 32)
 
   const int x0 = p.x_cu[b];
   const int xl = p.x_cu[b + 1] - x0;
@@ -61,190 +140,209 @@ __global__ __launch_bounds__(256) void topk_kernel(NsaTopkParams p) {
   const int nb_max = p.nb_max;
   const int Bs = p.block_size, Kz = p.kernel_size, St = p.stride;
 
-  float* imp_w = imp_all + (wave * TPW) * nb_max;  // this wave's token rows
-  for (int i = lane; i < TPW * nb_max; i += 64) imp_w[i] = 0.f;
-  float* pst_w = Pst + wave * TPW * PLD;
+  for (int i = tid; i < TWG * nb_max; i += 256) imp_all[i] = 0.f;
+  bf16_t* Ks = Ks_all + wave * UK * KLD;
 
-  // A-operand row of this lane
-  const int tokl_a = l32 / GP;
-  const int nw0 = n0 + wave * TPW;
-  const int n_a = min(nw0 + tokl_a, xl - 1);
   const int t_hi_wg = min(n0 + TWG - 1, xl - 1) + qoff;
   const int key_end = t_hi_wg >= Kz - 1 ? min((t_hi_wg - Kz + 1) / St + 1, nkeys) : 0;
-  const int tw_hi = min(nw0 + TPW - 1, xl - 1) + qoff;
-  const bool wave_active = nw0 < xl;
+  const int ntiles = (key_end + KT - 1) / KT;
 
-  // per-lane C-layout rows: lse and positions
-  float lse_r[16];
-  int t_r[16];
-  bf16x8 qf[D / 16];
-
+  // A-operand rows of this lane (row l32 of each block) and the lse of its C-layout rows
+  bf16x8 qf[RB][D / 16];
+  float lse_r[RB][16];
+  bool rows_full[RB];
   auto load_rows = [&](int hc) {
-    int g = hc * 32 + (l32 % GP);
-    if (g >= G) g = G - 1;
-    const bf16_t* qp = p.q + (int64_t)(x0 + n_a) * p.q_st + (int64_t)(kh * G + g) * p.q_sh + hl * 8;
 #pragma unroll
-    for (int kc = 0; kc < D / 16; kc++) qf[kc] = ld_global_b128(qp + kc * 16);
+    for (int rb = 0; rb < RB; rb++) {
+      int g = hc * 32 + (l32 % GP);
+      if (g >= G) g = G - 1;
+      const int n_a = min(n0 + rb * TPB + l32 / GP, xl - 1);
+      const bf16_t* qp = p.q + (int64_t)(x0 + n_a) * p.q_st + (int64_t)(kh * G + g) * p.q_sh + hl * 8;
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
-      int row = (i >> 2) * 8 + hl * 4 + (i & 3);
-      int gg = hc * 32 + (row % GP);
-      int nn = nw0 + row / GP;
-      bool ok = (gg < G) && (nn < xl);
-      t_r[i] = ok ? nn + qoff : -1;  // -1: nothing visible
-      lse_r[i] = ok ? p.lse[(int64_t)(x0 + nn) * p.lse_st + (int64_t)(kh * G + gg) * p.lse_sh] : 0.f;
+      for (int kc = 0; kc < D / 16; kc++) qf[rb][kc] = ld_global_b128(qp + kc * 16);
+      bool mine = true;
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        int row = (i >> 2) * 8 + hl * 4 + (i & 3);
+        int gg = hc * 32 + (row % GP);
+        int nn = n0 + rb * TPB + row / GP;
+        bool ok = (gg < G) && (nn < xl);
+        mine = mine && ok;
+        lse_r[rb][i] = ok ? p.lse[(int64_t)(x0 + nn) * p.lse_st + (int64_t)(kh * G + gg) * p.lse_sh] : 0.f;
+      }
+      rows_full[rb] = __builtin_amdgcn_ballot_w64(!mine) == 0;
     }
   };
-  if (n_hc == 1) load_rows(0);
+  if (GP < 32 || n_hc == 1) load_rows(0);
 
-  for (int kt = 0; kt < key_end; kt += KT) {
-    __syncthreads();
-    {
-      int64_t page_row0 = 0;
-      if (PAGED) {
-        int pg = table[kt / p.page_size];
-        page_row0 = (int64_t)pg * p.page_size + (kt % p.page_size);
-      }
-      constexpr int KP = D / 8;
+  // fold constants: a tile covers a whole number of selection blocks, so the blocks a tile touches, the offsets of
+  // their compressed keys inside the tile and the overlap weights are the same for every tile
+  const int f_nloops = (Bs + Kz - St) / St;
+  const int f_nj = (St * (KT - 1) + Kz - 1) / Bs + 1;
+  const bool fold_fast = (St * KT) % Bs == 0 && TWG * f_nj <= 256 && f_nloops <= 8;
+  const int f_tk = tid / f_nj, f_jj = tid - f_tk * f_nj;
+  const bool f_on = tid < TWG * f_nj;
+  const int f_rel0 = (f_jj * Bs - Kz) / St + 1;
+  float f_w[8];
+  {
+    int cs = St - Kz;
 #pragma unroll
-      for (int j = 0; j < (KT * KP) / 256; j++) {
-        int pc = tid + j * 256;
-        int kr = pc / KP, dp = pc - kr * KP;
-        bf16x8 val = zero_bf16x8();
-        if (kt + kr < key_end) {
-          int64_t row = PAGED ? page_row0 + kr : (int64_t)kbase + kt + kr;
-          val = ld_global_b128(p.ck + row * p.ck_sr + (int64_t)kh * p.ck_sh + dp * 8);
-        }
-        *reinterpret_cast<bf16x8*>(&Ks[kr * KLD + dp * 8]) = val;
+    for (int r = 0; r < 8; r++, cs += St) {
+      f_w[r] = (float)(min(cs + Kz, Bs) - max(cs, 0)) / (float)St;
+      asm volatile("" : "+v"(f_w[r]));  // keep the quotient in a register: the division must not sink into the loop
+    }
+  }
+
+  // rows of the wave's unit of the next tile travel through registers while the current one is computed
+  bf16x8 kreg[KJ];
+  uint32_t kboff[KJ];  // byte offset of the lane's 16-byte pieces inside a unit (same for every unit)
+#pragma unroll
+  for (int j = 0; j < KJ; j++) {
+    int pc = lane + j * 64;
+    kboff[j] = (uint32_t)(((int64_t)(pc / KP) * p.ck_sr + (pc % KP) * 8) * 2);
+  }
+  auto issue = [&](int key0) {
+    int64_t row0;
+    if (PAGED) row0 = (int64_t)table[key0 / p.page_size] * p.page_size + (key0 % p.page_size);
+    else row0 = (int64_t)kbase + key0;
+    const char* kb = reinterpret_cast<const char*>(p.ck + row0 * p.ck_sr + (int64_t)kh * p.ck_sh);
+    const int last = key_end - 1 - key0;
+    if (last >= UK - 1) {
+#pragma unroll
+      for (int j = 0; j < KJ; j++) kreg[j] = *reinterpret_cast<const bf16x8*>(kb + kboff[j]);
+    } else {  // the last unit: rows past the last visible key repeat it (masked below)
+#pragma unroll
+      for (int j = 0; j < KJ; j++) {
+        int pc = lane + j * 64;
+        int kr = min(pc / KP, last);
+        kreg[j] = ld_global_b128(p.ck + (row0 + kr) * p.ck_sr + (int64_t)kh * p.ck_sh + (pc % KP) * 8);
       }
     }
-    __syncthreads();
-    if (!wave_active) continue;
-    if (tw_hi < St * kt + Kz - 1) continue;  // tile invisible to every token of this wave
+  };
+  if (wave * UK < key_end) issue(wave * UK);
+  __syncthreads();  // score rows are zeroed
 
-    for (int hc = 0; hc < n_hc; hc++) {
-      if (n_hc > 1) load_rows(hc);
+  for (int tile = 0; tile < ntiles; tile++) {
+    const int key0 = tile * KT + wave * UK;
+    float* pst = Pst + (tile & 1) * TWG * PLD;
+    if (key0 < key_end) {
 #pragma unroll
-      for (int nt = 0; nt < 2; nt++) {
-        f32x16 sacc;
+      for (int j = 0; j < KJ; j++) {
+        int pc = lane + j * 64;
+        *reinterpret_cast<bf16x8*>(&Ks[(pc / KP) * KLD + (pc % KP) * 8]) = kreg[j];
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      if (key0 + KT < key_end) issue(key0 + KT);
+      bf16x8 kf[D / 16];
 #pragma unroll
-        for (int i = 0; i < 16; i++) sacc[i] = 0.f;
-        const bf16_t* kp = &Ks[(nt * 32 + l32) * KLD + hl * 8];
+      for (int kc = 0; kc < D / 16; kc++)
+        kf[kc] = *reinterpret_cast<const bf16x8*>(&Ks[l32 * KLD + hl * 8 + kc * 16]);
+      const int key = key0 + l32;
+      const int vis_from = St * key + Kz - 1;  // first position that sees this key
+      for (int hc = 0; hc < n_hc; hc++) {
+        if (GP == 32 && n_hc > 1) load_rows(hc);
 #pragma unroll
-        for (int kc = 0; kc < D / 16; kc++) {
-          bf16x8 kf = *reinterpret_cast<const bf16x8*>(kp + kc * 16);
-          sacc = mfma32(qf[kc], kf, sacc);
-        }
-        const int key = kt + nt * 32 + l32;
-        const int vis_from = St * key + Kz - 1;  // first position that sees this key
-        float ps[SM::NSLOT];
+        for (int rb = 0; rb < RB; rb++) {
+          f32x16 sacc;
 #pragma unroll
-        for (int s = 0; s < SM::NSLOT; s++) ps[s] = 0.f;
+          for (int i = 0; i < 16; i++) sacc[i] = 0.f;
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-          bool vis = (key < nkeys) && (t_r[i] >= vis_from);
-          float pv = vis ? fast_exp2(sacc[i] * p.scale_log2 - lse_r[i]) : 0.f;
-          ps[SM::slot_of(i)] += pv;
-        }
+          for (int kc = 0; kc < D / 16; kc++) sacc = mfma32(qf[rb][kc], kf[kc], sacc);
+          float ps[SM::NSLOT];
 #pragma unroll
-        for (int s = 0; s < SM::NSLOT; s++) {
-          float v = ps[s];
-          if (SM::CROSS) v += __shfl_xor(v, 32, 64);
-          if (!SM::CROSS || hl == 0) {
-            int tk = SM::token_of(s, hl);
-            float* dst = &pst_w[tk * PLD + nt * 32 + l32];
-            *dst = (hc == 0) ? v : *dst + v;
+          for (int s2 = 0; s2 < SM::NSLOT; s2++) ps[s2] = 0.f;
+          // wave-uniform: away from the causal boundary every (row, key) pair of the unit is visible
+          const bool all_vis = rows_full[rb] && key0 + UK <= nkeys &&
+                               n0 + rb * TPB + qoff >= St * (key0 + UK - 1) + Kz - 1;
+          if (all_vis) {
+#pragma unroll
+            for (int i = 0; i < 16; i++)
+              ps[SM::slot_of(i)] += fast_exp2(__builtin_fmaf(sacc[i], p.scale_log2, -lse_r[rb][i]));
+          } else {
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+              int row = (i >> 2) * 8 + hl * 4 + (i & 3);
+              int nn = n0 + rb * TPB + row / GP;
+              bool vis = (hc * 32 + (row % GP) < G) && (nn < xl) && (key < nkeys) && (nn + qoff >= vis_from);
+              float pv = vis ? fast_exp2(__builtin_fmaf(sacc[i], p.scale_log2, -lse_r[rb][i])) : 0.f;
+              ps[SM::slot_of(i)] += pv;
+            }
+          }
+#pragma unroll
+          for (int s2 = 0; s2 < SM::NSLOT; s2++) {
+            float v = ps[s2];
+            if (SM::CROSS) v = xhalf_sum(v);
+            if (!SM::CROSS || hl == 0) {
+              int tk = rb * TPB + SM::token_of(s2, hl);
+              float* dst = &pst[tk * PLD + wave * UK + l32];
+              *dst = (hc == 0) ? v : *dst + v;
+            }
           }
         }
       }
+    } else {
+      for (int i = lane; i < TWG * UK; i += 64) pst[(i / UK) * PLD + wave * UK + (i % UK)] = 0.f;
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    // ---- fold the 64 compressed keys of this tile into selection-block scores ----
-    {
-      const int nloops = (Bs + Kz - St) / St;
+    __syncthreads();
+    // ---- fold the 128 compressed keys of this tile into selection-block scores ----
+    const int kt = tile * KT;
+    if (fold_fast) {
+      const int j = (St * kt) / Bs + f_jj;
+      if (f_on && j < nb_max) {
+        float acc = imp_all[f_tk * nb_max + j];
+#pragma unroll
+        for (int r = 0; r < 8; r++) {
+          const int i = f_rel0 + r;
+          if (r < f_nloops && i >= 0 && i < KT) acc += pst[f_tk * PLD + i] * f_w[r];
+        }
+        imp_all[f_tk * nb_max + j] = acc;
+      }
+    } else {
       const int j_lo = (St * kt) / Bs;
       const int j_hi = min((St * (kt + KT - 1) + Kz - 1) / Bs, nb_max - 1);
       const int nj = j_hi - j_lo + 1;
-      for (int it = lane; it < TPW * nj; it += 64) {
+      for (int it = tid; it < TWG * nj; it += 256) {
         int tk = it / nj;
         int j = j_lo + (it - tk * nj);
         int i0 = (j * Bs - Kz) / St + 1;  // exact: block and kernel sizes are multiples of the stride
-        float acc = imp_w[tk * nb_max + j];
+        float acc = imp_all[tk * nb_max + j];
         int cs = St - Kz;
-        for (int r = 0; r < nloops; r++, cs += St) {
+        for (int r = 0; r < f_nloops; r++, cs += St) {
           int i = i0 + r;
           if (i >= kt && i < kt + KT) {
             int area = min(cs + Kz, Bs) - max(cs, 0);
-            acc += pst_w[tk * PLD + (i - kt)] * ((float)area / (float)St);
+            acc += pst[tk * PLD + (i - kt)] * ((float)area / (float)St);
           }
         }
-        imp_w[tk * nb_max + j] = acc;
+        imp_all[tk * nb_max + j] = acc;
       }
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
-  if (!wave_active) return;
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  __syncthreads();
 
-  // ---- selection, one token at a time ----
-  for (int tk = 0; tk < TPW; tk++) {
-    const int n = nw0 + tk;
+  // ---- selection: the tokens of the workgroup are dealt to the waves ----
+  for (int tk = wave; tk < TWG; tk += 4) {
+    const int n = n0 + tk;
     if (n >= xl) break;
     const int t = n + qoff;
-    const int nk = t / Bs;
-    float* imp = imp_w + tk * nb_max;
+    float* imp = imp_all + tk * nb_max;
     const int64_t tok = x0 + n;
     if (p.imp_out != nullptr) {
       for (int j = lane; j < p.imp_cols; j += 64)
         p.imp_out[(int64_t)kh * p.imp_sh + tok * p.imp_st + j] = j < nb_max ? imp[j] : 0.f;
     }
-    int result = p.ignore_index;
-    __builtin_amdgcn_wave_barrier();
-    if (lane == 0) {
-      for (int s = 0; s < p.num_init; s++)
-        if (s < nb_max) imp[s] = -1.f;
-      for (int i = 0; i < p.num_local; i++)
-        if (nk - i >= 0 && nk - i < nb_max) imp[nk - i] = -1.f;
-    }
-    if (lane < p.num_init) {
-      if (lane <= nk) result = lane;
-    } else if (lane < p.num_init + p.num_local) {
-      if (lane <= nk) result = nk - (lane - p.num_init);
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const int nsel = min(p.top_n, nk + 1);
-    const int jmax = min(nk, nb_max - 1);
-    for (int slot = p.num_init + p.num_local; slot < nsel; slot++) {
-      float best = -2.f;
-      int bj = 0x7fffffff;
-      for (int j = lane; j <= jmax; j += 64) {
-        float v = imp[j];
-        if (v > best) { best = v; bj = j; }
-      }
-      bj = wave_argmax_lowest(best, bj, bj != 0x7fffffff);
-      if (lane == slot) result = bj;
-      if (lane == 0 && bj <= jmax) imp[bj] = -1.f;
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    }
+    const int result = nb_max <= 1024 ? select_row<true>(imp, t, nb_max, p, lane) : select_row<false>(imp, t, nb_max, p, lane);
     if (lane < p.top_n) p.topk[(int64_t)kh * p.tk_sh + tok * p.tk_st + lane] = result;
   }
 }
 
 template <int D, int GP, bool PAGED>
 int launch_topk(const NsaTopkParams& p, int B, int max_q_len, hipStream_t stream) {
-  constexpr int TWG = 4 * (32 / GP);
+  constexpr int TWG = 2 * (32 / GP);
   size_t dyn = (size_t)TWG * p.nb_max * sizeof(float);
-  size_t stat = 64 * (D + NSA_LDS_PAD) * 2 + 4 * (32 / GP) * 65 * 4;
+  size_t stat = 128 * (D + NSA_LDS_PAD) * 2 + 2 * TWG * 132 * 4;
   if (dyn + stat > 160 * 1024) {
     nsa_set_error("top-k: %d selection blocks x %d tokens per workgroup do not fit LDS", p.nb_max, TWG);
     return NSA_ERR_UNSUPPORTED;
