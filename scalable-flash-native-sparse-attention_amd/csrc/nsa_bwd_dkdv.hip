@@ -18,11 +18,12 @@ constexpr int MODE_CMP = 0;
 constexpr int MODE_SWA = 1;
 constexpr int MODE_SLC = 2;
 
-template <int D, int VD, int MODE, int NW>
+template <int D, int VD, int MODE, int NW, int KB>
 __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
   constexpr int NT = NW * 64;
-  constexpr int KW = NW * 32;
-  constexpr int RT = 64;
+  constexpr int KPW = 32 * KB;   // keys per wave: KB blocks of 32, every Q / dO fragment read from LDS serves KB MFMAs
+  constexpr int KW = NW * KPW;
+  constexpr int RT = KB > 1 ? 32 : 64;  // query rows per tile
   constexpr int QLD = D + NSA_LDS_PAD;
   constexpr int OLD = VD + NSA_LDS_PAD;
   constexpr int T_INVALID = -0x40000000;
@@ -31,6 +32,10 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
   __shared__ __attribute__((aligned(16))) float lse_s[RT];
   __shared__ __attribute__((aligned(16))) float delta_s[RT];
   __shared__ __attribute__((aligned(16))) int t_s[RT];
+  // KB > 1: the V rows of the workgroup's keys live in LDS (dP = dO V^T reads its B fragments from there), which
+  // leaves the registers to the 2*KB accumulator blocks and the K fragments
+  constexpr bool V_LDS = KB > 1;
+  __shared__ __attribute__((aligned(16))) bf16_t Vk[V_LDS ? KW * OLD : 8];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -105,27 +110,40 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
   if (row_begin >= row_end) return;
 
   // ---- this wave's keys: K and V fragments as B operands ----
-  const int kw0 = key0 + wave * 32;
-  const int my_key = kw0 + l32;
-  bf16x8 kf[D / 16], vf[VD / 16];
-  {
-    const int kr = min(my_key, nkeys - 1);
+  const int kw0 = key0 + wave * KPW;
+  bf16x8 kf[KB][D / 16], vf[V_LDS ? 1 : KB][VD / 16];
+#pragma unroll
+  for (int kb = 0; kb < KB; kb++) {
+    const int kr = min(kw0 + kb * 32 + l32, nkeys - 1);
     const bf16_t* kp = p.k + ((int64_t)kbase + kr) * p.k_sr + (int64_t)kh * p.k_sh + hl * 8;
 #pragma unroll
-    for (int kc = 0; kc < D / 16; kc++) kf[kc] = ld_global_b128(kp + kc * 16);
-    const bf16_t* vp = p.v + ((int64_t)kbase + kr) * p.v_sr + (int64_t)kh * p.v_sh + hl * 8;
+    for (int kc = 0; kc < D / 16; kc++) kf[kb][kc] = ld_global_b128(kp + kc * 16);
+    if (!V_LDS) {
+      const bf16_t* vp = p.v + ((int64_t)kbase + kr) * p.v_sr + (int64_t)kh * p.v_sh + hl * 8;
 #pragma unroll
-    for (int kc = 0; kc < VD / 16; kc++) vf[kc] = ld_global_b128(vp + kc * 16);
+      for (int kc = 0; kc < VD / 16; kc++) vf[kb][kc] = ld_global_b128(vp + kc * 16);
+    }
   }
-  f32x16 dkacc[D / 32], dvacc[VD / 32];
+  if (V_LDS) {
+    constexpr int VP = VD / 8;
+    for (int pc = tid; pc < KW * VP; pc += NT) {
+      const int kr = min(key0 + pc / VP, nkeys - 1);
+      *reinterpret_cast<bf16x8*>(&Vk[(pc / VP) * OLD + (pc % VP) * 8]) =
+          ld_global_b128(p.v + ((int64_t)kbase + kr) * p.v_sr + (int64_t)kh * p.v_sh + (pc % VP) * 8);
+    }
+  }
+  f32x16 dkacc[KB][D / 32], dvacc[KB][VD / 32];
 #pragma unroll
-  for (int dt = 0; dt < D / 32; dt++)
+  for (int kb = 0; kb < KB; kb++) {
 #pragma unroll
-    for (int i = 0; i < 16; i++) dkacc[dt][i] = 0.f;
+    for (int dt = 0; dt < D / 32; dt++)
 #pragma unroll
-  for (int dt = 0; dt < VD / 32; dt++)
+      for (int i = 0; i < 16; i++) dkacc[kb][dt][i] = 0.f;
 #pragma unroll
-    for (int i = 0; i < 16; i++) dvacc[dt][i] = 0.f;
+    for (int dt = 0; dt < VD / 32; dt++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) dvacc[kb][dt][i] = 0.f;
+  }
   const float sc = p.scale_log2;
   const bool wave_has_keys = kw0 < nkeys;
 
@@ -210,33 +228,63 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
       tsn = list[n];
     }
   };
+  // Range-keyed modes with a power-of-two group: a thread's rows advance by a whole number of tokens per tile, so
+  // its global addresses advance by a constant; the loop then needs one 64-bit add per load instead of the
+  // (token, head) -> address arithmetic.  Partial tiles (only the last one) take the general path.
+  const bool ptr_mode = (MODE != MODE_SLC) && fastG;
+  const bf16_t* qptr[QJ];
+  const bf16_t* optr[OJ];
+  const float* lptr = p.lse;
+  const float* dptr = p.delta;
+  if (ptr_mode) {
+#pragma unroll
+    for (int j = 0; j < QJ; j++) qptr[j] = p.q + (int64_t)(x0 + qn[j]) * p.q_st + qoffs[j];
+#pragma unroll
+    for (int j = 0; j < OJ; j++) optr[j] = p.dO + (int64_t)(x0 + on[j]) * p.do_st + ooffs[j];
+    lptr = p.lse + (int64_t)(x0 + sn) * p.lse_st + (int64_t)(kh * G + sg) * p.lse_sh;
+    dptr = p.delta + (int64_t)(x0 + sn) * p.delta_st + (int64_t)(kh * G + sg) * p.delta_sh;
+  }
+  const int64_t q_step = (int64_t)n_step * p.q_st, o_step = (int64_t)n_step * p.do_st;
+  const int64_t l_step = (int64_t)n_step * p.lse_st, d_step = (int64_t)n_step * p.delta_st;
   auto gload = [&](int rt0) {
+    if (ptr_mode && rt0 + RT <= row_end) {
 #pragma unroll
-    for (int j = 0; j < QJ; j++) {
-      int pc = tid + j * NT, n;
-      int64_t off;
-      locate(rt0, pc / QP, qn[j], qoffs[j], qoff_last, (pc % QP) * 8, p.q_sh, n, off);
-      if (MODE == MODE_SLC) n = tq[j];
-      qreg[j] = ld_global_b128(p.q + (int64_t)(x0 + n) * p.q_st + off);
-    }
+      for (int j = 0; j < QJ; j++) qreg[j] = ld_global_b128(qptr[j]);
 #pragma unroll
-    for (int j = 0; j < OJ; j++) {
-      int pc = tid + j * NT, n;
-      int64_t off;
-      locate(rt0, pc / OP, on[j], ooffs[j], ooff_last, (pc % OP) * 8, p.do_sh, n, off);
-      if (MODE == MODE_SLC) n = (QP == OP) ? tq[j] : to[j];
-      oreg[j] = ld_global_b128(p.dO + (int64_t)(x0 + n) * p.do_st + off);
-    }
-    if (tid < RT) {
-      const bool ok = rt0 + tid <= row_last;
-      int n;
-      int64_t hoff;
-      locate(rt0, tid, sn, (int64_t)(kh * G + sg), (int64_t)(kh * G + g_lastrow), 0, 1, n, hoff);
-      if (MODE == MODE_SLC) n = tsn;
-      const int64_t tok = x0 + n;
-      lse_reg = p.lse[tok * p.lse_st + hoff * p.lse_sh];
-      delta_reg = p.delta[tok * p.delta_st + hoff * p.delta_sh];
-      t_reg = ok ? n : T_INVALID;
+      for (int j = 0; j < OJ; j++) oreg[j] = ld_global_b128(optr[j]);
+      if (tid < RT) {
+        lse_reg = *lptr;
+        delta_reg = *dptr;
+        t_reg = sn;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < QJ; j++) {
+        int pc = tid + j * NT, n;
+        int64_t off;
+        locate(rt0, pc / QP, qn[j], qoffs[j], qoff_last, (pc % QP) * 8, p.q_sh, n, off);
+        if (MODE == MODE_SLC) n = tq[j];
+        qreg[j] = ld_global_b128(p.q + (int64_t)(x0 + n) * p.q_st + off);
+      }
+#pragma unroll
+      for (int j = 0; j < OJ; j++) {
+        int pc = tid + j * NT, n;
+        int64_t off;
+        locate(rt0, pc / OP, on[j], ooffs[j], ooff_last, (pc % OP) * 8, p.do_sh, n, off);
+        if (MODE == MODE_SLC) n = (QP == OP) ? tq[j] : to[j];
+        oreg[j] = ld_global_b128(p.dO + (int64_t)(x0 + n) * p.do_st + off);
+      }
+      if (tid < RT) {
+        const bool ok = rt0 + tid <= row_last;
+        int n;
+        int64_t hoff;
+        locate(rt0, tid, sn, (int64_t)(kh * G + sg), (int64_t)(kh * G + g_lastrow), 0, 1, n, hoff);
+        if (MODE == MODE_SLC) n = tsn;
+        const int64_t tok = x0 + n;
+        lse_reg = p.lse[tok * p.lse_st + hoff * p.lse_sh];
+        delta_reg = p.delta[tok * p.delta_st + hoff * p.delta_sh];
+        t_reg = ok ? n : T_INVALID;
+      }
     }
     // advance the bookkeeping to the next tile, then start fetching that tile's tokens
 #pragma unroll
@@ -244,6 +292,14 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
 #pragma unroll
     for (int j = 0; j < OJ; j++) on[j] += n_step;
     sn += n_step;
+    if (ptr_mode) {
+#pragma unroll
+      for (int j = 0; j < QJ; j++) qptr[j] += q_step;
+#pragma unroll
+      for (int j = 0; j < OJ; j++) optr[j] += o_step;
+      lptr += l_step;
+      dptr += d_step;
+    }
     if (rt0 + RT < row_end) fetch_tokens(rt0 + RT);
   };
   fetch_tokens(row_begin);
@@ -275,39 +331,58 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
     const int t_min = __builtin_amdgcn_readfirstlane(t_s[0]);
     const int t_max = __builtin_amdgcn_readfirstlane(t_s[n_in - 1]);
     bool any_vis, full_vis;
+    constexpr int KL = KPW - 1;  // offset of the wave's last key
     if (MODE == MODE_CMP) {
       any_vis = t_max >= p.stride * kw0 + p.kernel_size - 1;
-      full_vis = (n_in == RT) && (t_min >= p.stride * (kw0 + 31) + p.kernel_size - 1) && (kw0 + 31 < nkeys);
+      full_vis = (n_in == RT) && (t_min >= p.stride * (kw0 + KL) + p.kernel_size - 1) && (kw0 + KL < nkeys);
     } else if (MODE == MODE_SWA) {
-      any_vis = (kw0 <= t_max) && (kw0 + 31 >= t_min - p.window);
-      full_vis = (n_in == RT) && (kw0 + 31 <= t_min) && (kw0 >= t_max - p.window) && (kw0 + 31 < nkeys);
+      any_vis = (kw0 <= t_max) && (kw0 + KL >= t_min - p.window);
+      full_vis = (n_in == RT) && (kw0 + KL <= t_min) && (kw0 >= t_max - p.window) && (kw0 + KL < nkeys);
     } else {
       any_vis = kw0 <= t_max;
-      full_vis = (n_in == RT) && (kw0 + 31 <= t_min) && (kw0 + 31 < nkeys);
+      full_vis = (n_in == RT) && (kw0 + KL <= t_min) && (kw0 + KL < nkeys);
     }
     if (!any_vis) continue;
 
 #pragma unroll
-    for (int mt = 0; mt < 2; mt++) {
-      f32x16 sacc, pacc;
+    for (int mt = 0; mt < RT / 32; mt++) {
+      f32x16 sacc[KB], pacc[KB];
 #pragma unroll
-      for (int i = 0; i < 16; i++) { sacc[i] = 0.f; pacc[i] = 0.f; }
+      for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) { sacc[kb][i] = 0.f; pacc[kb][i] = 0.f; }
       const bf16_t* qp = &Qs[(mt * 32 + l32) * QLD + hl * 8];
       const bf16_t* dp = &dOs[(mt * 32 + l32) * OLD + hl * 8];
 #pragma unroll
-      for (int kc = 0; kc < D / 16; kc++)
-        sacc = mfma32(*reinterpret_cast<const bf16x8*>(qp + kc * 16), kf[kc], sacc);
+      for (int kc = 0; kc < D / 16; kc++) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(qp + kc * 16);
 #pragma unroll
-      for (int kc = 0; kc < VD / 16; kc++)
-        pacc = mfma32(*reinterpret_cast<const bf16x8*>(dp + kc * 16), vf[kc], pacc);
+        for (int kb = 0; kb < KB; kb++) sacc[kb] = mfma32(a, kf[kb][kc], sacc[kb]);
+      }
+#pragma unroll
+      for (int kc = 0; kc < VD / 16; kc++) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(dp + kc * 16);
+#pragma unroll
+        for (int kb = 0; kb < KB; kb++) {
+          if (V_LDS) {
+            const bf16x8 bv =
+                *reinterpret_cast<const bf16x8*>(&Vk[(wave * KPW + kb * 32 + l32) * OLD + hl * 8 + kc * 16]);
+            pacc[kb] = mfma32(a, bv, pacc[kb]);
+          } else {
+            pacc[kb] = mfma32(a, vf[kb][kc], pacc[kb]);
+          }
+        }
+      }
       // P = exp2(S*c - lse);  dS = P o (dP - delta)
 #pragma unroll
       for (int i4 = 0; i4 < 4; i4++) {
         const int rbase = mt * 32 + i4 * 8 + hl * 4;
         f32x4 l4 = *reinterpret_cast<const f32x4*>(&lse_s[rbase]);
 #pragma unroll
-        for (int ii = 0; ii < 4; ii++)
-          sacc[i4 * 4 + ii] = fast_exp2(__builtin_fmaf(sacc[i4 * 4 + ii], sc, -l4[ii]));
+        for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+          for (int ii = 0; ii < 4; ii++)
+            sacc[kb][i4 * 4 + ii] = fast_exp2(__builtin_fmaf(sacc[kb][i4 * 4 + ii], sc, -l4[ii]));
       }
       if (!full_vis) {  // wave-uniform: only tiles that straddle a visibility boundary pay for the mask
 #pragma unroll
@@ -316,11 +391,15 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
 #pragma unroll
           for (int ii = 0; ii < 4; ii++) {
             int tr = t_s[rbase + ii];
-            bool vis;
-            if (MODE == MODE_CMP) vis = (my_key < nkeys) && (tr >= p.stride * my_key + p.kernel_size - 1);
-            else if (MODE == MODE_SWA) vis = (my_key <= tr) && (my_key >= tr - p.window) && (my_key < nkeys);
-            else vis = (my_key <= tr) && (my_key < nkeys);
-            sacc[i4 * 4 + ii] = vis ? sacc[i4 * 4 + ii] : 0.f;
+#pragma unroll
+            for (int kb = 0; kb < KB; kb++) {
+              const int my_key = kw0 + kb * 32 + l32;
+              bool vis;
+              if (MODE == MODE_CMP) vis = (my_key < nkeys) && (tr >= p.stride * my_key + p.kernel_size - 1);
+              else if (MODE == MODE_SWA) vis = (my_key <= tr) && (my_key >= tr - p.window) && (my_key < nkeys);
+              else vis = (my_key <= tr) && (my_key < nkeys);
+              sacc[kb][i4 * 4 + ii] = vis ? sacc[kb][i4 * 4 + ii] : 0.f;
+            }
           }
         }
       }
@@ -329,14 +408,21 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
         const int rbase = mt * 32 + i4 * 8 + hl * 4;
         f32x4 d4 = *reinterpret_cast<const f32x4*>(&delta_s[rbase]);
 #pragma unroll
-        for (int ii = 0; ii < 4; ii++) pacc[i4 * 4 + ii] = sacc[i4 * 4 + ii] * (pacc[i4 * 4 + ii] - d4[ii]);
+        for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+          for (int ii = 0; ii < 4; ii++)
+            pacc[kb][i4 * 4 + ii] = sacc[kb][i4 * 4 + ii] * (pacc[kb][i4 * 4 + ii] - d4[ii]);
       }
 #pragma unroll
       for (int c = 0; c < 2; c++) {
-        bf16x8 pf = pack8(sacc[c * 8 + 0], sacc[c * 8 + 1], sacc[c * 8 + 2], sacc[c * 8 + 3], sacc[c * 8 + 4],
-                          sacc[c * 8 + 5], sacc[c * 8 + 6], sacc[c * 8 + 7]);
-        bf16x8 df = pack8(pacc[c * 8 + 0], pacc[c * 8 + 1], pacc[c * 8 + 2], pacc[c * 8 + 3], pacc[c * 8 + 4],
-                          pacc[c * 8 + 5], pacc[c * 8 + 6], pacc[c * 8 + 7]);
+        bf16x8 pf[KB], df[KB];
+#pragma unroll
+        for (int kb = 0; kb < KB; kb++) {
+          pf[kb] = pack8(sacc[kb][c * 8 + 0], sacc[kb][c * 8 + 1], sacc[kb][c * 8 + 2], sacc[kb][c * 8 + 3],
+                         sacc[kb][c * 8 + 4], sacc[kb][c * 8 + 5], sacc[kb][c * 8 + 6], sacc[kb][c * 8 + 7]);
+          df[kb] = pack8(pacc[kb][c * 8 + 0], pacc[kb][c * 8 + 1], pacc[kb][c * 8 + 2], pacc[kb][c * 8 + 3],
+                         pacc[kb][c * 8 + 4], pacc[kb][c * 8 + 5], pacc[kb][c * 8 + 6], pacc[kb][c * 8 + 7]);
+        }
         const int rb0 = mt * 32 + (2 * c) * 8 + hl * 4 + (i16 >> 2);
         const int rb1 = rb0 + 8;
 #pragma unroll
@@ -344,23 +430,22 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
           const int col = dt * 32 + (g16 & 1) * 16 + 4 * (i16 & 3);
           bf16x4 a0 = lds_read_tr(&dOs[rb0 * OLD + col]);
           bf16x4 a1 = lds_read_tr(&dOs[rb1 * OLD + col]);
-          dvacc[dt] = mfma32(cat4(a0, a1), pf, dvacc[dt]);
+#pragma unroll
+          for (int kb = 0; kb < KB; kb++) dvacc[kb][dt] = mfma32(cat4(a0, a1), pf[kb], dvacc[kb][dt]);
         }
 #pragma unroll
         for (int dt = 0; dt < D / 32; dt++) {
           const int col = dt * 32 + (g16 & 1) * 16 + 4 * (i16 & 3);
           bf16x4 a0 = lds_read_tr(&Qs[rb0 * QLD + col]);
           bf16x4 a1 = lds_read_tr(&Qs[rb1 * QLD + col]);
-          dkacc[dt] = mfma32(cat4(a0, a1), df, dkacc[dt]);
+#pragma unroll
+          for (int kb = 0; kb < KB; kb++) dkacc[kb][dt] = mfma32(cat4(a0, a1), df[kb], dkacc[kb][dt]);
         }
       }
     }
   }
 
-  if (my_key >= nkeys) return;
   const float osc = p.sm_scale;
-  const int64_t koff = ((int64_t)kbase + my_key) * p.dk_sr + (int64_t)kh * p.dk_sh;
-  const int64_t voff = ((int64_t)kbase + my_key) * p.dv_sr + (int64_t)kh * p.dv_sh;
   auto emit = [&](void* base, int64_t off, f32x4 val) {
     if (p.dkv_mode == 0) {
       *reinterpret_cast<bf16x4*>((bf16_t*)base + off) = pack4(val[0], val[1], val[2], val[3]);
@@ -373,47 +458,62 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
     }
   };
 #pragma unroll
-  for (int dt = 0; dt < D / 32; dt++)
+  for (int kb = 0; kb < KB; kb++) {
+    const int my_key = kw0 + kb * 32 + l32;
+    if (my_key >= nkeys) continue;
+    const int64_t koff = ((int64_t)kbase + my_key) * p.dk_sr + (int64_t)kh * p.dk_sh;
+    const int64_t voff = ((int64_t)kbase + my_key) * p.dv_sr + (int64_t)kh * p.dv_sh;
 #pragma unroll
-    for (int i4 = 0; i4 < 4; i4++) {
-      int d = dt * 32 + i4 * 8 + hl * 4;
-      emit(p.dk, koff + d, f32x4{dkacc[dt][i4 * 4 + 0] * osc, dkacc[dt][i4 * 4 + 1] * osc,
-                                 dkacc[dt][i4 * 4 + 2] * osc, dkacc[dt][i4 * 4 + 3] * osc});
-    }
+    for (int dt = 0; dt < D / 32; dt++)
 #pragma unroll
-  for (int dt = 0; dt < VD / 32; dt++)
+      for (int i4 = 0; i4 < 4; i4++) {
+        int d = dt * 32 + i4 * 8 + hl * 4;
+        emit(p.dk, koff + d, f32x4{dkacc[kb][dt][i4 * 4 + 0] * osc, dkacc[kb][dt][i4 * 4 + 1] * osc,
+                                   dkacc[kb][dt][i4 * 4 + 2] * osc, dkacc[kb][dt][i4 * 4 + 3] * osc});
+      }
 #pragma unroll
-    for (int i4 = 0; i4 < 4; i4++) {
-      int d = dt * 32 + i4 * 8 + hl * 4;
-      emit(p.dv, voff + d, f32x4{dvacc[dt][i4 * 4 + 0], dvacc[dt][i4 * 4 + 1], dvacc[dt][i4 * 4 + 2],
-                                 dvacc[dt][i4 * 4 + 3]});
-    }
+    for (int dt = 0; dt < VD / 32; dt++)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; i4++) {
+        int d = dt * 32 + i4 * 8 + hl * 4;
+        emit(p.dv, voff + d, f32x4{dvacc[kb][dt][i4 * 4 + 0], dvacc[kb][dt][i4 * 4 + 1], dvacc[kb][dt][i4 * 4 + 2],
+                                   dvacc[kb][dt][i4 * 4 + 3]});
+      }
+  }
 }
 
 template <int D, int VD>
 int launch(const NsaBwdTileParams& p0, int mode, int B, int max_q_len, int max_k_len, int n_items_bound,
            hipStream_t stream) {
   NsaBwdTileParams p = p0;
+  static const int kb_cmp = nsa_tuning_knob("NSA_DKDV_KB", 1);  // 32-key blocks per wave of the cmp / swa kernels
   if (mode == MODE_CMP) {
     if (B <= 0 || max_k_len <= 0) return NSA_OK;
+    const int KW = 4 * 32 * (kb_cmp == 2 ? 2 : 1);
     const int nch = cdiv_i(max_q_len, p.q_chunk_tokens);
     int total = 0;
-    for (int kt = 0; kt * 128 < max_k_len; kt++)
-      total += nch - (nch < (p.stride * kt * 128 + p.kernel_size - 1) / p.q_chunk_tokens
-                          ? nch
-                          : (p.stride * kt * 128 + p.kernel_size - 1) / p.q_chunk_tokens);
+    for (int kt = 0; kt * KW < max_k_len; kt++) {
+      const int fc = (p.stride * kt * KW + p.kernel_size - 1) / p.q_chunk_tokens;
+      total += nch - (nch < fc ? nch : fc);
+    }
     if (total <= 0) return NSA_OK;
     dim3 grid(total, B, p.KH);
-    bwd_dkdv_kernel<D, VD, MODE_CMP, 4><<<grid, 256, 0, stream>>>(p);
+    if (kb_cmp == 2) bwd_dkdv_kernel<D, VD, MODE_CMP, 4, 2><<<grid, 256, 0, stream>>>(p);
+    else bwd_dkdv_kernel<D, VD, MODE_CMP, 4, 1><<<grid, 256, 0, stream>>>(p);
   } else if (mode == MODE_SWA) {
     if (B <= 0 || max_k_len <= 0) return NSA_OK;
-    dim3 grid(cdiv_i(max_k_len, 128), B, p.KH);
-    bwd_dkdv_kernel<D, VD, MODE_SWA, 4><<<grid, 256, 0, stream>>>(p);
+    if (kb_cmp == 2) {
+      dim3 grid(cdiv_i(max_k_len, 256), B, p.KH);
+      bwd_dkdv_kernel<D, VD, MODE_SWA, 4, 2><<<grid, 256, 0, stream>>>(p);
+    } else {
+      dim3 grid(cdiv_i(max_k_len, 128), B, p.KH);
+      bwd_dkdv_kernel<D, VD, MODE_SWA, 4, 1><<<grid, 256, 0, stream>>>(p);
+    }
   } else {
     if (n_items_bound <= 0) return NSA_OK;
     dim3 grid(n_items_bound, 1, p.KH);
-    if (p.block_size == 64) bwd_dkdv_kernel<D, VD, MODE_SLC, 2><<<grid, 128, 0, stream>>>(p);
-    else if (p.block_size == 128) bwd_dkdv_kernel<D, VD, MODE_SLC, 4><<<grid, 256, 0, stream>>>(p);
+    if (p.block_size == 64) bwd_dkdv_kernel<D, VD, MODE_SLC, 2, 1><<<grid, 128, 0, stream>>>(p);
+    else if (p.block_size == 128) bwd_dkdv_kernel<D, VD, MODE_SLC, 4, 1><<<grid, 256, 0, stream>>>(p);
     else {
       nsa_set_error("selected attention dk/dv: block_size %d not built (64 or 128)", p.block_size);
       return NSA_ERR_UNSUPPORTED;
