@@ -9,6 +9,9 @@ compressed K for the importance pass is an implementation choice and is not coun
 import torch
 
 PEAK_HBM_GBS = 8000.0
+# bytes per step crossing the L2 <-> memory-side boundary (rocprofv3 --pmc FETCH_SIZE x2.000 + WRITE_SIZE x1.000, the
+# factors being what the counters read for a 1 GiB copy), measured for the default case of build_case()
+MEASURED_TRAFFIC_DEFAULT_CASE = 333.8e6
 
 
 def build_case(dev, B=64, QH=64, KH=4, D=128, page=256, lo=4096, hi=32768, seed=3):
@@ -105,7 +108,7 @@ def decode_bench(dev, reps=200, warmup=20):
                         "d=128, bf16, hipGraph replay", "us_per_step": us, "eager_us_per_step": eager_us,
             "graph_equals_eager": same, "algorithmic_bytes": nbytes,
             "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                         "frac": gbs / PEAK_HBM_GBS, "traffic": None}}
+                         "frac": gbs / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_DEFAULT_CASE}}
 
 
 if __name__ == "__main__":
