@@ -289,3 +289,32 @@ def test_one_launch_decode_pools_the_new_row_itself(device):
                            cmp_slot_mapping=slots.to(device))
     assert torch.equal(d1["k"], d2["k"]) and torch.equal(d1["v"], d2["v"])
     assert torch.equal(o1, o2)
+
+
+def test_decode_qk192_v128_equals_training_last_row(device):
+    """Dqk = 192, Dv = 128, 2 kv heads (the head shape of upstream's inference notebook, cell 43): nsa_decode takes
+    the stage-by-stage kernels here; its output equals the last row of the training forward on the gathered
+    contiguous sequence."""
+    from flash_nsa import nsa_decode, NSAConfig, NSACore
+    QH, KH, D, VD = 16, 2, 192, 128
+    ctx = [1000, 333, 64, 2049]
+    case = build_pool(ctx, KH, D, VD, page=128, seed=51)
+    prepool(case, [L - 1 for L in ctx])
+    slots = decode_slot_mapping(case)
+    B = len(ctx)
+    q, w = randn_bf16(B, QH, D, seed=52), randn_bf16(B, QH, 3, seed=53)
+    d = to_dev(case, device)
+    ctx_t = torch.tensor(ctx, dtype=torch.int32, device=device)
+    o = nsa_decode(q.to(device), d["k"], d["v"], w.to(device), ctx_t, d["bt"], slots.to(device), d["cbt"],
+                   fixed_y_maxlen=256, fixed_num_slc_blocks=64)
+    assert o.shape == (B, QH, VD) and torch.isfinite(o).all()
+    core = NSACore(NSAConfig(qk_head_dim=D, v_head_dim=VD, num_heads=QH, num_kv_heads=KH))
+    for b in range(B):
+        L = ctx[b]
+        ks = O.gather_rows(case["k"], case["bt"][b], L).to(device)
+        vs = O.gather_rows(case["v"], case["bt"][b], L).to(device)
+        qs, ws = randn_bf16(L, QH, D, seed=300 + b), randn_bf16(L, QH, 3, seed=400 + b)
+        qs[-1], ws[-1] = q[b], w[b]
+        with torch.no_grad():
+            full = core(qs.to(device), ks, vs, ws.to(device), torch.tensor([0, L], dtype=torch.int32, device=device))
+        assert_close(o[b], full[-1], f"decode vs training row (request {b})", atol=1e-2, rtol=1e-2)
