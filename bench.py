@@ -137,9 +137,11 @@ def staged_step(timer, q, k, v, w, wv, do, sm_scale):
                                     bind["chunk_tokens"], bind["n_items_bound"], H.batch, QH, KH, D, VD,
                                     H.block_size, sm_scale, st))
     cc = common(cmp_k, cmp_v, cmp_lse, cmp_lse.stride(1), cmp_lse.stride(0), delta[0], dcmp_o)
-    R("cmp_dq", lambda: _lib.call("nsa_cmp_attn_bwd_dq", *cc, dq.data_ptr(), dq.stride(0), dq.stride(1), 2,
-                                  H.x_cu_seqlens.data_ptr(), H.y_cu_seqlens.data_ptr(), H.batch, H.x_maxlen, QH, KH,
-                                  D, VD, H.kernel_size, H.stride, sm_scale, st))
+    dq_out = torch.empty_like(q)  # the last dq kernel adds the fp32 partial sum and stores q's dtype
+    R("cmp_dq", lambda: _lib.call("nsa_cmp_attn_bwd_dq_final", *cc, dq.data_ptr(), dq.stride(0), dq.stride(1),
+                                  dq_out.data_ptr(), dq_out.stride(0), dq_out.stride(1), H.x_cu_seqlens.data_ptr(),
+                                  H.y_cu_seqlens.data_ptr(), H.batch, H.x_maxlen, QH, KH, D, VD, H.kernel_size,
+                                  H.stride, sm_scale, st))
     dck = torch.zeros(cmp_k.shape, device=q.device, dtype=torch.float32)
     dcv = torch.zeros(cmp_v.shape, device=q.device, dtype=torch.float32)
     R("cmp_dkdv", lambda: _lib.call("nsa_cmp_attn_bwd_dkdv", *cc, dck.data_ptr(), dck.stride(0), dck.stride(1),
@@ -155,7 +157,6 @@ def staged_step(timer, q, k, v, w, wv, do, sm_scale):
         return torch.matmul(dhid.flatten(0, 1).t(), win_v.flatten(-2, -1).flatten(0, 1))
 
     R("cmp_v_bwd", cmp_v_bwd)
-    R("dq_cast", lambda: dq.to(q.dtype))
 
 
 def cpu_baseline(min_seconds=12.0):

@@ -90,6 +90,17 @@ int nsa_cmp_attn_bwd_dq(const void* q, int64_t q_st, int64_t q_sh, const void* c
                         int64_t delta_sh, void* dq, int64_t dq_st, int64_t dq_sh, int dq_mode, const int32_t* x_cu,
                         const int32_t* y_cu, int B, int x_maxlen, int QH, int KH, int D, int VD, int kernel_size,
                         int stride, float sm_scale, void* stream);
+/* Same kernel as nsa_cmp_attn_bwd_dq, as the LAST branch of the fused backward
+ * (flash_nsa/modules/megatron_level_nsa.py:129-159 accumulates the three branches' dq and returns it in q's dtype):
+ * dq [T,QH,D] bf16 = this branch's dq + dq_partial (fp32, the sum of the other branches), which saves the fp32
+ * read-modify-write and the separate cast pass. */
+int nsa_cmp_attn_bwd_dq_final(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr,
+                              int64_t ck_sh, const void* cv, int64_t cv_sr, int64_t cv_sh, const void* dO,
+                              int64_t do_st, int64_t do_sh, const float* lse, int64_t lse_st, int64_t lse_sh,
+                              const float* delta, int64_t delta_st, int64_t delta_sh, const float* dq_partial,
+                              int64_t dqp_st, int64_t dqp_sh, void* dq, int64_t dq_st, int64_t dq_sh,
+                              const int32_t* x_cu, const int32_t* y_cu, int B, int x_maxlen, int QH, int KH, int D,
+                              int VD, int kernel_size, int stride, float sm_scale, void* stream);
 /* flash_nsa/ops/compress_attn.py:650-690 (_cmp_dkdv_kernel launch, dkdv_repeat=False): fp32 atomic adds into
  * dck/dcv [y_len,KH,*], which the caller zero-fills; queries are cut into chunks of q_chunk_tokens */
 int nsa_cmp_attn_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr, int64_t ck_sh,

@@ -176,24 +176,47 @@ NsaBwdTileParams make_bwd(const BwdCommon& c, int QH, int KH, float sm_scale) {
 
 extern "C" {
 
+static int cmp_bwd_dq_impl(const char* who, const BwdCommon& c, void* dq, int64_t dq_st, int64_t dq_sh, int dq_mode,
+                           const float* dq_partial, int64_t dqp_st, int64_t dqp_sh, const int32_t* x_cu,
+                           const int32_t* y_cu, int B, int x_maxlen, int QH, int KH, int D, int VD, int kernel_size,
+                           int stride, float sm_scale, void* stream) {
+  int rc = check_heads(who, QH, KH, D, VD);
+  if (rc) return rc;
+  rc = check_nsa_sizes(who, kernel_size, stride, 0);
+  if (rc) return rc;
+  NsaBwdTileParams p = make_bwd(c, QH, KH, sm_scale);
+  p.dq = dq; p.dq_st = dq_st; p.dq_sh = dq_sh; p.dq_mode = dq_mode;
+  p.dq_partial = dq_partial; p.dqp_st = dqp_st; p.dqp_sh = dqp_sh;
+  p.x_cu = x_cu; p.k_cu = y_cu;
+  p.kernel_size = kernel_size; p.stride = stride;
+  return nsa_bwd_dq_tile_launch(p, 0, B, x_maxlen, D, VD, (hipStream_t)stream);
+}
+
 int nsa_cmp_attn_bwd_dq(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr, int64_t ck_sh,
                         const void* cv, int64_t cv_sr, int64_t cv_sh, const void* dO, int64_t do_st, int64_t do_sh,
                         const float* lse, int64_t lse_st, int64_t lse_sh, const float* delta, int64_t delta_st,
                         int64_t delta_sh, void* dq, int64_t dq_st, int64_t dq_sh, int dq_mode, const int32_t* x_cu,
                         const int32_t* y_cu, int B, int x_maxlen, int QH, int KH, int D, int VD, int kernel_size,
                         int stride, float sm_scale, void* stream) {
-  int rc = check_heads("cmp_attn_bwd_dq", QH, KH, D, VD);
-  if (rc) return rc;
-  rc = check_nsa_sizes("cmp_attn_bwd_dq", kernel_size, stride, 0);
-  if (rc) return rc;
   NSA_REQUIRE(dq_mode >= 0 && dq_mode <= 2, NSA_ERR_BAD_ARG, "cmp_attn_bwd_dq: dq_mode %d not in {0,1,2}", dq_mode);
   BwdCommon c{q, q_st, q_sh, ck, ck_sr, ck_sh, cv, cv_sr, cv_sh, dO, do_st, do_sh, lse, lse_st, lse_sh, delta,
               delta_st, delta_sh};
-  NsaBwdTileParams p = make_bwd(c, QH, KH, sm_scale);
-  p.dq = dq; p.dq_st = dq_st; p.dq_sh = dq_sh; p.dq_mode = dq_mode;
-  p.x_cu = x_cu; p.k_cu = y_cu;
-  p.kernel_size = kernel_size; p.stride = stride;
-  return nsa_bwd_dq_tile_launch(p, 0, B, x_maxlen, D, VD, (hipStream_t)stream);
+  return cmp_bwd_dq_impl("cmp_attn_bwd_dq", c, dq, dq_st, dq_sh, dq_mode, nullptr, 0, 0, x_cu, y_cu, B, x_maxlen, QH,
+                         KH, D, VD, kernel_size, stride, sm_scale, stream);
+}
+
+int nsa_cmp_attn_bwd_dq_final(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr,
+                              int64_t ck_sh, const void* cv, int64_t cv_sr, int64_t cv_sh, const void* dO,
+                              int64_t do_st, int64_t do_sh, const float* lse, int64_t lse_st, int64_t lse_sh,
+                              const float* delta, int64_t delta_st, int64_t delta_sh, const float* dq_partial,
+                              int64_t dqp_st, int64_t dqp_sh, void* dq, int64_t dq_st, int64_t dq_sh,
+                              const int32_t* x_cu, const int32_t* y_cu, int B, int x_maxlen, int QH, int KH, int D,
+                              int VD, int kernel_size, int stride, float sm_scale, void* stream) {
+  NSA_REQUIRE(dq_partial != nullptr && dq != nullptr, NSA_ERR_BAD_ARG, "cmp_attn_bwd_dq_final: null dq buffers");
+  BwdCommon c{q, q_st, q_sh, ck, ck_sr, ck_sh, cv, cv_sr, cv_sh, dO, do_st, do_sh, lse, lse_st, lse_sh, delta,
+              delta_st, delta_sh};
+  return cmp_bwd_dq_impl("cmp_attn_bwd_dq_final", c, dq, dq_st, dq_sh, 3, dq_partial, dqp_st, dqp_sh, x_cu, y_cu, B,
+                         x_maxlen, QH, KH, D, VD, kernel_size, stride, sm_scale, stream);
 }
 
 int nsa_cmp_attn_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr, int64_t ck_sh,

@@ -63,7 +63,9 @@ struct NsaBwdTileParams {
   const bf16_t* dO; int64_t do_st, do_sh;
   const float* lse; int64_t lse_st, lse_sh;
   const float* delta; int64_t delta_st, delta_sh;
-  void* dq; int64_t dq_st, dq_sh; int dq_mode;      // 0: store bf16, 1: store fp32, 2: add into fp32
+  void* dq; int64_t dq_st, dq_sh; int dq_mode;      // 0: store bf16, 1: store fp32, 2: add into fp32,
+                                                    // 3 (dq tile kernel): bf16 store of (result + fp32 dq_partial)
+  const float* dq_partial; int64_t dqp_st, dqp_sh;
   void* dk; int64_t dk_sr, dk_sh;                   // dkdv kernels
   void* dv; int64_t dv_sr, dv_sh;
   int dkv_mode;                                     // 0: store bf16, 1: store fp32, 3: atomic add into fp32

@@ -214,6 +214,9 @@ __global__ __launch_bounds__(256, MINB) void bwd_dq_tile_kernel(NsaBwdTileParams
                    dqacc[dt][i4 * 4 + 3] * osc};
       if (p.dq_mode == 0) {
         *reinterpret_cast<bf16x4*>((bf16_t*)p.dq + off + d) = pack4(val[0], val[1], val[2], val[3]);
+      } else if (p.dq_mode == 3) {
+        val += *reinterpret_cast<const f32x4*>(p.dq_partial + tok * p.dqp_st + (int64_t)head * p.dqp_sh + d);
+        *reinterpret_cast<bf16x4*>((bf16_t*)p.dq + off + d) = pack4(val[0], val[1], val[2], val[3]);
       } else {
         float* dst = (float*)p.dq + off + d;
         if (p.dq_mode == 2) val += *reinterpret_cast<f32x4*>(dst);

@@ -121,11 +121,11 @@ class NSAFunction(torch.autograd.Function):
                             dq=_store_into(dq), dkv_fp32=True)
         slc_attn_bwd(q, k, v, topk, slc_o, slc_lse, dslc_o, dq, dk, dv, sm_scale=sm_scale, helper=helper,
                      delta=delta[1])
-        _, dcmp_k, dcmp_v = cmp_attn_bwd(q, cmp_k, cmp_v, cmp_o, cmp_lse, dcmp_o, dq, sm_scale=sm_scale,
-                                         helper=helper, delta=delta[0])
+        dq, dcmp_k, dcmp_v = cmp_attn_bwd(q, cmp_k, cmp_v, cmp_o, cmp_lse, dcmp_o, dq, sm_scale=sm_scale,
+                                          helper=helper, delta=delta[0], finalize_dq=True)
         _, dwk = compress_kv_bwd(k, cmp_k_weight, win_k, hid_k, dcmp_k, dk, k_method, helper)
         _, dwv = compress_kv_bwd(v, cmp_v_weight, win_v, hid_v, dcmp_v, dv, v_method, helper)
-        return dq.to(q.dtype), dk, dv, dw, dwk, dwv, None
+        return dq, dk, dv, dw, dwk, dwv, None
 
 
 class _StoreTarget:
