@@ -1,7 +1,7 @@
 // dQ of selected-block attention: one wave per (query token, kv head), 16 q-heads as the MFMA N dimension.
 //   S^T = K Q^T,  P^T = exp2(S^T*c - lse),  dP^T = V dO^T,  dS^T = P^T o (dP^T - delta),  dQ^T += K^T dS^T
-// K is staged row-major in a wave-private LDS region (read both as row fragments and, transposed, through
-// ds_read_b64_tr_b16); V fragments are loaded straight from global memory.
+// K and V rows are staged row-major in wave-private LDS regions (K is read both as row fragments and, transposed,
+// through ds_read_b64_tr_b16; V as row fragments).
 // Upstream: flash_nsa/ops/select_attn.py:336-437 (_dq_kernel).
 #include "nsa_common.h"
 #include "nsa_api_internal.h"

@@ -2,10 +2,10 @@
 // (up to 16) q-heads that share the kv head, N is 16 keys, v_mfma_f32_16x16x32_bf16.
 // Upstream: flash_nsa/ops/select_attn.py:21-108 (training), flash_nsa/inference/select_attn.py:21-100 (paged).
 //
-// K fragments are loaded straight from global memory into the A operand (the contraction index d is contiguous
-// in a key row); V is staged row-major in a wave-private LDS region and read back through
-// ds_read_b64_tr_b16, which delivers the key-contraction slices.  Keys are gathered by the per-token block
-// list topk[kh, t, 0 .. min(top_n, t/block+1)).
+// The keys of the selected blocks are processed in units of 32.  The K and V rows of a unit are fetched as whole
+// coalesced rows (16 lanes x 16 bytes per row) into registers one unit ahead, pass through wave-private LDS
+// regions, and are read back as MFMA fragments (K row-major, V through ds_read_b64_tr_b16, which delivers the
+// key-contraction slices).  Keys are gathered by the per-token block list topk[kh, t, 0 .. min(top_n, t/block+1)).
 #include "nsa_common.h"
 #include "nsa_api_internal.h"
 
