@@ -115,39 +115,38 @@ def staged_step(timer, q, k, v, w, wv, do, sm_scale):
                 vv.stride(0), vv.stride(1), dout.data_ptr(), dout.stride(0), dout.stride(1), lse.data_ptr(), lse_st,
                 lse_sh, dlt.data_ptr(), dlt.stride(0), dlt.stride(1))
 
-    st = _lib.stream_ptr()
     dk = torch.empty(T, KH, D, device=q.device, dtype=torch.float32)
     dv = torch.empty(T, KH, VD, device=q.device, dtype=torch.float32)
     cs = common(k, v, swa_lse, swa_lse.stride(0), swa_lse.stride(1), delta[2], dswa_o)
     R("swa_dq", lambda: _lib.call("nsa_swa_bwd_dq", *cs, dq.data_ptr(), dq.stride(0), dq.stride(1), 1,
                                   H.x_cu_seqlens.data_ptr(), H.batch, H.x_maxlen, QH, KH, D, VD, H.window_size,
-                                  sm_scale, st))
+                                  sm_scale, _lib.stream_ptr()))
     R("swa_dkdv", lambda: _lib.call("nsa_swa_bwd_dkdv", *cs, dk.data_ptr(), dk.stride(0), dk.stride(1),
                                     dv.data_ptr(), dv.stride(0), dv.stride(1), 1, H.x_cu_seqlens.data_ptr(), H.batch,
-                                    H.x_maxlen, QH, KH, D, VD, H.window_size, sm_scale, st))
+                                    H.x_maxlen, QH, KH, D, VD, H.window_size, sm_scale, _lib.stream_ptr()))
     cl = common(k, v, slc_lse, slc_lse.stride(0), slc_lse.stride(1), delta[1], dslc_o)
     R("slc_dq", lambda: _lib.call("nsa_slc_attn_bwd_dq", *cl, topk.data_ptr(), topk.stride(0), topk.stride(1),
                                   dq.data_ptr(), dq.stride(0), dq.stride(1), 2, H.x_cu_seqlens.data_ptr(), H.batch,
-                                  H.x_maxlen, QH, KH, D, VD, H.block_size, topk.size(-1), sm_scale, st))
+                                  H.x_maxlen, QH, KH, D, VD, H.block_size, topk.size(-1), sm_scale, _lib.stream_ptr()))
     bind = R("inverse_index", lambda: get_bind_from_find(topk))
     R("slc_dkdv", lambda: _lib.call("nsa_slc_attn_bwd_dkdv", *cl, dk.data_ptr(), dk.stride(0), dk.stride(1),
                                     dv.data_ptr(), dv.stride(0), dv.stride(1), H.x_cu_seqlens.data_ptr(),
                                     H.k_cu_seqlens.data_ptr(), H.blk_seq.data_ptr(), bind["csr_off"].data_ptr(),
                                     bind["csr_tok"].data_ptr(), bind["item_off"].data_ptr(), bind["nblk"],
                                     bind["chunk_tokens"], bind["n_items_bound"], H.batch, QH, KH, D, VD,
-                                    H.block_size, sm_scale, st))
+                                    H.block_size, sm_scale, _lib.stream_ptr()))
     cc = common(cmp_k, cmp_v, cmp_lse, cmp_lse.stride(1), cmp_lse.stride(0), delta[0], dcmp_o)
     dq_out = torch.empty_like(q)  # the last dq kernel adds the fp32 partial sum and stores q's dtype
     R("cmp_dq", lambda: _lib.call("nsa_cmp_attn_bwd_dq_final", *cc, dq.data_ptr(), dq.stride(0), dq.stride(1),
                                   dq_out.data_ptr(), dq_out.stride(0), dq_out.stride(1), H.x_cu_seqlens.data_ptr(),
                                   H.y_cu_seqlens.data_ptr(), H.batch, H.x_maxlen, QH, KH, D, VD, H.kernel_size,
-                                  H.stride, sm_scale, st))
+                                  H.stride, sm_scale, _lib.stream_ptr()))
     dck = torch.zeros(cmp_k.shape, device=q.device, dtype=torch.float32)
     dcv = torch.zeros(cmp_v.shape, device=q.device, dtype=torch.float32)
     R("cmp_dkdv", lambda: _lib.call("nsa_cmp_attn_bwd_dkdv", *cc, dck.data_ptr(), dck.stride(0), dck.stride(1),
                                     dcv.data_ptr(), dcv.stride(0), dcv.stride(1), H.x_cu_seqlens.data_ptr(),
                                     H.y_cu_seqlens.data_ptr(), H.batch, H.x_maxlen, H.y_maxlen, QH, KH, D, VD,
-                                    H.kernel_size, H.stride, 2048, sm_scale, st))
+                                    H.kernel_size, H.stride, 2048, sm_scale, _lib.stream_ptr()))
     R("pool_k_bwd", lambda: mean_pooling_bwd(k, dck.to(k.dtype), dk))
 
     def cmp_v_bwd():

@@ -3,6 +3,7 @@ across the three branches and optional recomputation of saved activations
 (mirrors the interface of upstream flash_nsa/modules/megatron_level_nsa.py:46-159, 386-545; the
 context-parallel function of that file is outside this single-GPU build)."""
 import math
+import os
 
 import torch
 
@@ -15,6 +16,22 @@ from ..ops.topk import slc_topk_indices
 from ..ops.act import swiglu_fwd, swiglu_bwd, sigmoid_mul_fwd, sigmoid_mul_bwd
 from ..ops.combine import combine_fwd, combine_bwd
 from ..ops.sliding_window_attention import swa_fwd, swa_bwd
+
+
+# The backward runs on two streams: the memory-bound selected-block dq kernel leaves the matrix cores idle and the
+# dense dk/dv kernels leave the memory side idle, so the dq chain (window -> selected -> compressed) runs next to the
+# dk/dv kernels (measured: about 1 ms of a 75 ms step; the same split of the forward gained nothing).
+# NSA_OVERLAP_STREAMS=0 puts everything back on the caller's stream.
+OVERLAP_STREAMS = os.environ.get("NSA_OVERLAP_STREAMS", "1") != "0"
+_side_streams = {}
+
+
+def _side_stream(device):
+    key = device.index if device.index is not None else torch.cuda.current_device()
+    s = _side_streams.get(key)
+    if s is None:
+        s = _side_streams[key] = torch.cuda.Stream(device=device)
+    return s
 
 
 def weight_grad(inp, grad_out, weight):
@@ -115,16 +132,36 @@ class NSAFunction(torch.autograd.Function):
 
         # the combine backward also yields rowsum(branch * dbranch) of the three branches
         dcmp_o, dslc_o, dswa_o, dw, delta = combine_bwd(cmp_o, slc_o, swa_o, combine_weight, do, return_delta=True)
-        dq = torch.empty(q.shape, device=q.device, dtype=torch.float32)
-        # window branch first: it writes every element of dq / dk / dv, the other branches add to them
-        _, dk, dv = swa_bwd(q, k, v, swa_o, swa_lse, dswa_o, sm_scale=sm_scale, helper=helper, delta=delta[2],
-                            dq=_store_into(dq), dkv_fp32=True)
-        slc_attn_bwd(q, k, v, topk, slc_o, slc_lse, dslc_o, dq, dk, dv, sm_scale=sm_scale, helper=helper,
-                     delta=delta[1])
-        dq, dcmp_k, dcmp_v = cmp_attn_bwd(q, cmp_k, cmp_v, cmp_o, cmp_lse, dcmp_o, dq, sm_scale=sm_scale,
-                                          helper=helper, delta=delta[0], finalize_dq=True)
+        dq32 = torch.empty(q.shape, device=q.device, dtype=torch.float32)
+        kw = dict(sm_scale=sm_scale, helper=helper)
+        if OVERLAP_STREAMS:
+            main, side = torch.cuda.current_stream(), _side_stream(q.device)
+            side.wait_stream(main)
+            with torch.cuda.stream(side):
+                # dq chain: the window branch stores, the selected branch adds, the compressed branch adds and
+                # writes q's dtype
+                swa_bwd(q, k, v, swa_o, swa_lse, dswa_o, delta=delta[2], dq=_store_into(dq32), parts="dq", **kw)
+                slc_attn_bwd(q, k, v, topk, slc_o, slc_lse, dslc_o, dq32, delta=delta[1], parts="dq", **kw)
+                dq, _, _ = cmp_attn_bwd(q, cmp_k, cmp_v, cmp_o, cmp_lse, dcmp_o, dq32, delta=delta[0],
+                                        finalize_dq=True, parts="dq", **kw)
+                dq.record_stream(main)
+            # dk/dv kernels on the caller's stream; the window branch writes every element of dk / dv, the
+            # selected branch adds to them
+            _, dk, dv = swa_bwd(q, k, v, swa_o, swa_lse, dswa_o, delta=delta[2], dkv_fp32=True, parts="dkdv", **kw)
+            slc_attn_bwd(q, k, v, topk, slc_o, slc_lse, dslc_o, None, dk, dv, delta=delta[1], parts="dkdv", **kw)
+            _, dcmp_k, dcmp_v = cmp_attn_bwd(q, cmp_k, cmp_v, cmp_o, cmp_lse, dcmp_o, delta=delta[0], parts="dkdv",
+                                             **kw)
+        else:
+            # window branch first: it writes every element of dq / dk / dv, the other branches add to them
+            _, dk, dv = swa_bwd(q, k, v, swa_o, swa_lse, dswa_o, delta=delta[2], dq=_store_into(dq32), dkv_fp32=True,
+                                **kw)
+            slc_attn_bwd(q, k, v, topk, slc_o, slc_lse, dslc_o, dq32, dk, dv, delta=delta[1], **kw)
+            dq, dcmp_k, dcmp_v = cmp_attn_bwd(q, cmp_k, cmp_v, cmp_o, cmp_lse, dcmp_o, dq32, delta=delta[0],
+                                              finalize_dq=True, **kw)
         _, dwk = compress_kv_bwd(k, cmp_k_weight, win_k, hid_k, dcmp_k, dk, k_method, helper)
         _, dwv = compress_kv_bwd(v, cmp_v_weight, win_v, hid_v, dcmp_v, dv, v_method, helper)
+        if OVERLAP_STREAMS:
+            main.wait_stream(side)
         return dq, dk, dv, dw, dwk, dwv, None
 
 

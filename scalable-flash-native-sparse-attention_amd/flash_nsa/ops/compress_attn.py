@@ -25,10 +25,11 @@ def cmp_attn_fwd(q, k, v, sm_scale=None, helper=NSAHelper):
 
 
 def cmp_attn_bwd(q, k, v, o, lse, do, dq=None, dkdv_repeat=False, sm_scale=None, helper=NSAHelper, delta=None,
-                 q_chunk_tokens=2048, finalize_dq=False):
+                 q_chunk_tokens=2048, finalize_dq=False, parts="both"):
     """Backward of compressed attention.  Returns (dq, dk, dv).
     dq: fresh bf16 tensor, or the caller's fp32 buffer, which is added into; with finalize_dq the fp32 buffer is
     only read and the returned dq is a fresh tensor in q's dtype holding buffer + this branch.
+    parts = "dq" / "dkdv" launches only that kernel (the other results are None).
     dk, dv: fp32 [y_len,KH,*] accumulated with atomics over the q-heads of a group and over query chunks
     (non-deterministic summation order, as upstream's dkdv_repeat=False path); `dkdv_repeat` is accepted for call
     compatibility and ignored.  delta may be passed when already known (delta[T,QH] fp32 = rowsum(o*do))."""
@@ -43,21 +44,26 @@ def cmp_attn_bwd(q, k, v, o, lse, do, dq=None, dkdv_repeat=False, sm_scale=None,
               lse.stride(0), delta.data_ptr(), delta.stride(0), delta.stride(1))
     tail = (helper.x_cu_seqlens.data_ptr(), helper.y_cu_seqlens.data_ptr(), helper.batch, helper.x_maxlen, QH, KH,
             D, VD, helper.kernel_size, helper.stride, sm_scale, _lib.stream_ptr())
-    if finalize_dq:
-        # last branch of a fused backward: dq (fp32 sum of the other branches) + this branch -> fresh tensor in q's dtype
-        assert dq is not None and dq.dtype == torch.float32 and dq.shape == q.shape and dq.stride(-1) == 1
-        dq_buf = torch.empty_like(q)
-        _lib.call("nsa_cmp_attn_bwd_dq_final", *common, dq.data_ptr(), dq.stride(0), dq.stride(1), dq_buf.data_ptr(),
-                  dq_buf.stride(0), dq_buf.stride(1), *tail)
-    else:
-        dq_buf, mode = dq_target(q, dq)
-        _lib.call("nsa_cmp_attn_bwd_dq", *common, dq_buf.data_ptr(), dq_buf.stride(0), dq_buf.stride(1), mode, *tail)
-    dk = torch.zeros(Y, KH, D, device=q.device, dtype=torch.float32)
-    dv = torch.zeros(Y, KH, VD, device=q.device, dtype=torch.float32)
-    _lib.call("nsa_cmp_attn_bwd_dkdv", *common, dk.data_ptr(), dk.stride(0), dk.stride(1), dv.data_ptr(),
-              dv.stride(0), dv.stride(1), helper.x_cu_seqlens.data_ptr(), helper.y_cu_seqlens.data_ptr(),
-              helper.batch, helper.x_maxlen, helper.y_maxlen, QH, KH, D, VD, helper.kernel_size, helper.stride,
-              q_chunk_tokens, sm_scale, _lib.stream_ptr())
+    dq_buf = dk = dv = None
+    if parts in ("both", "dq"):
+        if finalize_dq:
+            # last branch of a fused backward: dq (fp32 sum of the other branches) + this branch -> fresh tensor in
+            # q's dtype
+            assert dq is not None and dq.dtype == torch.float32 and dq.shape == q.shape and dq.stride(-1) == 1
+            dq_buf = torch.empty_like(q)
+            _lib.call("nsa_cmp_attn_bwd_dq_final", *common, dq.data_ptr(), dq.stride(0), dq.stride(1),
+                      dq_buf.data_ptr(), dq_buf.stride(0), dq_buf.stride(1), *tail)
+        else:
+            dq_buf, mode = dq_target(q, dq)
+            _lib.call("nsa_cmp_attn_bwd_dq", *common, dq_buf.data_ptr(), dq_buf.stride(0), dq_buf.stride(1), mode,
+                      *tail)
+    if parts in ("both", "dkdv"):
+        dk = torch.zeros(Y, KH, D, device=q.device, dtype=torch.float32)
+        dv = torch.zeros(Y, KH, VD, device=q.device, dtype=torch.float32)
+        _lib.call("nsa_cmp_attn_bwd_dkdv", *common, dk.data_ptr(), dk.stride(0), dk.stride(1), dv.data_ptr(),
+                  dv.stride(0), dv.stride(1), helper.x_cu_seqlens.data_ptr(), helper.y_cu_seqlens.data_ptr(),
+                  helper.batch, helper.x_maxlen, helper.y_maxlen, QH, KH, D, VD, helper.kernel_size, helper.stride,
+                  q_chunk_tokens, sm_scale, _lib.stream_ptr())
     return dq_buf, dk, dv
 
 

@@ -25,11 +25,12 @@ def slc_attn_fwd(q, k, v, topk, sm_scale=None, helper=NSAHelper):
 
 
 def slc_attn_bwd(q, k, v, topk, o, lse, do, dq=None, dk=None, dv=None, sm_scale=None, helper=NSAHelper, delta=None,
-                 bind=None):
+                 bind=None, parts="both"):
     """Backward of selected attention.  Returns (dq, dk, dv).
     dq: fresh bf16 tensor, or the caller's fp32 buffer (added into).  dk/dv: fp32 [T,KH,*]; the caller's buffers
     are added into with atomics (summation order is not deterministic, as upstream), otherwise zero-filled ones are
-    created.  `bind` is the inverse index from get_bind_from_find (built here when absent)."""
+    created.  `bind` is the inverse index from get_bind_from_find (built here when absent).
+    parts = "dq" / "dkdv" launches only that kernel (the other results are None)."""
     from .topk import get_bind_from_find
     check_thd(do, "do")
     T, QH, D = q.shape
@@ -37,13 +38,17 @@ def slc_attn_bwd(q, k, v, topk, o, lse, do, dq=None, dk=None, dv=None, sm_scale=
     sm_scale = default_scale(q, sm_scale)
     if delta is None:
         delta = delta_of(o, do)
-    dq_buf, mode = dq_target(q, dq)
     common = (q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), k.stride(0), k.stride(1), v.data_ptr(),
               v.stride(0), v.stride(1), do.data_ptr(), do.stride(0), do.stride(1), lse.data_ptr(), lse.stride(0),
               lse.stride(1), delta.data_ptr(), delta.stride(0), delta.stride(1))
-    _lib.call("nsa_slc_attn_bwd_dq", *common, topk.data_ptr(), topk.stride(0), topk.stride(1), dq_buf.data_ptr(),
-              dq_buf.stride(0), dq_buf.stride(1), mode, helper.x_cu_seqlens.data_ptr(), helper.batch,
-              helper.x_maxlen, QH, KH, D, VD, helper.block_size, topk.size(-1), sm_scale, _lib.stream_ptr())
+    dq_buf = None
+    if parts in ("both", "dq"):
+        dq_buf, mode = dq_target(q, dq)
+        _lib.call("nsa_slc_attn_bwd_dq", *common, topk.data_ptr(), topk.stride(0), topk.stride(1), dq_buf.data_ptr(),
+                  dq_buf.stride(0), dq_buf.stride(1), mode, helper.x_cu_seqlens.data_ptr(), helper.batch,
+                  helper.x_maxlen, QH, KH, D, VD, helper.block_size, topk.size(-1), sm_scale, _lib.stream_ptr())
+    if parts == "dq":
+        return dq_buf, None, None
     if dk is None:
         dk = torch.zeros(T, KH, D, device=q.device, dtype=torch.float32)
     if dv is None:

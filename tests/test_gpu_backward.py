@@ -234,3 +234,36 @@ def test_nsa_core_qk192_v128(device):
     assert_close(kd.grad, kr.grad, "dk", row_scale=True)
     assert_close(vd.grad, vr.grad, "dv", row_scale=True)
     assert_close(wd.grad, wr.grad, "dw", atol=5e-2)
+
+
+def test_two_stream_backward_equals_single_stream(device):
+    """The fused backward puts its dq chain on a second stream next to the dk/dv kernels: same results as with
+    everything on one stream (dq bit-equal; dk/dv up to the order of the fp32 atomics)."""
+    from flash_nsa import NSAConfig, NSACore
+    from flash_nsa.modules import megatron_level_nsa as M
+    lens, QH, KH, D = [1500, 700, 333], 32, 2, 128
+    cu = make_cu(lens)
+    T = int(cu[-1])
+    q, k, v, w = make_qkvw(T, QH, KH, D, D, seed=90)
+    do = randn_bf16(T, QH, D, seed=91).to(device)
+    core = NSACore(NSAConfig(head_dim=D, num_heads=QH, num_kv_heads=KH, cmp_v_method="sigmoid-mul"))
+    core = core.to(device=device, dtype=torch.bfloat16)
+
+    def run(overlap):
+        old = M.OVERLAP_STREAMS
+        M.OVERLAP_STREAMS = overlap
+        try:
+            ts = [t.to(device).requires_grad_() for t in (q, k, v, w)]
+            core.zero_grad()
+            out = core(*ts, cu.to(device))
+            out.backward(do)
+            torch.cuda.synchronize()
+            return [out.detach()] + [t.grad for t in ts] + [core.cmp_v_weight.grad.clone()]
+        finally:
+            M.OVERLAP_STREAMS = old
+
+    a, b = run(True), run(False)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1]) and torch.equal(a[4], b[4])
+    assert_close(a[2], b[2], "dk", atol=2e-3, rtol=8e-3, row_scale=True)
+    assert_close(a[3], b[3], "dv", atol=2e-3, rtol=8e-3, row_scale=True)
+    assert_close(a[5], b[5], "d cmp_v_weight", atol=2e-3, rtol=2e-2, row_scale=True)
