@@ -56,7 +56,8 @@ class NSAHelper:
     k_len = 0
     blk_seq = None  # [k_len] sequence id of every selection block (used by the inverse index)
     batch = 0
-    _key = None
+    _registered = None          # the cu_seqlens tensor object of the registered batch and its version counter
+    _registered_version = -1
     _host_cu = None
 
     @classmethod
@@ -71,7 +72,7 @@ class NSAHelper:
         cls.num_init_blocks = num_init_blocks
         cls.num_local_blocks = num_local_blocks
         if changed:
-            cls._key = None
+            cls._registered = None
             cls.x_cu_seqlens = None
 
     @classmethod
@@ -106,19 +107,22 @@ class NSAHelper:
 
     @classmethod
     def _need_init(cls, cu):
+        """False when `cu` holds the registered lengths (upstream flash_nsa/utils.py:216-226 compares values).
+        The same, unmodified tensor object is recognised without a device read; the helper keeps a reference to it,
+        so its address cannot be handed to another tensor in the meantime."""
         if cls.x_cu_seqlens is None:
             return True
-        key = (cu.data_ptr(), cu._version, cu.numel(), cu.device)
-        if key == cls._key:
+        if cu is cls._registered and cu._version == cls._registered_version:
             return False
-        host = cu.tolist()
-        return host != cls._host_cu
+        if cu.numel() != len(cls._host_cu):
+            return True
+        return [int(v) for v in cu.tolist()] != cls._host_cu
 
     @classmethod
     def init_cu_seqlens(cls, x_cu_seqlens: torch.Tensor, x_cu_seqlens_np=None, cp_mode=1):
         """Registers a packed batch: cu_seqlens int tensor [B+1] with cu[0]=0, cu[-1]=T."""
         if not cls._need_init(x_cu_seqlens):
-            cls._key = (x_cu_seqlens.data_ptr(), x_cu_seqlens._version, x_cu_seqlens.numel(), x_cu_seqlens.device)
+            cls._registered, cls._registered_version = x_cu_seqlens, x_cu_seqlens._version
             return
         host = [int(v) for v in x_cu_seqlens.tolist()]
         assert len(host) >= 2 and host[0] == 0, "cu_seqlens must start at 0"
@@ -149,7 +153,7 @@ class NSAHelper:
         cls.blk_seq = torch.repeat_interleave(torch.arange(len(ks), dtype=torch.int32), torch.tensor(ks)).to(
             device=dev, dtype=torch.int32)
         cls._host_cu = host
-        cls._key = (x_cu_seqlens.data_ptr(), x_cu_seqlens._version, x_cu_seqlens.numel(), x_cu_seqlens.device)
+        cls._registered, cls._registered_version = x_cu_seqlens, x_cu_seqlens._version
 
     @classmethod
     def clear_tensor_data(cls, *tensors):

@@ -158,6 +158,11 @@ def test_combine_bwd(device):
     ([1500], 16, 1, 128, ("mean", "mean")),
     ([5, 31, 48, 333, 700, 900], 8, 2, 128, ("mean", "sigmoid-mul")),
     ([300, 800], 4, 2, 64, ("linear", "swiglu")),
+    ([700, 260], 32, 1, 128, ("mean", "mean")),       # 32 q-heads per kv head
+    ([515], 64, 1, 64, ("mean", "mean")),             # 64 q-heads per kv head (two head chunks in the selector)
+    ([400, 330], 16, 2, 128, ("mean", "mean")),       # groups of 8
+    ([400, 330], 6, 3, 64, ("mean", "mean")),         # groups of 2
+    ([400, 330], 12, 4, 64, ("mean", "mean")),        # groups of 3 (not a power of two)
 ])
 def test_nsa_core_fwd_bwd(device, core, lens, QH, KH, D, methods):
     """HFNSACore and NSACore against the composed oracle (upstream only compares them with each other)."""

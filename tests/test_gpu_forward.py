@@ -72,8 +72,11 @@ def test_swa_fwd(device, lens, QH, KH, D):
     setup_helper(cu.to(device))
 
 
-@pytest.mark.parametrize("lens", LENS_CASES)
-@pytest.mark.parametrize("QH,KH,D", HEAD_CASES)
+GROUP_CASES = [(32, 1, 128), (64, 1, 64), (16, 2, 128), (6, 3, 64), (12, 4, 64)]  # groups of 32, 64, 8, 2, 3
+
+
+@pytest.mark.parametrize("lens,QH,KH,D", [(l, *h) for l in LENS_CASES for h in HEAD_CASES] +
+                         [(LENS_CASES[1], *h) for h in GROUP_CASES])
 def test_topk_and_slc_fwd(device, lens, QH, KH, D):
     from flash_nsa.ops.compress_kv import mean_pooling_fwd
     from flash_nsa.ops.compress_attn import cmp_attn_fwd

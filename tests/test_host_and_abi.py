@@ -76,3 +76,24 @@ def test_bench_flop_model_matches_closed_form():
     f = bench.stage_flops([65536], 64, 128, 128)
     assert abs(f["fwd_total"] / 1e12 - 9.87) < 0.01
     assert abs(f["bwd_total"] / 1e12 - 19.19) < 0.01
+
+
+def test_helper_does_not_confuse_a_new_tensor_with_the_registered_one():
+    """A second cu_seqlens tensor with other lengths must be re-registered even when it is as long as the first one
+    (an allocator may even hand it the same address); the same unmodified object is recognised without a read."""
+    import torch
+    from flash_nsa import NSAHelper
+    NSAHelper.set_hyperparameters()
+    a = torch.tensor([0, 700, 960], dtype=torch.int32)
+    NSAHelper.init_cu_seqlens(a)
+    assert (NSAHelper.x_maxlen, NSAHelper.y_len) == (700, 42 + 15)
+    del a
+    b = torch.tensor([0, 400, 730], dtype=torch.int32)
+    NSAHelper.init_cu_seqlens(b)
+    assert (NSAHelper.x_maxlen, NSAHelper.y_len) == (400, 24 + 19)
+    NSAHelper.init_cu_seqlens(b)
+    assert NSAHelper.x_maxlen == 400
+    b[1] = 330                      # in-place edit of the registered tensor bumps its version
+    NSAHelper.init_cu_seqlens(b)
+    assert (NSAHelper.x_maxlen, NSAHelper.y_len) == (400, 19 + 24)
+    assert NSAHelper._host_cu == [0, 330, 730]
