@@ -294,8 +294,9 @@ def main():
         result["roofline"]["memory_side_gbs"] = traffic / (stages[dom] * 1e-3) / 1e9
         result["roofline"]["memory_side_frac_of_hbm_peak"] = result["roofline"]["memory_side_gbs"] / PEAK_HBM_GBS
     if not args.no_decode:
-        from bench_decode import decode_bench
+        from bench_decode import decode_bench, cache_writer_bench
         result["decode"] = decode_bench(dev)
+        result["cache_writer"] = cache_writer_bench(dev)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))

@@ -104,11 +104,87 @@ def decode_bench(dev, reps=200, warmup=20):
     eager_us = s.elapsed_time(e) * 1e3 / 20
     nbytes = algorithmic_bytes(c["lens"])
     gbs = nbytes / (us * 1e-6) / 1e9
-    return {"workload": "paged NSA decode, batch 64, ctx uniform [4096,32768] (seed 3), page 256, 64q/4kv heads, "
-                        "d=128, bf16, hipGraph replay", "us_per_step": us, "eager_us_per_step": eager_us,
-            "graph_equals_eager": same, "algorithmic_bytes": nbytes,
-            "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                         "frac": gbs / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_DEFAULT_CASE}}
+    res = {"workload": "paged NSA decode, batch 64, ctx uniform [4096,32768] (seed 3), page 256, 64q/4kv heads, "
+                       "d=128, bf16, hipGraph replay", "us_per_step": us, "eager_us_per_step": eager_us,
+           "graph_equals_eager": same, "algorithmic_bytes": nbytes,
+           "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                        "frac": gbs / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_DEFAULT_CASE}}
+    # the same step with the cache write of the newest token's K/V inside the launch (KV-cache writer fused)
+    page = c["page"]
+    B, KH, D = len(c["lens"]), c["k"].size(2), c["k"].size(3)
+    new_k = c["k"].view(-1, KH, D)[[int(c["bt"][b, (L - 1) // page]) * page + (L - 1) % page
+                                     for b, L in enumerate(c["lens"])]].clone()
+    new_v = c["v"].view(-1, KH, D)[[int(c["bt"][b, (L - 1) // page]) * page + (L - 1) % page
+                                     for b, L in enumerate(c["lens"])]].clone()
+    raw_slots = torch.tensor([int(c["bt"][b, (L - 1) // page]) * page + (L - 1) % page
+                              for b, L in enumerate(c["lens"])], dtype=torch.int32, device=dev)
+    kw2 = dict(kw, new_k=new_k, new_v=new_v, slot_mapping=raw_slots)
+    out2 = nsa_decode(*args, **kw2)
+    torch.cuda.synchronize()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        nsa_decode(*args, **kw2)
+    torch.cuda.current_stream().wait_stream(side)
+    graph2 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph2):
+        out2 = nsa_decode(*args, **kw2)
+    for _ in range(warmup):
+        graph2.replay()
+    torch.cuda.synchronize()
+    s.record()
+    for _ in range(reps):
+        graph2.replay()
+    e.record()
+    torch.cuda.synchronize()
+    res["us_per_step_with_cache_write"] = s.elapsed_time(e) * 1e3 / reps
+    res["cache_write_equals_plain"] = bool(torch.equal(out2, eager))
+    return res
+
+
+def cache_writer_bench(dev, reps=50):
+    """KV-cache writer on the chunked-prefill configuration (16 requests, cached prefix uniform in [0,16384] from
+    seed 2, 2048 new tokens each, page 256, 4 kv heads, d=128): plain scatter, and the scatter fused with the pooling
+    of the compressed rows the chunk completes, against the three separate launches."""
+    from flash_nsa.inference import (PageTableBuilder, allocate_kv_pools, store_kvcache,
+                                     store_kvcache_and_pool_prefill, mean_pooling_prefill)
+    KH, D, page, chunk = 4, 128, 256, 2048
+    g = torch.Generator().manual_seed(2)
+    cached = torch.randint(0, 16385, (16,), generator=g).tolist()
+    (kc, vc), = allocate_kv_pools(2000, page, KH, D, device=dev)
+    kc.normal_()
+    vc.normal_()
+    b = PageTableBuilder(2000, page)
+    ids = list(range(16))
+    b.prefill(ids, [max(c, 1) for c in cached], device=dev)
+    st = b.prefill(ids, [chunk] * 16, device=dev)
+    t = 16 * chunk
+    gd = torch.Generator(device=dev).manual_seed(2)
+    key = torch.randn(t, KH, D, device=dev, generator=gd, dtype=torch.float32).to(torch.bfloat16)
+    val = torch.randn(t, KH, D, device=dev, generator=gd, dtype=torch.float32).to(torch.bfloat16)
+
+    def timeit(fn):
+        fn()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(reps):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        return s.elapsed_time(e) * 1e3 / reps
+
+    pool_args = (st["y_cu_seqlens"], st["y_maxlen"], st["block_tables"], st["cmp_slot_mapping"])
+    store_us = timeit(lambda: store_kvcache(key, val, kc, vc, st["slot_mapping"]))
+    pool_us = timeit(lambda: (mean_pooling_prefill(kc, *pool_args), mean_pooling_prefill(vc, *pool_args)))
+    fused_us = timeit(lambda: store_kvcache_and_pool_prefill(
+        key, val, kc, vc, st["x_cu_seqlens"], st["x_maxlen"], st["context_lens"], st["slot_mapping"],
+        st["y_cu_seqlens"], st["y_maxlen"], st["cmp_slot_mapping"], st["block_tables"]))
+    nbytes = 2 * 2 * t * KH * D * 2  # K and V rows, read once and written once
+    return {"workload": "store_kvcache of 16 x 2048 new tokens, 4 kv heads, d=128, bf16, page 256",
+            "store_us": store_us, "algorithmic_bytes": nbytes,
+            "roofline": {"bound": "hbm", "achieved": nbytes / (store_us * 1e-6) / 1e9, "peak": PEAK_HBM_GBS,
+                         "unit": "GB/s", "frac": nbytes / (store_us * 1e-6) / 1e9 / PEAK_HBM_GBS, "traffic": None},
+            "store_then_pool_us": store_us + pool_us, "fused_store_pool_us": fused_us}
 
 
 if __name__ == "__main__":
@@ -117,4 +193,5 @@ if __name__ == "__main__":
     import sys
     root = os.path.dirname(os.path.abspath(__file__))
     sys.path.insert(0, os.path.join(root, "scalable-flash-native-sparse-attention_amd"))
-    print(json.dumps(decode_bench(torch.device("cuda:0"))))
+    print(json.dumps({"decode": decode_bench(torch.device("cuda:0")),
+                      "cache_writer": cache_writer_bench(torch.device("cuda:0"))}))

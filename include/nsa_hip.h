@@ -196,6 +196,24 @@ int nsa_paged_pool_decode(void* k_cache, int64_t k_sr, int64_t k_sh, int Dk, voi
                           int table_stride, const int32_t* cmp_slot_mapping, int B, int page_size, int H,
                           int kernel_size, int stride, void* stream);
 
+/* ---- KV-cache writer (the caller side of the paged entry points) ----
+ * nano-vllm/nanovllm/layers/attention.py:123-153 store_kvcache: row n of key / value (k_row_elems = KH*D contiguous
+ * elements, row stride k_st) is copied to flat pool row slot_mapping[n] of k_cache / v_cache (row stride kc_sr);
+ * negative slots are skipped. */
+int nsa_store_kvcache(const void* key, int64_t k_st, const void* value, int64_t v_st, void* k_cache, int64_t kc_sr,
+                      void* v_cache, int64_t vc_sr, const int32_t* slot_mapping, int N, int k_row_elems,
+                      int v_row_elems, void* stream);
+/* One launch for a prefill chunk: store_kvcache of the chunk's new tokens (key / value [t,KH,D] packed by x_cu,
+ * slot_mapping [t]) + mean pooling of the compressed rows listed in cmp_slot_mapping (as nsa_paged_pool_prefill,
+ * flash_nsa/inference/compress_kv.py:191-220, for K and V).  Source rows of a pooled window are taken from the
+ * chunk when they are new (position >= context_lens[b] - new tokens of b) and from the pool otherwise. */
+int nsa_paged_store_pool_prefill(const void* key, int64_t k_st, int64_t k_sh, int Dk, const void* value, int64_t v_st,
+                                 int64_t v_sh, int Dv, void* k_cache, int64_t kc_sr, int64_t kc_sh, void* v_cache,
+                                 int64_t vc_sr, int64_t vc_sh, const int32_t* x_cu, const int32_t* context_lens,
+                                 const int32_t* slot_mapping, const int32_t* y_cu, const int32_t* cmp_slot_mapping,
+                                 const int32_t* block_tables, int table_stride, int B, int x_maxlen, int y_maxlen,
+                                 int page_size, int H, int kernel_size, int stride, void* stream);
+
 /* ---- fused decode step (one query token per request; q [B,QH,D], at most 16 q-heads per kv head) ----
  * Replaces flash_nsa/inference/compress_attn.py:540-667 (cmp_attn_decode) + inference/topk.py:495-623 (topk_decode):
  * compressed attention (cmp_o [B,QH,VD], optional lse addressed b*lse_st + head*lse_sh) and the top-n selection
@@ -238,6 +256,9 @@ int nsa_decode_slc_swa_combine(const void* q, int64_t q_st, int64_t q_sh, const 
  * are optional outputs (NULL to skip).  cmp_slot_mapping [B] (optional): when given, the kernel also pools the
  * compressed K and V row that the newest token completes (flat pool row, -1: none), i.e. it includes
  * nsa_paged_pool_decode (flash_nsa/inference/compress_kv.py:253-287) and the step is a single launch.
+ * new_k / new_v [B,KH,D] / [B,KH,VD] + slot_mapping [B] (optional, all three or none): the newest token's K and V
+ * rows are first written to flat pool row slot_mapping[b] (-1: skip), i.e. the kernel also includes
+ * store_kvcache (nano-vllm/nanovllm/layers/attention.py:123-153).
  * Needs fixed_y_maxlen / fixed_num_slc_blocks / table_stride small enough for
  * 160 KB of LDS (nsa_decode_fused_fits returns 1; e.g. contexts up to 32K tokens at kernel 32 / stride 16);
  * otherwise use nsa_decode_cmp_topk + nsa_decode_slc_swa_combine. */
@@ -249,7 +270,8 @@ int nsa_decode_fused(const void* q, int64_t q_st, int64_t q_sh, const void* k_ca
                      int64_t co_sh, float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk, int64_t tk_sh,
                      int64_t tk_st, const int32_t* context_lens, const int32_t* block_tables, int table_stride,
                      const int32_t* cmp_block_tables, int cmp_table_stride,
-                     const int32_t* cmp_slot_mapping, int page_size, int B, int QH, int KH,
+                     const int32_t* cmp_slot_mapping, const void* new_k, int64_t nk_st, int64_t nk_sh,
+                     const void* new_v, int64_t nv_st, int64_t nv_sh, const int32_t* slot_mapping, int page_size, int B, int QH, int KH,
                      int D, int VD, int fixed_y_maxlen, int fixed_num_slc_blocks, int kernel_size, int stride,
                      int block_size, int top_n, int num_init, int num_local, int ignore_index, int window,
                      float sm_scale, void* stream);

@@ -388,6 +388,17 @@ def gather_rows(cache, table_row, n):
     return flat[pages * page + r % page]
 
 
+def store_kvcache(key, value, k_cache, v_cache, slot_mapping):
+    """Cache writer (nano-vllm/nanovllm/layers/attention.py:123-153 upstream): row n of key / value is copied to
+    flat pool row slot_mapping[n]; negative slots are skipped.  In place on the [pages, page, KH, *] pools."""
+    kf = k_cache.view(-1, *k_cache.shape[2:])
+    vf = v_cache.view(-1, *v_cache.shape[2:])
+    for n, slot in enumerate(slot_mapping.tolist()):
+        if slot >= 0:
+            kf[slot] = key[n].to(kf.dtype)
+            vf[slot] = value[n].to(vf.dtype)
+
+
 def paged_pool_prefill(cache, y_cu_seqlens, context_lens, block_tables, cmp_slot_mapping, kernel_size=32,
                        stride=16):
     """In-place: for every compressed row with slot != -1, write mean of its window (read through the raw block

@@ -586,7 +586,8 @@ int nsa_decode_fused(const void* q, int64_t q_st, int64_t q_sh, const void* k_ca
                      int64_t co_sh, float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk, int64_t tk_sh,
                      int64_t tk_st, const int32_t* context_lens, const int32_t* block_tables, int table_stride,
                      const int32_t* cmp_block_tables, int cmp_table_stride,
-                     const int32_t* cmp_slot_mapping, int page_size, int B, int QH, int KH,
+                     const int32_t* cmp_slot_mapping, const void* new_k, int64_t nk_st, int64_t nk_sh,
+                     const void* new_v, int64_t nv_st, int64_t nv_sh, const int32_t* slot_mapping, int page_size, int B, int QH, int KH,
                      int D, int VD, int fixed_y_maxlen, int fixed_num_slc_blocks, int kernel_size, int stride,
                      int block_size, int top_n, int num_init, int num_local, int ignore_index, int window,
                      float sm_scale, void* stream) {
@@ -618,6 +619,11 @@ int nsa_decode_fused(const void* q, int64_t q_st, int64_t q_sh, const void* k_ca
   p.table = block_tables; p.table_stride = table_stride;
   p.cmp_table = cmp_block_tables; p.cmp_table_stride = cmp_table_stride; p.page_size = page_size;
   p.cmp_slots = cmp_slot_mapping;
+  NSA_REQUIRE((new_k == nullptr) == (new_v == nullptr) && (new_k == nullptr) == (slot_mapping == nullptr),
+              NSA_ERR_BAD_ARG, "decode_fused: new_k, new_v and slot_mapping must be given together");
+  p.new_k = (const bf16_t*)new_k; p.nk_st = nk_st; p.nk_sh = nk_sh;
+  p.new_v = (const bf16_t*)new_v; p.nv_st = nv_st; p.nv_sh = nv_sh;
+  p.raw_slots = slot_mapping;
   p.G = QH / KH; p.KH = KH;
   p.scale_log2 = sm_scale * NSA_LOG2E;
   p.kernel_size = kernel_size; p.stride = stride; p.block_size = block_size; p.window = window;

@@ -119,6 +119,9 @@ struct NsaDecodeParams {
   const int32_t* table; int table_stride;       // raw block tables
   const int32_t* cmp_table; int cmp_table_stride;
   const int32_t* cmp_slots;                     // one-launch kernel: flat row of the compressed row completed now (-1: none), or null
+  const bf16_t* new_k; int64_t nk_st, nk_sh;    // one-launch kernel: K / V of the newest token [B, KH, D] to be written
+  const bf16_t* new_v; int64_t nv_st, nv_sh;    // to flat pool row raw_slots[b] first (null: the caller stored them)
+  const int32_t* raw_slots;
   int page_size;
   int G, KH;
   float scale_log2;

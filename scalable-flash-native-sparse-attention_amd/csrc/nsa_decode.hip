@@ -730,32 +730,58 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_fused_kernel(NsaDecodeP
       if (i < nc) ctab_s[i] = ctab[i];
       else tab_s[i - nc] = tab[i - nc];
     }
-    // the compressed row that the newest token completes: mean of the last kernel_size raw rows of this kv head,
-    // summed in row order in fp32 like nsa_paged_pool_decode (flash_nsa/inference/compress_kv.py:253-287 upstream);
-    // wave 0 pools K, wave 1 pools V.  The row is written to the pool and read back below as the last key.
-    const int slot = p.cmp_slots != nullptr ? p.cmp_slots[b] : -1;
-    if (slot >= 0 && L >= p.kernel_size && wave < 2) {
-      bf16_t* cache = const_cast<bf16_t*>(wave == 0 ? p.k : p.v);
-      const int64_t c_sr = wave == 0 ? p.k_sr : p.v_sr, c_sh = wave == 0 ? p.k_sh : p.v_sh;
-      const int C = (wave == 0 ? D : VD) / 8;
-      if (lane < C) {
+  }
+  // Cache maintenance of this (request, kv head), wave 0 for K and wave 1 for V, one 16-byte piece per lane:
+  //  * the newest token's row goes to its pool row (upstream store_kvcache,
+  //    nano-vllm/nanovllm/layers/attention.py:123-153), when the caller passes it;
+  //  * the compressed row that the newest token completes = mean of the last kernel_size raw rows, summed in
+  //    row order in fp32 like nsa_paged_pool_decode (flash_nsa/inference/compress_kv.py:253-287 upstream).
+  // Both are written to the pool and read back by the attention phases of this workgroup after a fence and a
+  // barrier.  The compressed phase only needs the pooled row, so when nothing is pooled at this step the store
+  // runs after the first barrier and its fence is covered by the barriers that separate the phases.
+  const int raw_slot = (p.raw_slots != nullptr && L > 0) ? p.raw_slots[b] : -1;
+  const int cmp_slot = p.cmp_slots != nullptr ? p.cmp_slots[b] : -1;
+  const bool pool_now = cmp_slot >= 0 && L >= p.kernel_size;
+  auto maintain = [&]() {
+    bf16_t* cache = const_cast<bf16_t*>(wave == 0 ? p.k : p.v);
+    const int64_t c_sr = wave == 0 ? p.k_sr : p.v_sr, c_sh = wave == 0 ? p.k_sh : p.v_sh;
+    const int C = (wave == 0 ? D : VD) / 8;
+    if (lane < C) {
+      bf16x8 newest = zero_bf16x8();
+      if (raw_slot >= 0) {
+        const bf16_t* src = wave == 0 ? p.new_k + (int64_t)b * p.nk_st + (int64_t)kh * p.nk_sh
+                                      : p.new_v + (int64_t)b * p.nv_st + (int64_t)kh * p.nv_sh;
+        newest = ld_global_b128(src + lane * 8);
+        *reinterpret_cast<bf16x8*>(cache + (int64_t)raw_slot * c_sr + (int64_t)kh * c_sh + lane * 8) = newest;
+      }
+      if (pool_now) {
+        const int32_t* tab = p.table + (int64_t)b * p.table_stride;
         const int st = ((L - p.kernel_size) / p.stride) * p.stride;
         float a[8] = {0, 0, 0, 0, 0, 0, 0, 0};
         for (int r = 0; r < p.kernel_size; r++) {
           const int n = st + r;
-          const int64_t row = (int64_t)tab[n / page] * page + (n % page);
-          bf16x8 x = ld_global_b128(cache + row * c_sr + (int64_t)kh * c_sh + lane * 8);
+          bf16x8 x;
+          if (raw_slot >= 0 && n == L - 1) {
+            x = newest;  // the row just stored: taken from the register, not read back
+          } else {
+            const int64_t row = (int64_t)tab[n / page] * page + (n % page);
+            x = ld_global_b128(cache + row * c_sr + (int64_t)kh * c_sh + lane * 8);
+          }
 #pragma unroll
           for (int e = 0; e < 8; e++) a[e] += (float)x[e];
         }
         const float inv = 1.f / (float)p.kernel_size;
-        *reinterpret_cast<bf16x8*>(cache + (int64_t)slot * c_sr + (int64_t)kh * c_sh + lane * 8) =
+        *reinterpret_cast<bf16x8*>(cache + (int64_t)cmp_slot * c_sr + (int64_t)kh * c_sh + lane * 8) =
             pack8(a[0] * inv, a[1] * inv, a[2] * inv, a[3] * inv, a[4] * inv, a[5] * inv, a[6] * inv, a[7] * inv);
       }
-      __threadfence();
     }
-  }
+    // the rows are read back only by waves of this workgroup (same CU, same vector L1): a workgroup-scope release
+    // is enough, and much cheaper than a device-scope fence, which writes back the L2 slice of the XCD
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  };
+  if (pool_now && wave < 2) maintain();
   __syncthreads();
+  if (!pool_now && raw_slot >= 0 && wave < 2) maintain();
   const bf16_t* kbase = p.k + (int64_t)kh * p.k_sh;
   const bf16_t* vbase = p.v + (int64_t)kh * p.v_sh;
   const int l16 = lane & 15;

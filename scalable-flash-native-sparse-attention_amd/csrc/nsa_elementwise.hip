@@ -327,6 +327,75 @@ __global__ void paged_pool_decode_kernel(bf16_t* kc, int64_t k_sr, int64_t k_sh,
       pack8(a[0] * inv, a[1] * inv, a[2] * inv, a[3] * inv, a[4] * inv, a[5] * inv, a[6] * inv, a[7] * inv);
 }
 
+// ------------------------------------------------------------------------------------------ KV-cache writer
+// store_kvcache (upstream nano-vllm/nanovllm/layers/attention.py:123-153): row n of key / value goes to flat pool
+// row slot[n] (skipped when negative).  grid (cdiv(N*max(Wk,Wv)/8, 256), 2): y = 0 copies K, y = 1 copies V.
+__global__ void store_kvcache_kernel(const bf16_t* key, int64_t k_st, const bf16_t* value, int64_t v_st,
+                                     bf16_t* kc, int64_t kc_sr, bf16_t* vc, int64_t vc_sr, const int32_t* slots,
+                                     int N, int Wk, int Wv) {
+  const bool is_v = blockIdx.y == 1;
+  const int C = (is_v ? Wv : Wk) / 8;
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (int64_t)N * C) return;
+  const int n = idx / C, c = idx - (int64_t)n * C;
+  const int slot = slots[n];
+  if (slot < 0) return;
+  if (is_v) *reinterpret_cast<bf16x8*>(vc + (int64_t)slot * vc_sr + c * 8) = ld_global_b128(value + n * v_st + c * 8);
+  else *reinterpret_cast<bf16x8*>(kc + (int64_t)slot * kc_sr + c * 8) = ld_global_b128(key + n * k_st + c * 8);
+}
+
+// Prefill chunk in one launch: scatter the chunk's new K/V rows into the pool AND pool the compressed rows that the
+// chunk completes.  A pooled row reads a source row from the chunk itself when that row is new (position >=
+// context - new tokens) and from the pool otherwise, so the two halves of the kernel do not depend on each other.
+// grid (cdiv(max(new_max, y_max)*H*C, 256), B, 2): z = 0 K, z = 1 V.
+__global__ void paged_store_pool_prefill_kernel(const bf16_t* key, int64_t k_st, int64_t k_sh, int Dk,
+                                                const bf16_t* value, int64_t v_st, int64_t v_sh, int Dv,
+                                                bf16_t* kc, int64_t kc_sr, int64_t kc_sh, bf16_t* vc, int64_t vc_sr,
+                                                int64_t vc_sh, const int32_t* x_cu, const int32_t* ctx_lens,
+                                                const int32_t* slots, const int32_t* y_cu, const int32_t* cmp_slots,
+                                                const int32_t* table, int table_stride, int page, int H, int K,
+                                                int S) {
+  const bool is_v = blockIdx.z == 1;
+  const bf16_t* src = is_v ? value : key;
+  const int64_t s_st = is_v ? v_st : k_st, s_sh = is_v ? v_sh : k_sh;
+  bf16_t* cache = is_v ? vc : kc;
+  const int64_t c_sr = is_v ? vc_sr : kc_sr, c_sh = is_v ? vc_sh : kc_sh;
+  const int D = is_v ? Dv : Dk;
+  const int C = D / 8;
+  const int b = blockIdx.y;
+  const int x0 = x_cu[b], xl = x_cu[b + 1] - x0;
+  const int y0 = y_cu[b], yl = y_cu[b + 1] - y0;
+  const int cached = ctx_lens[b] - xl;  // tokens of the request that are in the pool already
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int c = idx % C;
+  const int h = (idx / C) % H;
+  const int i = idx / ((int64_t)C * H);
+  if (i < xl) {  // scatter new token i of the request
+    const int slot = slots[x0 + i];
+    if (slot >= 0)
+      *reinterpret_cast<bf16x8*>(cache + (int64_t)slot * c_sr + (int64_t)h * c_sh + c * 8) =
+          ld_global_b128(src + (int64_t)(x0 + i) * s_st + (int64_t)h * s_sh + c * 8);
+  }
+  if (i < yl) {  // compressed row i of the request
+    const int slot = cmp_slots[y0 + i];
+    if (slot < 0) return;
+    const int32_t* tb = table + (int64_t)b * table_stride;
+    float a[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int r = 0; r < K; r++) {
+      const int n = S * i + r;
+      if (n >= cached) {
+        acc8(a, ld_global_b128(src + (int64_t)(x0 + n - cached) * s_st + (int64_t)h * s_sh + c * 8));
+      } else {
+        const int64_t row = (int64_t)tb[n / page] * page + (n % page);
+        acc8(a, ld_global_b128(cache + row * c_sr + (int64_t)h * c_sh + c * 8));
+      }
+    }
+    const float inv = 1.f / (float)K;
+    *reinterpret_cast<bf16x8*>(cache + (int64_t)slot * c_sr + (int64_t)h * c_sh + c * 8) =
+        pack8(a[0] * inv, a[1] * inv, a[2] * inv, a[3] * inv, a[4] * inv, a[5] * inv, a[6] * inv, a[7] * inv);
+  }
+}
+
 inline unsigned blocks_for(int64_t n, int bs) { return (unsigned)((n + bs - 1) / bs); }
 
 }  // namespace
@@ -472,6 +541,43 @@ int nsa_paged_pool_decode(void* k_cache, int64_t k_sr, int64_t k_sh, int Dk, voi
                                                                  table_stride, cmp_slot_mapping, page_size, H,
                                                                  kernel_size, stride);
   return nsa_check_launch("paged_pool_decode");
+}
+
+int nsa_store_kvcache(const void* key, int64_t k_st, const void* value, int64_t v_st, void* k_cache, int64_t kc_sr,
+                      void* v_cache, int64_t vc_sr, const int32_t* slot_mapping, int N, int k_row_elems,
+                      int v_row_elems, void* stream) {
+  NSA_REQUIRE(k_row_elems > 0 && v_row_elems > 0 && k_row_elems % 8 == 0 && v_row_elems % 8 == 0, NSA_ERR_BAD_ARG,
+              "store_kvcache: row widths %d / %d must be positive multiples of 8", k_row_elems, v_row_elems);
+  NSA_REQUIRE(k_st >= k_row_elems && v_st >= v_row_elems && kc_sr >= k_row_elems && vc_sr >= v_row_elems,
+              NSA_ERR_BAD_ARG, "store_kvcache: a row stride is smaller than the row");
+  if (N <= 0) return NSA_OK;
+  const int mx = k_row_elems > v_row_elems ? k_row_elems : v_row_elems;
+  dim3 grid(blocks_for((int64_t)N * (mx / 8), 256), 2);
+  store_kvcache_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const bf16_t*)key, k_st, (const bf16_t*)value, v_st,
+                                                              (bf16_t*)k_cache, kc_sr, (bf16_t*)v_cache, vc_sr,
+                                                              slot_mapping, N, k_row_elems, v_row_elems);
+  return nsa_check_launch("store_kvcache");
+}
+
+int nsa_paged_store_pool_prefill(const void* key, int64_t k_st, int64_t k_sh, int Dk, const void* value, int64_t v_st,
+                                 int64_t v_sh, int Dv, void* k_cache, int64_t kc_sr, int64_t kc_sh, void* v_cache,
+                                 int64_t vc_sr, int64_t vc_sh, const int32_t* x_cu, const int32_t* context_lens,
+                                 const int32_t* slot_mapping, const int32_t* y_cu, const int32_t* cmp_slot_mapping,
+                                 const int32_t* block_tables, int table_stride, int B, int x_maxlen, int y_maxlen,
+                                 int page_size, int H, int kernel_size, int stride, void* stream) {
+  NSA_REQUIRE(Dk % 8 == 0 && Dv % 8 == 0 && Dk > 0 && Dv > 0, NSA_ERR_BAD_ARG,
+              "paged_store_pool_prefill: head dims %d / %d must be positive multiples of 8", Dk, Dv);
+  NSA_REQUIRE(page_size > 0 && H > 0 && kernel_size > 0 && stride > 0, NSA_ERR_BAD_ARG,
+              "paged_store_pool_prefill: page_size, H, kernel_size and stride must be positive");
+  if (B <= 0 || (x_maxlen <= 0 && y_maxlen <= 0)) return NSA_OK;
+  const int rows = x_maxlen > y_maxlen ? x_maxlen : y_maxlen;
+  const int mx = Dk > Dv ? Dk : Dv;
+  dim3 grid(blocks_for((int64_t)rows * H * (mx / 8), 256), B, 2);
+  paged_store_pool_prefill_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(
+      (const bf16_t*)key, k_st, k_sh, Dk, (const bf16_t*)value, v_st, v_sh, Dv, (bf16_t*)k_cache, kc_sr, kc_sh,
+      (bf16_t*)v_cache, vc_sr, vc_sh, x_cu, context_lens, slot_mapping, y_cu, cmp_slot_mapping, block_tables,
+      table_stride, page_size, H, kernel_size, stride);
+  return nsa_check_launch("paged_store_pool_prefill");
 }
 
 }  // extern "C"

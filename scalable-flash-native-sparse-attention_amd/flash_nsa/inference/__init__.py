@@ -6,25 +6,34 @@ never synchronise with the host, so the decode step can be captured in a HIP gra
 from .stages import (mean_pooling_prefill, kv_mean_pooling_decode, cmp_attn_prefill, cmp_attn_decode, topk_prefill,
                      topk_decode, slc_attn_prefill, fused_slc_swa_attn_decode, swa_prefill, combine_prefill,
                      combine_decode, mean_pooling_decode, slc_attn_decode, fused_decode_supported, decode_cmp_topk,
-                     decode_slc_swa_combine, decode_cmp_split, decode_one_launch, decode_one_launch_fits)
+                     decode_slc_swa_combine, decode_cmp_split, decode_one_launch, decode_one_launch_fits,
+                     store_kvcache, store_kvcache_and_pool_prefill)
+from .paging import PageTableBuilder, allocate_kv_pools
 
 
 def nsa_prefill(q, k, v, w, x_cu_seqlens, y_cu_seqlens, x_maxlen, y_maxlen, context_lens, block_tables,
                 cmp_slot_mapping, cmp_block_tables, fixed_y_maxlen=8192, fixed_num_slc_blocks=2048, kernel_size=32,
                 stride=16, block_size=64, top_n=16, num_init_blocks=1, num_local_blocks=2, window_size=512,
-                sm_scale=None):
+                sm_scale=None, new_k=None, new_v=None, slot_mapping=None):
     """Chunked / prefix-cached prefill.
     q [t,QH,D] new tokens only; k, v [pages, page_size, KH, D|VD] pools; w [t,QH,3];
     x_cu_seqlens [B+1] offsets of the new tokens; y_cu_seqlens [B+1] offsets of ALL compressed rows per request;
     context_lens [B] total lengths; block_tables [B,N1]; cmp_slot_mapping [y_cu[-1]] flat destination row of each
-    compressed row or -1 if it was pooled by an earlier chunk; cmp_block_tables [B,N2].  Returns o [t,QH,VD]."""
+    compressed row or -1 if it was pooled by an earlier chunk; cmp_block_tables [B,N2].  Returns o [t,QH,VD].
+    As upstream, the new tokens' K/V are expected in the pools already; alternatively pass them as new_k / new_v
+    [t,KH,*] with their flat pool rows slot_mapping [t] and the cache write is fused with the pooling (one launch)."""
     assert k.size(1) % 64 == 0, "page size must be a multiple of 64"
     if sm_scale is None:
         sm_scale = q.size(-1) ** -0.5
-    mean_pooling_prefill(k, y_cu_seqlens, y_maxlen, block_table=block_tables, slot_mapping=cmp_slot_mapping,
-                         kernel_size=kernel_size, stride=stride)
-    mean_pooling_prefill(v, y_cu_seqlens, y_maxlen, block_table=block_tables, slot_mapping=cmp_slot_mapping,
-                         kernel_size=kernel_size, stride=stride)
+    if new_k is not None:
+        store_kvcache_and_pool_prefill(new_k, new_v, k, v, x_cu_seqlens, x_maxlen, context_lens, slot_mapping,
+                                       y_cu_seqlens, y_maxlen, cmp_slot_mapping, block_tables,
+                                       kernel_size=kernel_size, stride=stride)
+    else:
+        mean_pooling_prefill(k, y_cu_seqlens, y_maxlen, block_table=block_tables, slot_mapping=cmp_slot_mapping,
+                             kernel_size=kernel_size, stride=stride)
+        mean_pooling_prefill(v, y_cu_seqlens, y_maxlen, block_table=block_tables, slot_mapping=cmp_slot_mapping,
+                             kernel_size=kernel_size, stride=stride)
     cmp_o, lse = cmp_attn_prefill(q, k, v, x_cu_seqlens, x_maxlen, block_tables=cmp_block_tables,
                                   context_lens=context_lens, kernel_size=kernel_size, stride=stride,
                                   sm_scale=sm_scale)
@@ -42,9 +51,13 @@ def nsa_prefill(q, k, v, w, x_cu_seqlens, y_cu_seqlens, x_maxlen, y_maxlen, cont
 
 def nsa_decode(q, k, v, w, context_lens, block_tables, cmp_slot_mapping, cmp_block_tables, cmp_num_splits=0,
                slc_num_splits=0, fixed_y_maxlen=8192, fixed_num_slc_blocks=2048, kernel_size=32, stride=16,
-               block_size=64, top_n=16, num_init_blocks=1, num_local_blocks=2, window_size=512, sm_scale=None):
+               block_size=64, top_n=16, num_init_blocks=1, num_local_blocks=2, window_size=512, sm_scale=None,
+               new_k=None, new_v=None, slot_mapping=None):
     """One query token per request.  q [B,QH,D]; w [B,QH,3]; cmp_slot_mapping [B] (-1: no compressed row completes
-    at this step).  Rows with context_lens == 0 (graph padding) produce zeros.  Returns o [B,QH,VD]."""
+    at this step).  Rows with context_lens == 0 (graph padding) produce zeros.  Returns o [B,QH,VD].
+    As upstream, the newest token's K/V are expected in the pools already; alternatively pass them as new_k / new_v
+    [B,KH,*] with their flat pool rows slot_mapping [B] (-1: padding) and the cache write happens here (inside the
+    single decode launch when that path is taken)."""
     assert k.size(1) % 64 == 0, "page size must be a multiple of 64"
     if sm_scale is None:
         sm_scale = q.size(-1) ** -0.5
@@ -56,7 +69,10 @@ def nsa_decode(q, k, v, w, context_lens, block_tables, cmp_slot_mapping, cmp_blo
                                  fixed_y_maxlen=fixed_y_maxlen, fixed_num_slc_blocks=fixed_num_slc_blocks,
                                  kernel_size=kernel_size, stride=stride, block_size=block_size, top_n=top_n,
                                  num_inital=num_init_blocks, num_local=num_local_blocks, window_size=window_size,
-                                 sm_scale=sm_scale, cmp_slot_mapping=cmp_slot_mapping)
+                                 sm_scale=sm_scale, cmp_slot_mapping=cmp_slot_mapping, new_k=new_k, new_v=new_v,
+                                 slot_mapping=slot_mapping)
+    if new_k is not None:
+        store_kvcache(new_k, new_v, k, v, slot_mapping)
     kv_mean_pooling_decode(k, v, block_table=block_tables, slot_mapping=cmp_slot_mapping, context_lens=context_lens,
                            kernel_size=kernel_size, stride=stride)
     if fused_decode_supported(q, k, v):

@@ -32,6 +32,44 @@ def _i32(t):
     return t
 
 
+# ------------------------------------------------------------------------------------------------ cache writer
+def store_kvcache(key, value, k_cache, v_cache, slot_mapping):
+    """Scatter of new K/V rows into the paged pools (upstream nano-vllm/nanovllm/layers/attention.py:123-153):
+    key [N,KH,D], value [N,KH,VD] -> flat pool rows slot_mapping[n] of k_cache / v_cache [pages,page,KH,*]
+    (-1: skip the token)."""
+    check_bf16(key)
+    N, KH, D = key.shape
+    VD = value.size(-1)
+    assert value.shape[:2] == (N, KH) and key.stride(-1) == 1 and value.stride(-1) == 1
+    assert key.stride(1) == D and value.stride(1) == VD, "the heads of a token must be contiguous"
+    assert k_cache.dim() == 4 and k_cache.is_contiguous() and v_cache.is_contiguous()
+    assert k_cache.shape[2:] == (KH, D) and v_cache.shape[2:] == (KH, VD)
+    assert slot_mapping.numel() == N
+    _lib.call("nsa_store_kvcache", key.data_ptr(), key.stride(0), value.data_ptr(), value.stride(0),
+              k_cache.data_ptr(), KH * D, v_cache.data_ptr(), KH * VD, _i32(slot_mapping).data_ptr(), N, KH * D,
+              KH * VD, _lib.stream_ptr())
+
+
+def store_kvcache_and_pool_prefill(key, value, k_cache, v_cache, x_cu_seqlens, x_maxlen, context_lens, slot_mapping,
+                                   y_cu_seqlens, y_maxlen, cmp_slot_mapping, block_tables, kernel_size=32, stride=16):
+    """One launch for a prefill chunk: store_kvcache of the new tokens (key/value [t,KH,*] packed by x_cu_seqlens)
+    and mean pooling of the compressed rows named by cmp_slot_mapping (what two mean_pooling_prefill calls do after a
+    separate store)."""
+    check_bf16(key)
+    t, KH, D = key.shape
+    VD = value.size(-1)
+    page = k_cache.size(1)
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and key.stride(-1) == 1 and value.stride(-1) == 1
+    assert k_cache.shape[2:] == (KH, D) and v_cache.shape[2:] == (KH, VD) and slot_mapping.numel() == t
+    B = x_cu_seqlens.numel() - 1
+    _lib.call("nsa_paged_store_pool_prefill", key.data_ptr(), key.stride(0), key.stride(1), D, value.data_ptr(),
+              value.stride(0), value.stride(1), VD, k_cache.data_ptr(), k_cache.stride(1), k_cache.stride(2),
+              v_cache.data_ptr(), v_cache.stride(1), v_cache.stride(2), _i32(x_cu_seqlens).data_ptr(),
+              _i32(context_lens).data_ptr(), _i32(slot_mapping).data_ptr(), _i32(y_cu_seqlens).data_ptr(),
+              _i32(cmp_slot_mapping).data_ptr(), _i32(block_tables).data_ptr(), block_tables.stride(0), B,
+              int(x_maxlen), int(y_maxlen), page, KH, kernel_size, stride, _lib.stream_ptr())
+
+
 # ------------------------------------------------------------------------------------------------ pooling
 def mean_pooling_prefill(x, y_cu_seqlens, y_maxlen, block_table, slot_mapping, kernel_size=32, stride=16):
     """In place: every compressed row whose slot != -1 is pooled from the raw rows (read through block_table)
@@ -194,12 +232,14 @@ def decode_one_launch_fits(q, k, v, block_tables, fixed_y_maxlen, fixed_num_slc_
 
 def decode_one_launch(q, k, v, w, block_tables, cmp_block_tables, context_lens, fixed_y_maxlen=8192,
                       fixed_num_slc_blocks=2048, kernel_size=32, stride=16, block_size=64, top_n=16, num_inital=1,
-                      num_local=2, window_size=512, sm_scale=None, return_parts=False, cmp_slot_mapping=None):
+                      num_local=2, window_size=512, sm_scale=None, return_parts=False, cmp_slot_mapping=None,
+                      new_k=None, new_v=None, slot_mapping=None):
     """The decode step in one launch (one workgroup per request and kv head): compressed attention,
     block scores, selection, window and selected-block attention, gated combine -> o [B,QH,VD]
     (return_parts: also cmp_o, slc_o, swa_o, topk [KH,B,top_n], lse [B,QH]).  With cmp_slot_mapping [B] the kernel
     first pools the compressed K/V row completed by the newest token (what kv_mean_pooling_decode does); without it
-    the caller has pooled already."""
+    the caller has pooled already.  With new_k / new_v [B,KH,*] and slot_mapping [B] it also writes the newest token's
+    K/V rows into the pools first (what store_kvcache does)."""
     check_bf16(q)
     page, KH, D, ksr, ksh = _pool_args(k)
     _, _, VD, vsr, vsh = _pool_args(v)
@@ -208,6 +248,10 @@ def decode_one_launch(q, k, v, w, block_tables, cmp_block_tables, context_lens, 
     dev = q.device
     out = torch.empty(B, QH, VD, device=dev, dtype=q.dtype)
     parts = [torch.empty_like(out) for _ in range(3)] if return_parts else [None] * 3
+    store = new_k is not None
+    if store:
+        assert new_v is not None and slot_mapping is not None and new_k.shape == (B, KH, D)
+        assert new_v.shape == (B, KH, VD) and new_k.stride(-1) == 1 and new_v.stride(-1) == 1
     topk = torch.empty(KH, B, top_n, device=dev, dtype=torch.int32) if return_parts else None
     lse = torch.empty(B, QH, device=dev, dtype=torch.float32) if return_parts else None
     _lib.call("nsa_decode_fused", q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), ksr, ksh, v.data_ptr(), vsr,
@@ -217,7 +261,10 @@ def decode_one_launch(q, k, v, w, block_tables, cmp_block_tables, context_lens, 
               _lib.ptr(topk), topk.stride(0) if return_parts else 0, topk.stride(1) if return_parts else 0,
               _i32(context_lens).data_ptr(), _i32(block_tables).data_ptr(), block_tables.stride(0),
               _i32(cmp_block_tables).data_ptr(), cmp_block_tables.stride(0),
-              None if cmp_slot_mapping is None else _i32(cmp_slot_mapping).data_ptr(), page, B, QH, KH, D, VD,
+              None if cmp_slot_mapping is None else _i32(cmp_slot_mapping).data_ptr(), _lib.ptr(new_k),
+              new_k.stride(0) if store else 0, new_k.stride(1) if store else 0, _lib.ptr(new_v),
+              new_v.stride(0) if store else 0, new_v.stride(1) if store else 0,
+              _i32(slot_mapping).data_ptr() if store else None, page, B, QH, KH, D, VD,
               int(fixed_y_maxlen), int(fixed_num_slc_blocks), kernel_size, stride, block_size, top_n, num_inital,
               num_local, -1, window_size, sm_scale, _lib.stream_ptr())
     if return_parts:
