@@ -158,6 +158,53 @@ def staged_step(timer, q, k, v, w, wv, do, sm_scale):
     R("cmp_v_bwd", cmp_v_bwd)
 
 
+def layer_bench(dev, T, QH, KH, D, reps=20):
+    """The step either side of the core: the fused rotary embedding of q and k at the headline shape (an HBM-bound
+    kernel: q and k read and written once, the fp32 tables read once), and, for scale, forward+backward of the whole
+    attention layer (library GEMM projections with hidden = QH*D, RoPE, core, output projection)."""
+    import torch
+    from flash_nsa import HFNSA, NSAConfig, fused_apply_rope
+    q = torch.randn(1, T, QH, D, device=dev, dtype=torch.bfloat16)
+    k = torch.randn(1, T, KH, D, device=dev, dtype=torch.bfloat16)
+    ang = torch.arange(T, device=dev, dtype=torch.float32)[:, None] / (
+        10000 ** (torch.arange(0, D, 2, device=dev, dtype=torch.float32) / D))[None]
+    cos, sin = torch.cat([ang.cos(), ang.cos()], -1)[None], torch.cat([ang.sin(), ang.sin()], -1)[None]
+
+    def timeit(fn, n):
+        fn()
+        torch.cuda.synchronize()
+        s_, e_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s_.record()
+        for _ in range(n):
+            fn()
+        e_.record()
+        torch.cuda.synchronize()
+        return s_.elapsed_time(e_) / n
+
+    rope_ms = timeit(lambda: fused_apply_rope(q, k, cos, sin, inplace=True), reps)
+    nbytes = 2 * (q.numel() + k.numel()) * 2 + 2 * cos.numel() * 4
+    out = {"rope_us": rope_ms * 1e3, "rope_algorithmic_bytes": nbytes,
+           "rope_roofline": {"bound": "hbm", "achieved": nbytes / (rope_ms * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
+                             "unit": "GB/s", "frac": nbytes / (rope_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None}}
+    del q, k
+    hidden = QH * D
+    torch.manual_seed(0)
+    layer = HFNSA(NSAConfig(hidden_size=hidden, head_dim=D, num_heads=QH, num_kv_heads=KH)).to(
+        device=dev, dtype=torch.bfloat16)
+    x = (torch.randn(1, T, hidden, device=dev, dtype=torch.bfloat16) * 0.1).requires_grad_()
+    dy = torch.randn(1, T, hidden, device=dev, dtype=torch.bfloat16)
+
+    def step():
+        layer(x, (cos, sin)).backward(dy)
+        x.grad = None
+        for p_ in layer.parameters():
+            p_.grad = None
+
+    out["layer_fwd_bwd_ms"] = timeit(step, 3)
+    out["layer_workload"] = f"HFNSA layer, hidden {hidden}, one sequence T={T}, mean compression"
+    return out
+
+
 def cpu_baseline(min_seconds=12.0):
     """Oracle forward+backward of the reference's CPU-runnable case (T=4096, 16 q / 1 kv heads, fp32),
     repeated until `min_seconds` of CPU work have been timed."""
@@ -297,6 +344,7 @@ def main():
         from bench_decode import decode_bench, cache_writer_bench
         result["decode"] = decode_bench(dev)
         result["cache_writer"] = cache_writer_bench(dev)
+        result["layer"] = layer_bench(dev, T, QH, KH, D)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))

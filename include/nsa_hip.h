@@ -196,6 +196,16 @@ int nsa_paged_pool_decode(void* k_cache, int64_t k_sr, int64_t k_sh, int Dk, voi
                           int table_stride, const int32_t* cmp_slot_mapping, int B, int page_size, int H,
                           int kernel_size, int stride, void* stream);
 
+/* ---- the layer around the core ----
+ * flash_nsa/ops/rope.py:13-232 fused_apply_rope: rotate-half RoPE of q [B,N,QH,D] and k [B,N,KH,D] (element strides
+ * per batch / token / head, last dim contiguous) with cos / sin [B,N,D] (bf16, or fp32 when cos_is_fp32; a batch
+ * stride of 0 broadcasts one table); qe / ke may alias q / k (in place).  backward != 0 applies the inverse
+ * rotation to incoming gradients. */
+int nsa_rope(const void* q, int64_t q_sb, int64_t q_sn, int64_t q_sh, const void* k, int64_t k_sb, int64_t k_sn,
+             int64_t k_sh, void* qe, int64_t qe_sb, int64_t qe_sn, int64_t qe_sh, void* ke, int64_t ke_sb,
+             int64_t ke_sn, int64_t ke_sh, const void* cos, const void* sin, int64_t c_sb, int64_t c_sn,
+             int cos_is_fp32, int B, int N, int QH, int KH, int D, int backward, void* stream);
+
 /* ---- KV-cache writer (the caller side of the paged entry points) ----
  * nano-vllm/nanovllm/layers/attention.py:123-153 store_kvcache: row n of key / value (k_row_elems = KH*D contiguous
  * elements, row stride k_st) is copied to flat pool row slot_mapping[n] of k_cache / v_cache (row stride kc_sr);

@@ -388,6 +388,15 @@ def gather_rows(cache, table_row, n):
     return flat[pages * page + r % page]
 
 
+def rope(x, cos, sin):
+    """Rotate-half rotary embedding of x [..., s, h, d] with cos / sin [..., s, d] (flash_nsa/ops/rope.py:84-97
+    upstream): out[:H] = x[:H]*cos[:H] - x[H:]*sin[:H], out[H:] = x[H:]*cos[H:] + x[:H]*sin[H:], H = d/2."""
+    H = x.size(-1) // 2
+    c, s_ = cos.unsqueeze(-2), sin.unsqueeze(-2)
+    x1, x2 = x[..., :H], x[..., H:]
+    return torch.cat([x1 * c[..., :H] - x2 * s_[..., :H], x2 * c[..., H:] + x1 * s_[..., H:]], -1)
+
+
 def store_kvcache(key, value, k_cache, v_cache, slot_mapping):
     """Cache writer (nano-vllm/nanovllm/layers/attention.py:123-153 upstream): row n of key / value is copied to
     flat pool row slot_mapping[n]; negative slots are skipped.  In place on the [pages, page, KH, *] pools."""

@@ -396,6 +396,80 @@ __global__ void paged_store_pool_prefill_kernel(const bf16_t* key, int64_t k_st,
   }
 }
 
+// ------------------------------------------------------------------------------------------ rotary embedding
+// Rotate-half RoPE of q and k of one token in one pass (upstream flash_nsa/ops/rope.py:13-124): with H = D/2,
+//   out[:H] = x[:H]*cos[:H] - x[H:]*sin[:H],   out[H:] = x[H:]*cos[H:] + x[:H]*sin[H:]
+// and for the backward the inverse rotation (sin halves swapped and negated).  A thread owns 8 channels of the
+// first half and the matching 8 of the second half, so in-place operation is safe; it reads its slice of the
+// token's tables once and walks the heads (q heads, then k heads) in batches whose loads are all issued before
+// the first store.
+// grid (N, B), block 256: thread = (head slot, channel octet), 256 / (D/16) head slots
+__device__ inline void load_table8(const float* p, float (&v)[8]) {
+  const float4 lo = *reinterpret_cast<const float4*>(p), hi = *reinterpret_cast<const float4*>(p + 4);
+  v[0] = lo.x, v[1] = lo.y, v[2] = lo.z, v[3] = lo.w, v[4] = hi.x, v[5] = hi.y, v[6] = hi.z, v[7] = hi.w;
+}
+__device__ inline void load_table8(const bf16_t* p, float (&v)[8]) {
+  const bf16x8 t = ld_global_b128(p);
+#pragma unroll
+  for (int e = 0; e < 8; e++) v[e] = (float)t[e];
+}
+
+template <typename CS>
+__global__ __launch_bounds__(256) void rope_kernel(
+    const bf16_t* q, int64_t q_sb, int64_t q_sn, int64_t q_sh, const bf16_t* k, int64_t k_sb, int64_t k_sn,
+    int64_t k_sh, bf16_t* qe, int64_t qe_sb, int64_t qe_sn, int64_t qe_sh, bf16_t* ke, int64_t ke_sb, int64_t ke_sn,
+    int64_t ke_sh, const CS* cos_, const CS* sin_, int64_t c_sb, int64_t c_sn, int QH, int KH, int D, int backward) {
+  constexpr int U = 3;
+  const int H2 = D / 2, C = H2 / 8, HT = QH + KH, slots = 256 / C;
+  const int c = threadIdx.x % C, hs = threadIdx.x / C;
+  if (hs >= slots) return;
+  const int64_t n = blockIdx.x, b = blockIdx.y;
+  float c1[8], c2[8], s1[8], s2[8];
+  {
+    const CS* cp = cos_ + b * c_sb + n * c_sn + c * 8;
+    const CS* sp = sin_ + b * c_sb + n * c_sn + c * 8;
+    load_table8(cp, c1), load_table8(cp + H2, c2);
+    if (backward) {
+      load_table8(sp + H2, s1), load_table8(sp, s2);
+#pragma unroll
+      for (int e = 0; e < 8; e++) s1[e] = -s1[e], s2[e] = -s2[e];
+    } else {
+      load_table8(sp, s1), load_table8(sp + H2, s2);
+    }
+  }
+  const bf16_t* qrow = q + b * q_sb + n * q_sn + c * 8;
+  const bf16_t* krow = k + b * k_sb + n * k_sn + c * 8;
+  bf16_t* qerow = qe + b * qe_sb + n * qe_sn + c * 8;
+  bf16_t* kerow = ke + b * ke_sb + n * ke_sn + c * 8;
+  for (int h0 = hs; h0 < HT; h0 += U * slots) {
+    bf16x8 x1[U], x2[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const int h = h0 + u * slots;
+      if (h < HT) {
+        const bf16_t* src = h >= QH ? krow + (int64_t)(h - QH) * k_sh : qrow + (int64_t)h * q_sh;
+        x1[u] = ld_global_b128(src), x2[u] = ld_global_b128(src + H2);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const int h = h0 + u * slots;
+      if (h < HT) {
+        float o1[8], o2[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          const float a = (float)x1[u][e], bb = (float)x2[u][e];
+          o1[e] = a * c1[e] - bb * s1[e];
+          o2[e] = bb * c2[e] + a * s2[e];
+        }
+        bf16_t* dst = h >= QH ? kerow + (int64_t)(h - QH) * ke_sh : qerow + (int64_t)h * qe_sh;
+        *reinterpret_cast<bf16x8*>(dst) = pack8(o1[0], o1[1], o1[2], o1[3], o1[4], o1[5], o1[6], o1[7]);
+        *reinterpret_cast<bf16x8*>(dst + H2) = pack8(o2[0], o2[1], o2[2], o2[3], o2[4], o2[5], o2[6], o2[7]);
+      }
+    }
+  }
+}
+
 inline unsigned blocks_for(int64_t n, int bs) { return (unsigned)((n + bs - 1) / bs); }
 
 }  // namespace
@@ -578,6 +652,38 @@ int nsa_paged_store_pool_prefill(const void* key, int64_t k_st, int64_t k_sh, in
       (bf16_t*)v_cache, vc_sr, vc_sh, x_cu, context_lens, slot_mapping, y_cu, cmp_slot_mapping, block_tables,
       table_stride, page_size, H, kernel_size, stride);
   return nsa_check_launch("paged_store_pool_prefill");
+}
+
+int nsa_rope(const void* q, int64_t q_sb, int64_t q_sn, int64_t q_sh, const void* k, int64_t k_sb, int64_t k_sn,
+             int64_t k_sh, void* qe, int64_t qe_sb, int64_t qe_sn, int64_t qe_sh, void* ke, int64_t ke_sb,
+             int64_t ke_sn, int64_t ke_sh, const void* cos, const void* sin, int64_t c_sb, int64_t c_sn,
+             int cos_is_fp32, int B, int N, int QH, int KH, int D, int backward, void* stream) {
+  NSA_REQUIRE(D > 0 && D % 16 == 0 && D <= 4096, NSA_ERR_BAD_ARG,
+              "rope: head dim %d must be a positive multiple of 16, at most 4096", D);
+  NSA_REQUIRE(QH >= 0 && KH >= 0 && QH + KH > 0, NSA_ERR_BAD_ARG, "rope: bad head counts %d / %d", QH, KH);
+  if (B <= 0 || N <= 0) return NSA_OK;
+  NSA_REQUIRE(B <= 65535, NSA_ERR_BAD_ARG, "rope: batch %d exceeds the grid limit 65535", B);
+  // every row is moved in 16-byte pieces
+  const int64_t strides[] = {q_sb, q_sn, q_sh, k_sb, k_sn, k_sh, qe_sb, qe_sn, qe_sh, ke_sb, ke_sn, ke_sh};
+  for (int64_t st : strides)
+    NSA_REQUIRE(st % 8 == 0, NSA_ERR_BAD_ARG, "rope: stride %lld is not a multiple of 8 elements", (long long)st);
+  const int tab_align = cos_is_fp32 ? 4 : 8;
+  NSA_REQUIRE(c_sb % tab_align == 0 && c_sn % tab_align == 0, NSA_ERR_BAD_ARG,
+              "rope: table strides %lld / %lld must be multiples of %d elements", (long long)c_sb, (long long)c_sn,
+              tab_align);
+  const void* ptrs[] = {q, k, qe, ke, cos, sin};
+  for (const void* ptr : ptrs)
+    NSA_REQUIRE(((uintptr_t)ptr & 15) == 0, NSA_ERR_BAD_ARG, "rope: pointer %p is not 16-byte aligned", ptr);
+  dim3 grid((unsigned)N, (unsigned)B);
+  if (cos_is_fp32)
+    rope_kernel<float><<<grid, 256, 0, (hipStream_t)stream>>>(
+        (const bf16_t*)q, q_sb, q_sn, q_sh, (const bf16_t*)k, k_sb, k_sn, k_sh, (bf16_t*)qe, qe_sb, qe_sn, qe_sh,
+        (bf16_t*)ke, ke_sb, ke_sn, ke_sh, (const float*)cos, (const float*)sin, c_sb, c_sn, QH, KH, D, backward);
+  else
+    rope_kernel<bf16_t><<<grid, 256, 0, (hipStream_t)stream>>>(
+        (const bf16_t*)q, q_sb, q_sn, q_sh, (const bf16_t*)k, k_sb, k_sn, k_sh, (bf16_t*)qe, qe_sb, qe_sn, qe_sh,
+        (bf16_t*)ke, ke_sb, ke_sn, ke_sh, (const bf16_t*)cos, (const bf16_t*)sin, c_sb, c_sn, QH, KH, D, backward);
+  return nsa_check_launch("rope");
 }
 
 }  // extern "C"

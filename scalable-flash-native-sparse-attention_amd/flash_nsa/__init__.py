@@ -14,3 +14,5 @@ from .ops.combine import fused_sigmoid_combine
 from .modules.megatron_level_nsa import NSACore, flash_nsa_varlen_func, cp_flash_nsa_varlen_func
 
 from .inference import nsa_prefill, nsa_decode
+from .ops.rope import fused_apply_rope
+from .layers import HFNSA, NSA

@@ -263,3 +263,28 @@ def test_paged_oracle_equals_contiguous():
     assert torch.allclose(o_chunk, o_ref[500:], atol=1e-10)
     o_dec = O.nsa_paged_forward(q[-1:], kc, vc, w[-1:], torch.tensor([0, 1]), ctx, bt, cbt, cfg)
     assert torch.allclose(o_dec, o_ref[-1:], atol=1e-10)
+
+
+def test_rope_is_a_rotation_of_channel_pairs():
+    """The oracle's rotate-half RoPE with the usual tables (cos/sin of position * inverse frequency, both halves
+    equal) is the complex multiplication (x1 + i x2) * exp(i theta) on the pairs (d, d + D/2); with independent
+    half-tables it is checked against an explicit per-element loop."""
+    g = torch.Generator().manual_seed(0)
+    s, h, d = 7, 3, 16
+    x = torch.randn(2, s, h, d, generator=g, dtype=torch.float64)
+    inv = 1.0 / (10000 ** (torch.arange(0, d, 2, dtype=torch.float64) / d))
+    ang = torch.arange(s, dtype=torch.float64)[:, None] * inv[None]          # [s, d/2]
+    cos, sin = torch.cat([ang.cos(), ang.cos()], -1), torch.cat([ang.sin(), ang.sin()], -1)
+    out = O.rope(x, cos.expand(2, s, d), sin.expand(2, s, d))
+    z = torch.complex(x[..., :d // 2], x[..., d // 2:]) * torch.polar(torch.ones_like(ang), ang)[None, :, None, :]
+    assert torch.allclose(out[..., :d // 2], z.real, atol=1e-12) and torch.allclose(out[..., d // 2:], z.imag, atol=1e-12)
+    assert torch.allclose(out.norm(dim=-1), x.norm(dim=-1), atol=1e-12)      # a rotation keeps the norm
+    c2, s2 = torch.randn(2, s, d, generator=g, dtype=torch.float64), torch.randn(2, s, d, generator=g, dtype=torch.float64)
+    out = O.rope(x, c2, s2)
+    H = d // 2
+    for b in range(2):
+        for n in range(s):
+            for e in range(H):
+                a, bb = x[b, n, 1, e], x[b, n, 1, H + e]
+                assert abs(out[b, n, 1, e] - (a * c2[b, n, e] - bb * s2[b, n, e])) < 1e-12
+                assert abs(out[b, n, 1, H + e] - (bb * c2[b, n, H + e] + a * s2[b, n, H + e])) < 1e-12
