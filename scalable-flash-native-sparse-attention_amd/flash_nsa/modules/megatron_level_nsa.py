@@ -41,7 +41,9 @@ def weight_grad(inp, grad_out, weight):
     main_grad = getattr(weight, "main_grad", None)
     if main_grad is None:
         return torch.matmul(grad_out.t(), inp)
-    main_grad.addmm_(grad_out.t().float(), inp.float())
+    # bf16 operands, fp32 accumulator added to the fp32 buffer in the GEMM's epilogue: no rounding of dW to bf16
+    # (upstream's wgrad GEMM adds its fp32 accumulator tiles the same way, flash_nsa/ops/gemm.py:131-133)
+    torch.addmm(main_grad, grad_out.t(), inp, out_dtype=torch.float32, out=main_grad)
     if hasattr(weight, "grad_added_to_main_grad"):
         weight.grad_added_to_main_grad = True
         return torch.empty(main_grad.shape, dtype=inp.dtype, device=inp.device)

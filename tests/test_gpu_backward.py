@@ -272,3 +272,78 @@ def test_two_stream_backward_equals_single_stream(device):
     assert_close(a[2], b[2], "dk", atol=2e-3, rtol=8e-3, row_scale=True)
     assert_close(a[3], b[3], "dv", atol=2e-3, rtol=8e-3, row_scale=True)
     assert_close(a[5], b[5], "d cmp_v_weight", atol=2e-3, rtol=2e-2, row_scale=True)
+
+
+@pytest.mark.parametrize("methods", [("mean", "mean"), ("sigmoid-mul", "swiglu"), ("linear", "mean")])
+def test_recompute_flags_change_memory_not_results(device, methods):
+    """Every recompute_* flag on (upstream flash_nsa/modules/megatron_level_nsa.py:107-147): the forward keeps fewer
+    bytes alive, the backward rebuilds them with the same kernels, so output and gradients are those of the run that
+    saved everything (dq / dWk / dWv bit for bit; dk / dv / dw up to the order of their fp32 atomic additions)."""
+    from flash_nsa import NSAConfig, NSACore, NSAHelper
+    lens, QH, KH, D = [900, 420], 8, 2, 128
+    cu = make_cu(lens).to(device)
+    T = sum(lens)
+    q, k, v, w = make_qkvw(T, QH, KH, D, seed=90)
+    do = randn_bf16(T, QH, D, seed=95).to(device)
+    flags = ("recompute_cmp_kv", "recompute_cmp_o", "recompute_slc_o", "recompute_swa_o")
+    runs = {}
+    for on in (False, True):
+        cfg = NSAConfig(head_dim=D, num_heads=QH, num_kv_heads=KH, top_n=8, window_size=128, cmp_k_method=methods[0],
+                        cmp_v_method=methods[1], **{f: on for f in flags})
+        torch.manual_seed(0)
+        mod = NSACore(cfg).to(device=device, dtype=torch.bfloat16)
+        leaves = [t.to(device).requires_grad_() for t in (q, k, v, w)]
+        torch.cuda.synchronize()
+        before = torch.cuda.memory_allocated()
+        out = mod(*leaves, cu)
+        torch.cuda.synchronize()
+        held = torch.cuda.memory_allocated() - before
+        out.backward(do)
+        grads = [t.grad for t in leaves] + [p.grad for p in (mod.cmp_k_weight, mod.cmp_v_weight) if p is not None]
+        runs[on] = (out.detach(), grads, held)
+        assert all(getattr(NSAHelper, f) == on for f in flags)
+    NSAHelper.set_recompute()
+    (o0, g0, held0), (o1, g1, held1) = runs[False], runs[True]
+    assert torch.equal(o0, o1)
+    assert torch.equal(g0[0], g1[0]), "dq"
+    for a, b, name in zip(g0[1:4], g1[1:4], ("dk", "dv", "dw")):
+        assert_close(a, b.float(), name, atol=1e-5, rtol=8e-3)
+    for a, b in zip(g0[4:], g1[4:]):
+        assert_close(a, b.float(), "dW", atol=1e-5, rtol=8e-3)
+    # three branch outputs [T,QH,D] bf16 + their lse are no longer kept
+    assert held0 - held1 >= 3 * T * QH * D * 2, (held0, held1)
+
+
+def test_weight_gradient_accumulates_into_main_grad(device):
+    """A compression weight with an fp32 `main_grad` (the mixed-precision optimizers of Megatron keep one, upstream
+    flash_nsa/modules/megatron_level_nsa.py:20-44): the backward adds dW to it without rounding to bf16 first and,
+    when the parameter carries `grad_added_to_main_grad`, sets it and returns a placeholder gradient."""
+    from flash_nsa import NSAConfig, NSACore
+    lens, QH, KH, D = [700, 300], 4, 2, 64
+    cu = make_cu(lens).to(device)
+    T = sum(lens)
+    q, k, v, w = make_qkvw(T, QH, KH, D, seed=100)
+    do = randn_bf16(T, QH, D, seed=105).to(device)
+    cfg = NSAConfig(head_dim=D, num_heads=QH, num_kv_heads=KH, top_n=8, window_size=128, cmp_k_method="linear",
+                    cmp_v_method="sigmoid-mul")
+
+    def run(with_main_grad):
+        torch.manual_seed(0)
+        mod = NSACore(cfg).to(device=device, dtype=torch.bfloat16)
+        if with_main_grad:
+            for i, p in enumerate((mod.cmp_k_weight, mod.cmp_v_weight)):
+                p.main_grad = torch.full(p.shape, 0.5 + i, device=device, dtype=torch.float32)
+            mod.cmp_v_weight.grad_added_to_main_grad = False
+        leaves = [t.to(device).requires_grad_() for t in (q, k, v, w)]
+        mod(*leaves, cu).backward(do)
+        return mod
+
+    plain, mixed = run(False), run(True)
+    for i, name in enumerate(("cmp_k_weight", "cmp_v_weight")):
+        want = getattr(plain, name).grad.float() + (0.5 + i)
+        got = getattr(mixed, name).main_grad
+        # the plain gradient went through one rounding to bf16, the accumulated one did not
+        assert_close(got, want, name, atol=2e-2, rtol=1e-2, row_scale=True)
+    assert mixed.cmp_k_weight.grad is None
+    assert mixed.cmp_v_weight.grad_added_to_main_grad is True
+    assert mixed.cmp_v_weight.grad is not None and mixed.cmp_v_weight.grad.shape == mixed.cmp_v_weight.shape

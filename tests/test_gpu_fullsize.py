@@ -54,6 +54,33 @@ def test_c2_prefix_consistency_and_oracle_slice(device):
     assert_close(o16, ref, "o (slice of the 64K run)")
 
 
+def test_c2_recompute_and_learned_compression_full_size(device):
+    """T = 65536 with the benchmark's learned V compression (sigmoid-mul) and a learned K compression: the run that
+    recomputes every intermediate in the backward returns the output and dq of the run that keeps them, bit for bit,
+    and the weight gradients agree to the order of the fp32 atomic additions feeding them."""
+    from flash_nsa import NSAConfig, NSACore, NSAHelper
+    T, QH, KH, D = 65536, 64, 4, 128
+    q, k, v, w, do = [dev_randn(s, 20 + i, device) for i, s in
+                      enumerate([(T, QH, D), (T, KH, D), (T, KH, D), (T, QH, 3), (T, QH, D)])]
+    cu = torch.tensor([0, T], dtype=torch.int32, device=device)
+    res = {}
+    for rec in (False, True):
+        cfg = NSAConfig(head_dim=D, num_heads=QH, num_kv_heads=KH, cmp_k_method="linear", cmp_v_method="sigmoid-mul",
+                        recompute_cmp_kv=rec, recompute_cmp_o=rec, recompute_slc_o=rec, recompute_swa_o=rec)
+        torch.manual_seed(0)
+        core = NSACore(cfg).to(device=device, dtype=torch.bfloat16)
+        qg = q.clone().requires_grad_()
+        out = core(qg, k, v, w, cu)
+        out.backward(do)
+        res[rec] = (out.detach(), qg.grad, core.cmp_k_weight.grad, core.cmp_v_weight.grad)
+    NSAHelper.set_recompute()
+    assert torch.isfinite(res[True][1]).all()
+    assert torch.equal(res[False][0], res[True][0]) and torch.equal(res[False][1], res[True][1])
+    for a, b, name in zip(res[False][2:], res[True][2:], ("dWk", "dWv")):
+        assert torch.isfinite(a).all()
+        assert_close(b, a.float(), name, atol=2e-2, rtol=1e-2, row_scale=True)
+
+
 def test_c3_packed_batch_equals_single_sequences(device):
     """8 sequences with lengths uniform in [4096, 8192] (seed 1), forward + backward: packed == one by one."""
     from flash_nsa import NSAConfig, NSACore
