@@ -1,6 +1,7 @@
 """Benchmark of the NSA hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--seq-len T] [--no-cpu] [--no-decode]
+    python bench.py --sweep 4096,8192,16384,32768,65536,131072,262144,524288,1048576
 
 A step is one forward+backward of the NSA core (NSACore: mean K-compression, sigmoid-mul V-compression,
 kernel 32 / stride 16 / block 64 / top-16 / window 512) on one causal sequence of T=65536 tokens,
@@ -146,7 +147,7 @@ def staged_step(timer, q, k, v, w, wv, do, sm_scale):
     R("cmp_dkdv", lambda: _lib.call("nsa_cmp_attn_bwd_dkdv", *cc, dck.data_ptr(), dck.stride(0), dck.stride(1),
                                     dcv.data_ptr(), dcv.stride(0), dcv.stride(1), H.x_cu_seqlens.data_ptr(),
                                     H.y_cu_seqlens.data_ptr(), H.batch, H.x_maxlen, H.y_maxlen, QH, KH, D, VD,
-                                    H.kernel_size, H.stride, 2048, sm_scale, _lib.stream_ptr()))
+                                    H.kernel_size, H.stride, 0, sm_scale, _lib.stream_ptr()))
     R("pool_k_bwd", lambda: mean_pooling_bwd(k, dck.to(k.dtype), dk))
 
     def cmp_v_bwd():
@@ -205,6 +206,54 @@ def layer_bench(dev, T, QH, KH, D, reps=20):
     return out
 
 
+# forward / backward ms the reference reports on one H800 for one causal sequence of this length, 64q/4kv heads,
+# d=128, mean compression (upstream README.md:213-237)
+REFERENCE_H800_MS = {4096: (1.370, 2.772), 8192: (2.630, 5.571), 16384: (5.660, 12.322), 32768: (13.237, 28.960),
+                     65536: (34.162, 73.689), 131072: (101.123, 213.904)}
+
+
+def length_sweep(lengths, QH=64, KH=4, D=128):
+    """Forward and backward time of NSACore (mean compression, as the reference's table) per sequence length; prints
+    one JSON line per length.  Lengths of 2^18 and more show that one GPU's memory holds what the reference shards
+    over eight (its 1M-token run: 575.6 / 1509.2 ms on 8 GPUs with context parallelism, upstream README.md:275-283)."""
+    import torch
+    from flash_nsa import NSAConfig, NSACore
+    dev = torch.device("cuda:0")
+    core = NSACore(NSAConfig(head_dim=D, num_heads=QH, num_kv_heads=KH))
+    for T in lengths:
+        g = torch.Generator(device=dev).manual_seed(0)
+        rnd = lambda *s_: torch.randn(*s_, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        q, k, v, w, do = rnd(T, QH, D), rnd(T, KH, D), rnd(T, KH, D), rnd(T, QH, 3), rnd(T, QH, D)
+        cu = torch.tensor([0, T], device=dev, dtype=torch.int32)
+        for t in (q, k, v, w):
+            t.requires_grad_()
+        reps = 5 if T <= 131072 else 2
+        ev = lambda: torch.cuda.Event(enable_timing=True)
+        fwd_ms = bwd_ms = 0.0
+        torch.cuda.reset_peak_memory_stats()
+        for it in range(reps + 1):  # the first pass is a warm-up
+            e0, e1, e2 = ev(), ev(), ev()
+            e0.record()
+            out = core(q, k, v, w, cu)
+            e1.record()
+            out.backward(do)
+            e2.record()
+            torch.cuda.synchronize()
+            if it:
+                fwd_ms += e0.elapsed_time(e1) / reps
+                bwd_ms += e1.elapsed_time(e2) / reps
+            for t in (q, k, v, w):
+                t.grad = None
+        fl = stage_flops([T], QH, D, D)
+        ref = REFERENCE_H800_MS.get(T)
+        print(json.dumps({"seq_len": T, "fwd_ms": round(fwd_ms, 3), "bwd_ms": round(bwd_ms, 3),
+                          "fwd_tflops": round(fl["fwd_total"] / fwd_ms / 1e9, 1),
+                          "bwd_tflops": round(fl["bwd_total"] / bwd_ms / 1e9, 1),
+                          "peak_mem_gib": round(torch.cuda.max_memory_allocated() / 2**30, 2),
+                          "reference_h800_fwd_bwd_ms": ref}), flush=True)
+        del q, k, v, w, do, out
+
+
 def cpu_baseline(min_seconds=12.0):
     """Oracle forward+backward of the reference's CPU-runnable case (T=4096, 16 q / 1 kv heads, fp32),
     repeated until `min_seconds` of CPU work have been timed."""
@@ -248,6 +297,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain 1 GiB device-to-device copy kernel, so that a counter run of this "
                          "command holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE with")
+    ap.add_argument("--sweep", type=str, default=None,
+                    help="comma-separated sequence lengths: print forward / backward times per length and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (--gpus 1); multi-GPU sharding is a design note only",
@@ -258,6 +309,9 @@ def main():
     from flash_nsa import NSAConfig, NSACore
     from flash_nsa import _lib
     _lib.LIB.load()  # fail loudly if the HIP library is missing
+    if args.sweep:
+        length_sweep([int(x) for x in args.sweep.split(",")])
+        return
     dev = torch.device("cuda:0")
     T, QH, KH, D = args.seq_len, 64, 4, 128
     g = torch.Generator(device=dev).manual_seed(0)

@@ -102,7 +102,8 @@ int nsa_cmp_attn_bwd_dq_final(const void* q, int64_t q_st, int64_t q_sh, const v
                               const int32_t* x_cu, const int32_t* y_cu, int B, int x_maxlen, int QH, int KH, int D,
                               int VD, int kernel_size, int stride, float sm_scale, void* stream);
 /* flash_nsa/ops/compress_attn.py:650-690 (_cmp_dkdv_kernel launch, dkdv_repeat=False): fp32 atomic adds into
- * dck/dcv [y_len,KH,*], which the caller zero-fills; queries are cut into chunks of q_chunk_tokens */
+ * dck/dcv [y_len,KH,*], which the caller zero-fills; queries are cut into chunks of q_chunk_tokens
+ * (<= 0: chosen from the sizes so that short batches still fill the GPU) */
 int nsa_cmp_attn_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr, int64_t ck_sh,
                           const void* cv, int64_t cv_sr, int64_t cv_sh, const void* dO, int64_t do_st,
                           int64_t do_sh, const float* lse, int64_t lse_st, int64_t lse_sh, const float* delta,
@@ -134,8 +135,12 @@ int nsa_slc_attn_bwd_dq(const void* q, int64_t q_st, int64_t q_sh, const void* k
  *   csr_off  [KH][nblk_total+1] absolute start of each (kv head, global block) list inside csr_tok
  *   csr_tok  [KH*T*top_n]       query tokens (index local to their sequence), ascending within a list
  *   item_off [KH][nblk_total+1] prefix count of list chunks of chunk_tokens tokens (work items of the dk/dv pass)
- *   workspace: int32 scratch of nsa_inverse_index_workspace_elems(T,KH,nblk_total) elements */
+ *   workspace: int32 scratch of nsa_inverse_index_workspace_elems(T,KH,nblk_total) elements
+ * nsa_slc_bwd_chunk_tokens: the chunk_tokens this library suggests for a batch of T tokens (1024 for long batches,
+ * less when that would leave the dk/dv pass too few work items); any positive value is valid as long as the
+ * builder and nsa_slc_attn_bwd_dkdv get the same one */
 int64_t nsa_inverse_index_workspace_elems(int T, int KH, int nblk_total);
+int nsa_slc_bwd_chunk_tokens(int T, int KH, int top_n);
 int nsa_build_inverse_index(const int32_t* topk, int64_t tk_sh, int64_t tk_st, int top_n, const int32_t* x_cu,
                             const int32_t* kblk_cu, int B, int T, int KH, int nblk_total, int block_size,
                             int chunk_tokens, int32_t* csr_off, int32_t* csr_tok, int32_t* item_off,

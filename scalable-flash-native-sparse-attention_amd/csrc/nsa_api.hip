@@ -230,7 +230,14 @@ int nsa_cmp_attn_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void*
   if (rc) return rc;
   rc = check_nsa_sizes("cmp_attn_bwd_dkdv", kernel_size, stride, 0);
   if (rc) return rc;
-  NSA_REQUIRE(q_chunk_tokens > 0, NSA_ERR_BAD_ARG, "cmp_attn_bwd_dkdv: q_chunk_tokens must be positive");
+  if (q_chunk_tokens <= 0) {
+    // Largest power of two in [128, 2048] that still cuts the launch into about four workgroups per CU:
+    // (128-key tiles) x (query chunks that see them, about half) x kv heads x sequences.
+    const int64_t tiles = (y_maxlen + 127) / 128;
+    const int64_t want = (int64_t)B * KH * tiles * x_maxlen / (2 * 1024);
+    q_chunk_tokens = 128;
+    while (q_chunk_tokens < 2048 && q_chunk_tokens * 2 <= want) q_chunk_tokens *= 2;
+  }
   BwdCommon c{q, q_st, q_sh, ck, ck_sr, ck_sh, cv, cv_sr, cv_sh, dO, do_st, do_sh, lse, lse_st, lse_sh, delta,
               delta_st, delta_sh};
   NsaBwdTileParams p = make_bwd(c, QH, KH, sm_scale);
@@ -241,6 +248,16 @@ int nsa_cmp_attn_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void*
   p.kernel_size = kernel_size; p.stride = stride;
   p.q_chunk_tokens = q_chunk_tokens;
   return nsa_bwd_dkdv_launch(p, 0, B, x_maxlen, y_maxlen, D, VD, 0, (hipStream_t)stream);
+}
+
+int nsa_slc_bwd_chunk_tokens(int T, int KH, int top_n) {
+  // list chunk (tokens per work item of the selected-attention dk/dv pass): 1024 for long batches, smaller when
+  // that would leave fewer than about 2048 two-wave work items; below 256 the fp32 atomic additions of the many
+  // items cost more than the idle CUs
+  const int64_t want = (int64_t)KH * T * top_n / 2048;
+  int c = 256;
+  while (c < 1024 && c * 2 <= want) c *= 2;
+  return c;
 }
 
 int nsa_swa_bwd_dq(const void* q, int64_t q_st, int64_t q_sh, const void* k, int64_t k_sr, int64_t k_sh,

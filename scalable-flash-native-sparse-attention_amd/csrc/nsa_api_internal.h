@@ -47,7 +47,8 @@ struct NsaTopkParams {
   int G, KH;
   float scale_log2;
   int kernel_size, stride, block_size, top_n, num_init, num_local, ignore_index;
-  int nb_max;  // selection blocks of the longest context (length of an LDS score row)
+  int nb_max;  // selection blocks of the longest context
+  int seg_blocks;  // set by the launcher: 0 = an LDS score row holds all nb_max blocks; else blocks per segment
 };
 
 int nsa_fwd_tile_launch(const NsaFwdTileParams& p, int mode, bool paged, int B, int max_q_len, int D, int VD,

@@ -133,6 +133,23 @@ NSA_DEVICE int wave_argmax_lowest(float score, int index, bool has_candidate) {
   return hi == 0 ? 0x7fffffff : (int)(0x7fffffff - lo);
 }
 
+// Same reduction, also returning the winner's score (undefined when there is no candidate).
+NSA_DEVICE int wave_argmax_lowest_score(float score, int index, bool has_candidate, float& win_score) {
+  uint32_t b = __builtin_bit_cast(uint32_t, score);
+  b = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+  uint64_t key = has_candidate ? (((uint64_t)b << 32) | (uint32_t)(0x7fffffff - index)) : 0ull;
+  key = dpp_max_step<0x111, 0xf>(key);
+  key = dpp_max_step<0x112, 0xf>(key);
+  key = dpp_max_step<0x114, 0xf>(key);
+  key = dpp_max_step<0x118, 0xf>(key);
+  key = dpp_max_step<0x142, 0xa>(key);
+  key = dpp_max_step<0x143, 0xc>(key);
+  uint32_t lo = __builtin_amdgcn_readlane((uint32_t)key, 63);
+  uint32_t hi = __builtin_amdgcn_readlane((uint32_t)(key >> 32), 63);
+  win_score = __builtin_bit_cast(float, (hi & 0x80000000u) ? (hi & 0x7fffffffu) : ~hi);
+  return hi == 0 ? 0x7fffffff : (int)(0x7fffffff - lo);
+}
+
 __host__ __device__ inline int cdiv_i(int a, int b) { return (a + b - 1) / b; }
 
 // error codes returned by the C entry points

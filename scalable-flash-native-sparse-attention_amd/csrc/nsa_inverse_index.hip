@@ -1,6 +1,6 @@
 // Inverse of the top-n selection: for every (kv head, selection block) the ascending list of query tokens that
 // selected the block, as a CSR (offsets + token ids), plus the prefix of fixed-size list chunks that the dK/dV
-// kernel uses as its work items.  Built by a deterministic counting sort: per-1024-token-chunk histograms,
+// kernel uses as its work items.  Built by a deterministic counting sort: per-token-chunk histograms,
 // a scan over chunks and blocks, then an in-order fill, so no sort and no dense (block x token) scratch.
 // Upstream: flash_nsa/ops/topk.py:782-945 (get_bind_from_find, dense scatter + per-row sort).
 #include "nsa_common.h"
@@ -8,7 +8,9 @@
 
 namespace {
 
-constexpr int CT = 1024;  // tokens per counting chunk
+// Tokens per counting chunk: short chunks give the serial in-order fill more parallelism, long ones keep the
+// [KH][chunks][blocks] histogram workspace small for very long batches.
+__host__ __device__ inline int counting_chunk(int T) { return T <= 131072 ? 256 : 1024; }
 
 __device__ __forceinline__ int find_seq(const int32_t* x_cu, int B, int tok) {
   int lo = 0, hi = B;  // last b with x_cu[b] <= tok
@@ -26,6 +28,7 @@ __global__ void csr_count_kernel(const int32_t* topk, int64_t tk_sh, int64_t tk_
   const int chunk = blockIdx.x, kh = blockIdx.y;
   for (int i = threadIdx.x; i < nblk; i += blockDim.x) hist[i] = 0;
   __syncthreads();
+  const int CT = counting_chunk(T);
   const int t0 = chunk * CT;
   const int t1 = min(T, t0 + CT);
   for (int idx = threadIdx.x; idx < (t1 - t0) * top_n; idx += blockDim.x) {
@@ -67,18 +70,19 @@ __global__ __launch_bounds__(1024) void csr_scan_kernel(int32_t* chunk_cnt, int 
     sum_a += base;
     sum_b += (base + chunk_tokens - 1) / chunk_tokens;
   }
+  // exclusive scan of the per-thread sums (Hillis-Steele over the 1024 threads)
   part_a[tid] = sum_a;
   part_b[tid] = sum_b;
   __syncthreads();
-  if (tid == 0) {
-    int ra = 0, rb = 0;
-    for (int i = 0; i < 1024; i++) {
-      int a = part_a[i], bb = part_b[i];
-      part_a[i] = ra; part_b[i] = rb;
-      ra += a; rb += bb;
-    }
+  for (int d = 1; d < 1024; d <<= 1) {
+    const int a = tid >= d ? part_a[tid - d] : 0, bb = tid >= d ? part_b[tid - d] : 0;
+    __syncthreads();
+    part_a[tid] += a;
+    part_b[tid] += bb;
+    __syncthreads();
   }
-  __syncthreads();
+  part_a[tid] -= sum_a;
+  part_b[tid] -= sum_b;
   int ra = part_a[tid] + (int)((int64_t)kh * list_cap), rb = part_b[tid];
   for (int j = j0; j < j1; j++) {
     int total = csr_off[(int64_t)kh * (nblk + 1) + j];
@@ -106,27 +110,50 @@ __global__ __launch_bounds__(64) void csr_fill_kernel(const int32_t* topk, int64
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const int CT = counting_chunk(T);
   const int t0 = chunk * CT;
   const int t1 = min(T, t0 + CT);
   if (t0 >= t1) return;
+  // The list positions depend on the order of the tokens, so the wave walks them one by one; the selection rows
+  // do not, and are fetched a batch ahead so that the walk never waits for memory.
+  constexpr int PF = 16;
   int b = find_seq(x_cu, B, t0);
-  for (int tok = t0; tok < t1; tok++) {
-    while (tok >= x_cu[b + 1]) b++;
-    const int n = tok - x_cu[b];
-    const int nvalid = min(top_n, n / block_size + 1);
-    if (lane < nvalid) {
-      int j = topk[(int64_t)kh * tk_sh + (int64_t)tok * tk_st + lane];
-      int nb = kblk_cu[b + 1] - kblk_cu[b];
-      if (j >= 0 && j < nb) {
-        int jb = kblk_cu[b] + j;
-        int pos = cursor[jb];
-        cursor[jb] = pos + 1;
-        csr_tok[pos] = n;
+  int x_begin = x_cu[b], x_end = x_cu[b + 1], kb_begin = kblk_cu[b], nb = kblk_cu[b + 1] - kb_begin;
+  const int32_t* row0 = topk + (int64_t)kh * tk_sh;
+  int nxt[PF], cur[PF];
+  auto fetch = [&](int tb) {
+#pragma unroll
+    for (int u = 0; u < PF; u++)
+      nxt[u] = (tb + u < t1 && lane < top_n) ? row0[(int64_t)(tb + u) * tk_st + lane] : -1;
+  };
+  fetch(t0);
+  for (int tb = t0; tb < t1; tb += PF) {
+#pragma unroll
+    for (int u = 0; u < PF; u++) cur[u] = nxt[u];
+    if (tb + PF < t1) fetch(tb + PF);
+#pragma unroll
+    for (int u = 0; u < PF; u++) {
+      const int tok = tb + u;
+      if (tok >= t1) break;
+      if (tok >= x_end) {  // next (non-empty) sequence: the only loads inside the walk
+        do { b++; } while (tok >= x_cu[b + 1]);
+        x_begin = x_cu[b], x_end = x_cu[b + 1], kb_begin = kblk_cu[b], nb = kblk_cu[b + 1] - kb_begin;
       }
+      const int n = tok - x_begin;
+      const int nvalid = min(top_n, n / block_size + 1);
+      if (lane < nvalid) {
+        const int j = cur[u];
+        if (j >= 0 && j < nb) {
+          const int jb = kb_begin + j;
+          const int pos = cursor[jb];
+          cursor[jb] = pos + 1;
+          csr_tok[pos] = n;
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
 }
 
@@ -135,6 +162,7 @@ __global__ __launch_bounds__(64) void csr_fill_kernel(const int32_t* topk, int64
 extern "C" {
 
 int64_t nsa_inverse_index_workspace_elems(int T, int KH, int nblk_total) {
+  const int CT = counting_chunk(T);
   int64_t nchunks = (T + CT - 1) / CT;
   return (int64_t)KH * nchunks * nblk_total;
 }
@@ -153,6 +181,7 @@ int nsa_build_inverse_index(const int32_t* topk, int64_t tk_sh, int64_t tk_st, i
   NSA_REQUIRE(workspace_elems >= nsa_inverse_index_workspace_elems(T, KH, nblk_total), NSA_ERR_WORKSPACE,
               "build_inverse_index: workspace of %lld ints is too small", (long long)workspace_elems);
   hipStream_t s = (hipStream_t)stream;
+  const int CT = counting_chunk(T);
   int nchunks = (T + CT - 1) / CT;
   size_t lds = (size_t)nblk_total * sizeof(int);
   dim3 grid(nchunks, KH);

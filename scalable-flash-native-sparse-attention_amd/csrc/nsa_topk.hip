@@ -97,6 +97,58 @@ NSA_DEVICE int select_row(float* imp, int t, int nb_max, const NsaTopkParams& p,
   return result;
 }
 
+// Segmented selection, for contexts whose score rows do not fit LDS.  The LDS row of a token holds the scores of one
+// segment of selection blocks (row[jj] = block j0 + jj); once the compressed keys of the segment are folded, its
+// `count` finished blocks are merged with the winners of the earlier segments (cand_s / cand_i, `ncand` slots in
+// LDS, empty slots have index 0x7fffffff) by the same repeated arg-max, lowest index on ties -- so the list after
+// the last segment is the list the one-pass selector produces.  Forced blocks never enter the list.  On return
+// lane r < ncand holds the r-th winner (index, or 0x7fffffff) and the LDS list is updated.
+NSA_DEVICE int merge_segment(float* row, int count, int j0, float* cand_s, int* cand_i, int ncand, bool first, int t,
+                             int nb_max, const NsaTopkParams& p, int lane) {
+  const int nk = t / p.block_size;
+  const int jmax = min(nk, nb_max - 1);
+  for (int jj = lane; jj < count; jj += 64) {
+    const int j = j0 + jj;
+    if (j > jmax || j < p.num_init || j > nk - p.num_local) row[jj] = -3.f;
+  }
+  if (first && lane < ncand) cand_i[lane] = 0x7fffffff;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  float my_s = -3.f;
+  int my_i = 0x7fffffff;
+  for (int r = 0; r < ncand; r++) {
+    float best = -2.f;
+    int bj = 0x7fffffff;
+    for (int jj = lane; jj < count; jj += 64) {
+      const float x = row[jj];
+      if (x > best) { best = x; bj = j0 + jj; }
+    }
+    if (lane < ncand) {  // winners of earlier segments: lower block numbers, so they win ties
+      const int ci = cand_i[lane];
+      const float x = cand_s[lane];
+      if (ci != 0x7fffffff && (x > best || (x == best && ci < bj))) { best = x; bj = ci; }
+    }
+    float ws;
+    const int w = wave_argmax_lowest_score(best, bj, bj != 0x7fffffff, ws);
+    if (w == 0x7fffffff) break;  // wave-uniform: nothing left
+    if (lane == r) { my_s = ws; my_i = w; }
+    if (w >= j0) {
+      if (lane == 0) row[w - j0] = -3.f;
+    } else if (lane < ncand && cand_i[lane] == w) {
+      cand_i[lane] = 0x7fffffff;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+  if (lane < ncand) { cand_s[lane] = my_s; cand_i[lane] = my_i; }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  return my_i;
+}
+
 // Workgroup = 4 waves on the same 64 (token, head) rows (two MFMA row blocks); the compressed keys are cut in units
 // of 32 that are dealt to the waves (wave w takes unit 4*tile + w of every 128-key tile).  A wave stages the rows of
 // its unit in a private LDS slot (coalesced whole-row loads, one tile ahead through registers), reads each K
@@ -116,7 +168,7 @@ __global__ __launch_bounds__(256, 2) void topk_kernel(NsaTopkParams p) {
   using SM = SlotMap<GP>;
   __shared__ __attribute__((aligned(16))) bf16_t Ks_all[4 * UK * KLD];
   __shared__ float Pst[2 * TWG * PLD];
-  extern __shared__ float imp_all[];  // [TWG][nb_max]
+  extern __shared__ float imp_all[];  // [TWG][W] scores, then (segmented mode) [TWG][ncand] scores + indices
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -139,8 +191,16 @@ __global__ __launch_bounds__(256, 2) void topk_kernel(NsaTopkParams p) {
   const int32_t* table = PAGED ? p.table + (int64_t)b * p.table_stride : nullptr;
   const int nb_max = p.nb_max;
   const int Bs = p.block_size, Kz = p.kernel_size, St = p.stride;
+  // segmented mode: a score row covers blocks [j0, j0 + seg] plus the block a segment's last tile only starts
+  const int seg = p.seg_blocks;
+  const int W = seg > 0 ? seg + 1 : nb_max;
+  const int ncand = max(p.top_n - p.num_init - p.num_local, 0);
+  float* cand_s_all = imp_all + TWG * W;
+  int* cand_i_all = reinterpret_cast<int*>(cand_s_all + TWG * ncand);
+  const int tiles_per_seg = seg > 0 ? seg / ((St * KT) / Bs) : 0x7fffffff;
+  int j0 = 0;
 
-  for (int i = tid; i < TWG * nb_max; i += 256) imp_all[i] = 0.f;
+  for (int i = tid; i < TWG * W; i += 256) imp_all[i] = 0.f;
   bf16_t* Ks = Ks_all + wave * UK * KLD;
 
   const int t_hi_wg = min(n0 + TWG - 1, xl - 1) + qoff;
@@ -291,13 +351,14 @@ __global__ __launch_bounds__(256, 2) void topk_kernel(NsaTopkParams p) {
     if (fold_fast) {
       const int j = (St * kt) / Bs + f_jj;
       if (f_on && j < nb_max) {
-        float acc = imp_all[f_tk * nb_max + j];
+        float* cell = &imp_all[f_tk * W + (j - j0)];  // j - j0 <= seg: a tile stays inside its segment
+        float acc = *cell;
 #pragma unroll
         for (int r = 0; r < 8; r++) {
           const int i = f_rel0 + r;
           if (r < f_nloops && i >= 0 && i < KT) acc += pst[f_tk * PLD + i] * f_w[r];
         }
-        imp_all[f_tk * nb_max + j] = acc;
+        *cell = acc;
       }
     } else {
       const int j_lo = (St * kt) / Bs;
@@ -319,8 +380,67 @@ __global__ __launch_bounds__(256, 2) void topk_kernel(NsaTopkParams p) {
         imp_all[tk * nb_max + j] = acc;
       }
     }
+    // ---- segmented mode: at the end of a segment merge its finished blocks into the running winners ----
+    if (seg > 0 && ((tile + 1) % tiles_per_seg == 0 || tile == ntiles - 1)) {
+      const bool last = tile == ntiles - 1;
+      const int count = last ? W : seg;
+      __syncthreads();  // the fold of this tile is complete
+      for (int tk = wave; tk < TWG; tk += 4) {
+        const int n = n0 + tk;
+        if (n >= xl) break;
+        float* row = imp_all + tk * W;
+        const int64_t tok = x0 + n;
+        if (p.imp_out != nullptr) {
+          float* dst = p.imp_out + (int64_t)kh * p.imp_sh + tok * p.imp_st;
+          for (int jj = lane; jj < count; jj += 64)
+            if (j0 + jj < p.imp_cols) dst[j0 + jj] = j0 + jj < nb_max ? row[jj] : 0.f;
+          if (last)
+            for (int j = j0 + count + lane; j < p.imp_cols; j += 64) dst[j] = 0.f;
+        }
+        const float carry = row[seg];
+        const int win = merge_segment(row, count, j0, cand_s_all + tk * ncand, cand_i_all + tk * ncand, ncand, j0 == 0,
+                                      n + qoff, nb_max, p, lane);
+        if (last) {
+          const int t = n + qoff, nk = t / Bs;
+          const int nsel = min(p.top_n, nk + 1), forced = p.num_init + p.num_local;
+          int result = p.ignore_index;
+          if (lane < p.num_init) {
+            if (lane <= nk) result = lane;
+          } else if (lane < forced) {
+            if (lane <= nk) result = nk - (lane - p.num_init);
+          }
+          const int from_list = __shfl(win, max(lane - forced, 0));
+          if (lane >= forced && lane < nsel) result = from_list;
+          if (lane < p.top_n) p.topk[(int64_t)kh * p.tk_sh + tok * p.tk_st + lane] = result;
+        } else {  // next segment: its first block keeps what this segment's last tile already added to it
+          for (int jj = lane; jj < W; jj += 64) row[jj] = jj == 0 ? carry : 0.f;
+        }
+      }
+      j0 += seg;
+      __syncthreads();
+    }
   }
   __syncthreads();
+  if (seg > 0) {
+    // a workgroup without any visible compressed key: forced blocks only
+    if (ntiles == 0)
+      for (int tk = wave; tk < TWG; tk += 4) {
+        const int n = n0 + tk;
+        if (n >= xl) break;
+        const int nk = (n + qoff) / Bs;
+        int result = p.ignore_index;
+        if (lane < p.num_init) {
+          if (lane <= nk) result = lane;
+        } else if (lane < p.num_init + p.num_local) {
+          if (lane <= nk) result = nk - (lane - p.num_init);
+        }
+        const int64_t tok = x0 + n;
+        if (lane < p.top_n) p.topk[(int64_t)kh * p.tk_sh + tok * p.tk_st + lane] = result;
+        if (p.imp_out != nullptr)
+          for (int j = lane; j < p.imp_cols; j += 64) p.imp_out[(int64_t)kh * p.imp_sh + tok * p.imp_st + j] = 0.f;
+      }
+    return;
+  }
 
   // ---- selection: the tokens of the workgroup are dealt to the waves ----
   for (int tk = wave; tk < TWG; tk += 4) {
@@ -339,10 +459,32 @@ __global__ __launch_bounds__(256, 2) void topk_kernel(NsaTopkParams p) {
 }
 
 template <int D, int GP, bool PAGED>
-int launch_topk(const NsaTopkParams& p, int B, int max_q_len, hipStream_t stream) {
+int launch_topk(const NsaTopkParams& p_in, int B, int max_q_len, hipStream_t stream) {
   constexpr int TWG = 2 * (32 / GP);
+  NsaTopkParams p = p_in;
+  const size_t stat = 128 * (D + NSA_LDS_PAD) * 2 + 2 * TWG * 132 * 4;
+  // One pass while the score rows of all blocks leave room for two workgroups per CU; else segments of the largest
+  // whole number of key tiles that does.  NSA_TOPK_SEG_BLOCKS forces a segment length (0 = never segment).
+  const int forced_seg = nsa_tuning_knob("NSA_TOPK_SEG_BLOCKS", -1);
+  const size_t budget = 80 * 1024;
   size_t dyn = (size_t)TWG * p.nb_max * sizeof(float);
-  size_t stat = 128 * (D + NSA_LDS_PAD) * 2 + 2 * TWG * 132 * 4;
+  p.seg_blocks = 0;
+  const int tile_span = p.stride * 128;  // positions covered by a 128-key tile
+  const bool aligned = tile_span % p.block_size == 0 && (p.block_size + p.kernel_size - p.stride) / p.stride <= 8 &&
+                       TWG * ((p.stride * 127 + p.kernel_size - 1) / p.block_size + 1) <= 256;
+  const bool want_seg = forced_seg > 0 || (forced_seg < 0 && dyn + stat > budget);
+  if (want_seg && aligned) {
+    const int bpt = tile_span / p.block_size;  // selection blocks per key tile
+    const int ncand = p.top_n - p.num_init - p.num_local > 0 ? p.top_n - p.num_init - p.num_local : 0;
+    const size_t fixed = stat + (size_t)TWG * ncand * 8 + (size_t)TWG * 4;
+    int seg = forced_seg > 0 ? forced_seg : (fixed < budget ? (int)((budget - fixed) / (TWG * 4)) : bpt);
+    seg = seg / bpt * bpt;
+    if (seg < bpt) seg = bpt;
+    if (seg < p.nb_max) {
+      p.seg_blocks = seg;
+      dyn = (size_t)TWG * (seg + 1) * sizeof(float) + (size_t)TWG * ncand * 8;
+    }
+  }
   if (dyn + stat > 160 * 1024) {
     nsa_set_error("top-k: %d selection blocks x %d tokens per workgroup do not fit LDS", p.nb_max, TWG);
     return NSA_ERR_UNSUPPORTED;

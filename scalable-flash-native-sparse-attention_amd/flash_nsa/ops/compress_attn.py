@@ -25,14 +25,15 @@ def cmp_attn_fwd(q, k, v, sm_scale=None, helper=NSAHelper):
 
 
 def cmp_attn_bwd(q, k, v, o, lse, do, dq=None, dkdv_repeat=False, sm_scale=None, helper=NSAHelper, delta=None,
-                 q_chunk_tokens=2048, finalize_dq=False, parts="both"):
+                 q_chunk_tokens=0, finalize_dq=False, parts="both"):
     """Backward of compressed attention.  Returns (dq, dk, dv).
     dq: fresh bf16 tensor, or the caller's fp32 buffer, which is added into; with finalize_dq the fp32 buffer is
     only read and the returned dq is a fresh tensor in q's dtype holding buffer + this branch.
     parts = "dq" / "dkdv" launches only that kernel (the other results are None).
     dk, dv: fp32 [y_len,KH,*] accumulated with atomics over the q-heads of a group and over query chunks
     (non-deterministic summation order, as upstream's dkdv_repeat=False path); `dkdv_repeat` is accepted for call
-    compatibility and ignored.  delta may be passed when already known (delta[T,QH] fp32 = rowsum(o*do))."""
+    compatibility and ignored.  delta may be passed when already known (delta[T,QH] fp32 = rowsum(o*do)).
+    q_chunk_tokens: queries per work item of the dk/dv kernel (0: chosen by the library from the sizes)."""
     check_thd(do, "do")
     T, QH, D = q.shape
     Y, KH, VD = v.shape

@@ -45,13 +45,15 @@ def slc_topk_indices(q, k, lse, sm_scale=None, return_slc_prob=False, align=True
 
 
 @torch.no_grad()
-def get_bind_from_find(topk, helper=NSAHelper, chunk_tokens=1024):
+def get_bind_from_find(topk, helper=NSAHelper, chunk_tokens=None):
     """Inverse of the selection: for every (kv head, selection block) the ascending list of query tokens that
     selected it.  Returns a dict with the CSR (csr_off [KH,nblk+1], csr_tok [KH*T*top_n]), the work-item prefix
     (item_off [KH,nblk+1]) and the static bound on the number of work items per kv head."""
     KH, T, N = topk.shape
     dev = topk.device
     nblk = helper.k_len
+    if chunk_tokens is None:
+        chunk_tokens = _lib.value("nsa_slc_bwd_chunk_tokens", T, KH, N)
     csr_off = torch.empty(KH, nblk + 1, device=dev, dtype=torch.int32)
     item_off = torch.empty(KH, nblk + 1, device=dev, dtype=torch.int32)
     csr_tok = torch.empty(KH * T * N, device=dev, dtype=torch.int32)

@@ -115,6 +115,49 @@ def test_topk_and_slc_fwd(device, lens, QH, KH, D):
     setup_helper(cu.to(device))
 
 
+@pytest.mark.parametrize("lens,QH,KH,D", [([9000, 2500, 700], 32, 2, 128), ([6000, 100], 4, 4, 64),
+                                          ([5000, 3000], 4, 2, 128), ([4500], 64, 1, 64)])
+def test_topk_segmented_selection_equals_one_pass(device, lens, QH, KH, D):
+    """Long contexts keep the block scores of one segment of blocks in LDS and merge every finished segment into a
+    running list of winners.  The segment length (an integer tuning variable read at every launch) must not change
+    the result: indices and returned scores are bit-identical to the one-pass selector, and match the oracle."""
+    import os
+    from flash_nsa.ops.compress_kv import mean_pooling_fwd
+    from flash_nsa.ops.compress_attn import cmp_attn_fwd
+    from flash_nsa.ops.topk import slc_topk_indices
+    cu = make_cu(lens)
+    T = int(cu[-1])
+    q, k, _, _ = make_qkvw(T, QH, KH, D, seed=33)
+    setup_helper(cu.to(device))
+    qd, kd = q.to(device), k.to(device)
+    ck = mean_pooling_fwd(kd)
+    _, lse = cmp_attn_fwd(qd, ck, ck)
+    G = QH // KH
+    results = {}
+    try:
+        for seg in (0, 32, 64, 96):
+            if seg == 0 and G <= 2:
+                continue  # the score rows of 64 / 32 tokens per workgroup do not fit in one pass at this length
+            os.environ["NSA_TOPK_SEG_BLOCKS"] = str(seg)
+            results[seg] = slc_topk_indices(qd, ck, lse, return_slc_prob=True)
+    finally:
+        os.environ.pop("NSA_TOPK_SEG_BLOCKS", None)
+    results["auto"] = slc_topk_indices(qd, ck, lse, return_slc_prob=True)
+    keys = list(results)
+    for key in keys[1:]:
+        assert torch.equal(results[key][0], results[keys[0]][0]), f"indices differ: segment {key} vs {keys[0]}"
+        assert torch.equal(results[key][1], results[keys[0]][1]), f"scores differ: segment {key} vs {keys[0]}"
+    topk, probs = results["auto"]
+    cfg = O.OracleConfig()
+    rt, imps = O.slc_topk(q.float(), ck.float().cpu(), None, cu, cfg, return_importance=True)
+    n_rows, n_diff, n_bad = O.topk_mismatch_report(topk.cpu(), rt, imps, cu, 64, 16, tie_tol=1e-3)
+    assert n_bad == 0, f"{n_bad} rows differ beyond score ties ({n_diff} differing of {n_rows})"
+    assert n_diff <= max(1, n_rows // 200)
+    for b in range(len(lens)):
+        a, e = int(cu[b]), int(cu[b + 1])
+        assert_close(probs[:, a:e, :imps[b].shape[-1]], imps[b], "block scores", atol=2e-3, rtol=2e-3)
+
+
 def test_combine_fwd(device):
     from flash_nsa.ops.combine import combine_fwd
     a, b, c = [randn_bf16(300, 8, 128, seed=s) for s in (1, 2, 3)]
