@@ -47,6 +47,65 @@ def build_case(dev, B=64, QH=64, KH=4, D=128, page=256, lo=4096, hi=32768, seed=
                 slots=torch.tensor(slots, dtype=torch.int32, device=dev), lens=lens, ys=ys, page=page)
 
 
+# Decode attention of one layer with a 4 GiB KV pool, batch = 4 GiB / (S * 4 kv heads * 2 (K,V) * 2 bytes * 128), every
+# request at context S, graph replay: microseconds the reference reports on one H800 (upstream README.md:291-300)
+REFERENCE_H800_DECODE_US = {4096: 689, 8192: 421, 16384: 279, 32768: 206, 65536: 172, 131072: 160}
+
+
+def pool_all_rows(c, dev):
+    """Pools every compressed row of the cached contexts of a build_case() dict (what earlier steps left behind)."""
+    from flash_nsa.inference import mean_pooling_prefill
+    B, page = len(c["lens"]), c["page"]
+    ycu = torch.zeros(B + 1, dtype=torch.int32)
+    ycu[1:] = torch.cumsum(torch.tensor(c["ys"]), 0)
+    slots = torch.cat([(c["cbt"][b].cpu()[torch.arange(y) // page].to(torch.int64) * page + torch.arange(y) % page)
+                       for b, y in enumerate(c["ys"])]).to(torch.int32).to(dev)
+    for cache in (c["k"], c["v"]):
+        mean_pooling_prefill(cache, ycu.to(dev), max(c["ys"]), c["bt"], slots)
+
+
+def decode_sweep(dev, lengths=(4096, 8192, 16384, 32768, 65536, 131072), reps=100):
+    """The reference's decode table: fixed 4 GiB KV pool, so the batch shrinks as the context grows (512 requests of
+    4K tokens ... 16 requests of 128K tokens).  nsa_decode picks its path itself: one launch per step while the
+    batch fills the GPU, the compressed branch cut into parts (two launches) for small batches of long contexts.
+    Prints one JSON line per context length."""
+    import json
+    from flash_nsa import nsa_decode
+    from flash_nsa.inference import auto_cmp_splits
+    for S in lengths:
+        B = (4 << 30) // (S * 4 * 2 * 2 * 128)
+        c = build_case(dev, B=B, lo=S, hi=S, seed=5)
+        pool_all_rows(c, dev)
+        args = (c["q"], c["k"], c["v"], c["w"], c["ctx"], c["bt"], c["slots"], c["cbt"])
+        kw = dict(fixed_y_maxlen=max(2048, (S // 16 + 255) // 256 * 256), fixed_num_slc_blocks=max(512, S // 64))
+        nsa_decode(*args, **kw)
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            nsa_decode(*args, **kw)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            nsa_decode(*args, **kw)
+        for _ in range(10):
+            graph.replay()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(reps):
+            graph.replay()
+        e.record()
+        torch.cuda.synchronize()
+        us = s.elapsed_time(e) * 1e3 / reps
+        nbytes = algorithmic_bytes(c["lens"])
+        print(json.dumps({"context": S, "batch": B, "us_per_step": round(us, 1),
+                          "cmp_parts": auto_cmp_splits(B, 4, kw["fixed_y_maxlen"]),
+                          "algorithmic_gbs": round(nbytes / us / 1e3, 1),
+                          "reference_h800_us": REFERENCE_H800_DECODE_US.get(S)}), flush=True)
+        del c, args, graph
+
+
 def algorithmic_bytes(lens, KH=4, D=128, VD=128, QH=64, top_n=16, block=64, window=512):
     tot = 0
     for L in lens:
@@ -195,3 +254,20 @@ if __name__ == "__main__":
     sys.path.insert(0, os.path.join(root, "scalable-flash-native-sparse-attention_amd"))
     print(json.dumps({"decode": decode_bench(torch.device("cuda:0")),
                       "cache_writer": cache_writer_bench(torch.device("cuda:0"))}))
+
+
+if __name__ == "__main__":
+    import argparse
+    import json
+    import os
+    import sys
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)),
+                                    "scalable-flash-native-sparse-attention_amd"))
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--sweep", action="store_true", help="context-length sweep with a fixed 4 GiB KV pool")
+    a = ap.parse_args()
+    device = torch.device("cuda:0")
+    if a.sweep:
+        decode_sweep(device)
+    else:
+        print(json.dumps(decode_bench(device)))

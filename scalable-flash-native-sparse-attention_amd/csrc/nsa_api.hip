@@ -540,6 +540,65 @@ int nsa_decode_cmp_split(const void* q, int64_t q_st, int64_t q_sh, const void* 
   return nsa_decode_cmp_split_launch(p, B, nsplit, D, VD, (hipStream_t)stream);
 }
 
+static void fill_decode_split(NsaDecodeParams& p, int fixed_y_maxlen, int fixed_num_slc_blocks, int table_stride) {
+  p.y_cap = fixed_y_maxlen; p.nb_cap = fixed_num_slc_blocks; p.table_stride = table_stride;
+}
+
+int nsa_decode_split_fits(int D, int VD, int fixed_y_maxlen, int fixed_num_slc_blocks, int table_stride) {
+  NsaDecodeParams p{};
+  fill_decode_split(p, fixed_y_maxlen, fixed_num_slc_blocks, table_stride);
+  return nsa_decode_split_lds_bytes(p, D, VD) > 0 ? 1 : 0;
+}
+
+int nsa_decode_split(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr, int64_t k_sh,
+                     const void* v_cache, int64_t v_sr, int64_t v_sh, const void* w, int64_t w_st, int64_t w_sh,
+                     void* out, int64_t o_st, int64_t o_sh, void* cmp_o, void* slc_o, void* swa_o, int64_t co_st,
+                     int64_t co_sh, float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk, int64_t tk_sh,
+                     int64_t tk_st, float* sp_m, float* sp_l, float* sp_o, void* sp_keep_p, float* sp_keep_m,
+                     int nsplit, const int32_t* context_lens, const int32_t* block_tables, int table_stride,
+                     const int32_t* cmp_block_tables, int cmp_table_stride, int page_size, int B, int QH, int KH,
+                     int D, int VD, int fixed_y_maxlen, int fixed_num_slc_blocks, int kernel_size, int stride,
+                     int block_size, int top_n, int num_init, int num_local, int ignore_index, int window,
+                     float sm_scale, void* stream) {
+  int rc = check_heads("decode_split", QH, KH, D, VD);
+  if (rc) return rc;
+  rc = check_nsa_sizes("decode_split", kernel_size, stride, block_size);
+  if (rc) return rc;
+  rc = check_page("decode_split", page_size);
+  if (rc) return rc;
+  NSA_REQUIRE(QH / KH <= 16, NSA_ERR_UNSUPPORTED, "decode_split: at most 16 q-heads per kv head (got %d)", QH / KH);
+  NSA_REQUIRE(nsplit >= 1 && nsplit <= 64, NSA_ERR_BAD_ARG, "decode_split: nsplit %d must be in [1,64]", nsplit);
+  NSA_REQUIRE(block_size % 32 == 0, NSA_ERR_UNSUPPORTED, "decode_split: block_size %d must be a multiple of 32",
+              block_size);
+  NSA_REQUIRE(top_n >= 1 && top_n <= 64 && num_init >= 0 && num_local >= 0 && num_init + num_local <= top_n,
+              NSA_ERR_BAD_ARG, "decode_split: bad top_n %d / num_init %d / num_local %d", top_n, num_init, num_local);
+  NSA_REQUIRE(fixed_y_maxlen >= 1 && fixed_num_slc_blocks >= 1, NSA_ERR_BAD_ARG,
+              "decode_split: fixed_y_maxlen %d and fixed_num_slc_blocks %d must be positive", fixed_y_maxlen,
+              fixed_num_slc_blocks);
+  NSA_REQUIRE(out && w && sp_m && sp_l && sp_o && sp_keep_p && sp_keep_m, NSA_ERR_BAD_ARG,
+              "decode_split: out, w and the five scratch buffers are required");
+  NsaDecodeParams p{};
+  p.q = (const bf16_t*)q; p.q_st = q_st; p.q_sh = q_sh;
+  p.k = (const bf16_t*)k_cache; p.k_sr = k_sr; p.k_sh = k_sh;
+  p.v = (const bf16_t*)v_cache; p.v_sr = v_sr; p.v_sh = v_sh;
+  p.w = (const bf16_t*)w; p.w_st = w_st; p.w_sh = w_sh;
+  p.out = (bf16_t*)out; p.o_st = o_st; p.o_sh = o_sh;
+  p.cmp_o = (bf16_t*)cmp_o; p.slc_o = (bf16_t*)slc_o; p.swa_o = (bf16_t*)swa_o; p.co_st = co_st; p.co_sh = co_sh;
+  p.lse_out = lse; p.lse_st = lse_st; p.lse_sh = lse_sh;
+  p.topk = topk; p.tk_sh = tk_sh; p.tk_st = tk_st;
+  p.sp_m = sp_m; p.sp_l = sp_l; p.sp_o = sp_o;
+  p.sp_keep_p = (_Float16*)sp_keep_p; p.sp_keep_m = sp_keep_m; p.nsplit = nsplit;
+  p.ctx_lens = context_lens;
+  p.table = block_tables;
+  p.cmp_table = cmp_block_tables; p.cmp_table_stride = cmp_table_stride; p.page_size = page_size;
+  p.G = QH / KH; p.KH = KH;
+  p.scale_log2 = sm_scale * NSA_LOG2E;
+  p.kernel_size = kernel_size; p.stride = stride; p.block_size = block_size; p.window = window; p.top_n = top_n;
+  p.num_init = num_init; p.num_local = num_local; p.ignore_index = ignore_index;
+  fill_decode_split(p, fixed_y_maxlen, fixed_num_slc_blocks, table_stride);
+  return nsa_decode_split_launch(p, B, D, VD, (hipStream_t)stream);
+}
+
 int nsa_decode_slc_swa_combine(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr,
                                int64_t k_sh, const void* v_cache, int64_t v_sr, int64_t v_sh, const void* w,
                                int64_t w_st, int64_t w_sh, int32_t* topk, int64_t tk_sh, int64_t tk_st,

@@ -130,9 +130,15 @@ struct NsaDecodeParams {
   int y_cap, nb_cap;                            // fixed_y_maxlen, fixed_num_slc_blocks
   // split compressed branch: fp32 scratch [B,KH,nsplit,16] (m, l), [B,KH,nsplit,16,VD] (o), pg [B,KH,y_cap]
   float* sp_m; float* sp_l; float* sp_o; float* pg;
+  // two-launch split path: the partial kernel also spills, per (request, kv head), the un-normalised fp16
+  // probabilities [16][ceil32(y_cap)] and the maxima they refer to [ceil32(y_cap)/32][16]; the final kernel merges
+  // the nsplit parts, folds the probabilities into block scores and selects
+  _Float16* sp_keep_p; float* sp_keep_m; int nsplit;
 };
 int nsa_decode_cmp_topk_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream);
 int nsa_decode_slc_swa_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream);
 int nsa_decode_fused_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream);
 int nsa_decode_fused_lds_bytes(const NsaDecodeParams& p, int D, int VD);  // 0: does not fit
 int nsa_decode_cmp_split_launch(const NsaDecodeParams& p, int B, int nsplit, int D, int VD, hipStream_t stream);
+int nsa_decode_split_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream);
+int nsa_decode_split_lds_bytes(const NsaDecodeParams& p, int D, int VD);  // final kernel; 0: does not fit

@@ -106,48 +106,45 @@ NSA_DEVICE float wave_sum(float v) {
 }
 
 // ---- wave-wide arg-max over (score, index) pairs with "lowest index wins ties", on the DPP crossbar (no LDS
-// traffic, a few cycles per step).  Scores must be >= -1 and finite; they are compared through their bit patterns
-// after a monotone remap, packed with the inverted index into one 64-bit key.  Returns the winning index in every
-// lane (0x7fffffff if no lane had a candidate).
+// traffic).  Scores must be finite.  A 32-bit float maximum is reduced first; the lanes that hold it are found with
+// one ballot, and only when several lanes tie is a second reduction (minimum index) needed.  Returns the winning
+// index in every lane (0x7fffffff if no lane had a candidate) and, on request, the winning score.
 template <int CTRL, int ROW_MASK>
-NSA_DEVICE uint64_t dpp_max_step(uint64_t key) {
-  uint32_t lo = (uint32_t)key, hi = (uint32_t)(key >> 32);
-  uint32_t lo2 = __builtin_amdgcn_update_dpp(lo, lo, CTRL, ROW_MASK, 0xf, false);
-  uint32_t hi2 = __builtin_amdgcn_update_dpp(hi, hi, CTRL, ROW_MASK, 0xf, false);
-  uint64_t other = ((uint64_t)hi2 << 32) | lo2;
-  return other > key ? other : key;
+NSA_DEVICE float dpp_fmax_step(float x) {
+  const int xi = __builtin_bit_cast(int, x);
+  return fmaxf(x, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(xi, xi, CTRL, ROW_MASK, 0xf, false)));
+}
+template <int CTRL, int ROW_MASK>
+NSA_DEVICE int dpp_imin_step(int x) {
+  return min(x, __builtin_amdgcn_update_dpp(x, x, CTRL, ROW_MASK, 0xf, false));
+}
+NSA_DEVICE int wave_argmax_lowest_score(float score, int index, bool has_candidate, float& win_score) {
+  float s = has_candidate ? score : -__builtin_inff();
+  float m = s;
+  m = dpp_fmax_step<0x111, 0xf>(m);  // row_shr:1
+  m = dpp_fmax_step<0x112, 0xf>(m);  // row_shr:2
+  m = dpp_fmax_step<0x114, 0xf>(m);  // row_shr:4
+  m = dpp_fmax_step<0x118, 0xf>(m);  // row_shr:8   -> lane 15 of every row holds the row maximum
+  m = dpp_fmax_step<0x142, 0xa>(m);  // row_bcast:15 into rows 1 and 3
+  m = dpp_fmax_step<0x143, 0xc>(m);  // row_bcast:31 into rows 2 and 3 -> lane 63 holds the wave maximum
+  m = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, m), 63));
+  win_score = m;
+  const uint64_t tied = __builtin_amdgcn_ballot_w64(has_candidate && s == m);
+  if (tied == 0) return 0x7fffffff;
+  if ((tied & (tied - 1)) == 0)  // one lane holds the maximum
+    return __builtin_amdgcn_readlane(index, (int)__builtin_ctzll(tied));
+  int i = (has_candidate && s == m) ? index : 0x7fffffff;
+  i = dpp_imin_step<0x111, 0xf>(i);
+  i = dpp_imin_step<0x112, 0xf>(i);
+  i = dpp_imin_step<0x114, 0xf>(i);
+  i = dpp_imin_step<0x118, 0xf>(i);
+  i = dpp_imin_step<0x142, 0xa>(i);
+  i = dpp_imin_step<0x143, 0xc>(i);
+  return __builtin_amdgcn_readlane(i, 63);
 }
 NSA_DEVICE int wave_argmax_lowest(float score, int index, bool has_candidate) {
-  // monotone map of a float to unsigned: flip all bits of negatives, the sign bit of non-negatives
-  uint32_t b = __builtin_bit_cast(uint32_t, score);
-  b = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
-  uint64_t key = has_candidate ? (((uint64_t)b << 32) | (uint32_t)(0x7fffffff - index)) : 0ull;
-  key = dpp_max_step<0x111, 0xf>(key);  // row_shr:1
-  key = dpp_max_step<0x112, 0xf>(key);  // row_shr:2
-  key = dpp_max_step<0x114, 0xf>(key);  // row_shr:4
-  key = dpp_max_step<0x118, 0xf>(key);  // row_shr:8   -> lane 15 of every row holds the row maximum
-  key = dpp_max_step<0x142, 0xa>(key);  // row_bcast:15 into rows 1 and 3
-  key = dpp_max_step<0x143, 0xc>(key);  // row_bcast:31 into rows 2 and 3 -> lane 63 holds the wave maximum
-  uint32_t lo = __builtin_amdgcn_readlane((uint32_t)key, 63);
-  uint32_t hi = __builtin_amdgcn_readlane((uint32_t)(key >> 32), 63);
-  return hi == 0 ? 0x7fffffff : (int)(0x7fffffff - lo);
-}
-
-// Same reduction, also returning the winner's score (undefined when there is no candidate).
-NSA_DEVICE int wave_argmax_lowest_score(float score, int index, bool has_candidate, float& win_score) {
-  uint32_t b = __builtin_bit_cast(uint32_t, score);
-  b = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
-  uint64_t key = has_candidate ? (((uint64_t)b << 32) | (uint32_t)(0x7fffffff - index)) : 0ull;
-  key = dpp_max_step<0x111, 0xf>(key);
-  key = dpp_max_step<0x112, 0xf>(key);
-  key = dpp_max_step<0x114, 0xf>(key);
-  key = dpp_max_step<0x118, 0xf>(key);
-  key = dpp_max_step<0x142, 0xa>(key);
-  key = dpp_max_step<0x143, 0xc>(key);
-  uint32_t lo = __builtin_amdgcn_readlane((uint32_t)key, 63);
-  uint32_t hi = __builtin_amdgcn_readlane((uint32_t)(key >> 32), 63);
-  win_score = __builtin_bit_cast(float, (hi & 0x80000000u) ? (hi & 0x7fffffffu) : ~hi);
-  return hi == 0 ? 0x7fffffff : (int)(0x7fffffff - lo);
+  float unused;
+  return wave_argmax_lowest_score(score, index, has_candidate, unused);
 }
 
 __host__ __device__ inline int cdiv_i(int a, int b) { return (a + b - 1) / b; }

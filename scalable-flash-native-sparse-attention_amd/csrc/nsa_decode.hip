@@ -13,6 +13,7 @@
 // pool through the block tables.
 #include "nsa_common.h"
 #include "nsa_api_internal.h"
+#include <type_traits>
 
 namespace {
 
@@ -39,7 +40,7 @@ struct UnitFlash {
   float sc;
   int l16, kq, lane;
   bf16_t* Ss;          // wave-private staging slot
-  _Float16* keep_p;    // [16][keep_ld] or null
+  _Float16* keep_p;    // [16][keep_ld] (keep_ld > 0), [units][16][UK] (keep_ld == 0: whole units contiguous), or null
   float* keep_m;       // [units][16]
   int keep_ld;
 
@@ -149,7 +150,9 @@ struct UnitFlash {
 #pragma unroll
       for (int jt = 0; jt < 2; jt++) {
         h4 hv = {(_Float16)sacc[jt][0], (_Float16)sacc[jt][1], (_Float16)sacc[jt][2], (_Float16)sacc[jt][3]};
-        *reinterpret_cast<h4*>(&keep_p[l16 * keep_ld + key0 + jt * 16 + kq * 4]) = hv;
+        const int at = keep_ld > 0 ? l16 * keep_ld + key0 + jt * 16 + kq * 4
+                                   : (key0 / UK) * (16 * UK) + l16 * UK + jt * 16 + kq * 4;
+        *reinterpret_cast<h4*>(&keep_p[at]) = hv;
       }
       if (kq == 0) keep_m[(key0 / UK) * 16 + l16] = m_safe;
     }
@@ -207,42 +210,56 @@ struct UnitFlash {
   }
 };
 
-// merged value of one (head, channel) from n wave partials; returns o (normalised) and optionally lse2
-NSA_DEVICE float merge_partials(const float* pm, const float* pl, const float* po, int nparts, int part_stride_ml,
-                                int part_stride_o, int head, int d, int VD, float sc, float* lse2_out) {
+// Merge of n wave partials (m in raw score units, l, un-normalised o) in two steps, so that the exponentials are
+// evaluated once per (part, head) and not once per output channel:
+//   merge_weights: one thread per head turns the l of every part into its normalised weight
+//                  exp2((m_part - m) * c) / l_total, in place, and returns lse2 (0 when nothing was visible);
+//   merge_value:   after a barrier, o[head][d] = sum over parts of weight * o_part.
+NSA_DEVICE float merge_weights(const float* pm, float* pl, int nparts, int part_stride_ml, int head, float sc) {
   float m = NSA_NEG_INF;
   for (int w = 0; w < nparts; w++) m = fmaxf(m, pm[w * part_stride_ml + head]);
   if (m == NSA_NEG_INF) {
-    if (lse2_out) *lse2_out = 0.f;
+    for (int w = 0; w < nparts; w++) pl[w * part_stride_ml + head] = 0.f;
     return 0.f;
   }
-  float l = 0.f, o = 0.f;
+  float l = 0.f;
   for (int w = 0; w < nparts; w++) {
-    float mw = pm[w * part_stride_ml + head];
-    float a = (mw == NSA_NEG_INF) ? 0.f : fast_exp2((mw - m) * sc);
+    const float mw = pm[w * part_stride_ml + head];
+    const float a = (mw == NSA_NEG_INF) ? 0.f : fast_exp2((mw - m) * sc);
     l += a * pl[w * part_stride_ml + head];
-    o += a * po[w * part_stride_o + head * VD + d];
+    pl[w * part_stride_ml + head] = a;
   }
-  if (lse2_out) *lse2_out = m * sc + fast_log2(l);
-  return l > 0.f ? o / l : 0.f;
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  for (int w = 0; w < nparts; w++) pl[w * part_stride_ml + head] *= inv;
+  return l > 0.f ? m * sc + fast_log2(l) : 0.f;
+}
+NSA_DEVICE float merge_value(const float* wgt, const float* po, int nparts, int part_stride_ml, int part_stride_o,
+                             int head, int d, int VD) {
+  float o = 0.f;
+  for (int w = 0; w < nparts; w++) o += wgt[w * part_stride_ml + head] * po[w * part_stride_o + head * VD + d];
+  return o;
 }
 
 // head-summed probabilities of the compressed keys -> scores of the selection blocks (ascending key order per
 // block); all threads of the workgroup
 NSA_DEVICE void fold_block_scores(const float* pg, float* imp, int y, int nb, int nb_cap, const NsaDecodeParams& p,
                                   int tid, int nthreads) {
+  // stride is a power of two and divides kernel_size and block_size: block j covers the compressed keys
+  // j*Bs/St - Kz/St + 1 + r, r = 0 .. (Bs+Kz-St)/St - 1, with overlap area (in positions) / St as the weight
   const int Bs = p.block_size, Kz = p.kernel_size, St = p.stride;
-  const int nloops = (Bs + Kz - St) / St;
+  const int bps = Bs / St, kps = Kz / St;
+  const int nloops = bps + kps - 1;
+  const float inv_st = 1.f / (float)St;
   for (int j = tid; j < nb_cap; j += nthreads) {
     float acc = 0.f;
     if (j < nb) {
-      int i0 = (j * Bs - Kz) / St + 1;
+      const int i0 = j * bps - kps + 1;
       int cs = St - Kz;
       for (int r = 0; r < nloops; r++, cs += St) {
-        int i = i0 + r;
+        const int i = i0 + r;
         if (i >= 0 && i < y) {
-          int area = min(cs + Kz, Bs) - max(cs, 0);
-          acc += pg[i] * ((float)area / (float)St);
+          const int area = min(cs + Kz, Bs) - max(cs, 0);
+          acc += pg[i] * ((float)area * inv_st);
         }
       }
     }
@@ -251,8 +268,82 @@ NSA_DEVICE void fold_block_scores(const float* pg, float* imp, int y, int nb, in
 }
 
 // one wave: forced initial and local blocks, then repeated arg-max over imp[0 .. min(t/block, nb_cap-1)] (lowest
-// index on ties; taken scores are overwritten with -1).  Returns the block of slot `lane`.
-NSA_DEVICE int select_blocks_wave(float* imp, int t, int nb_cap, const NsaDecodeParams& p, int lane) {
+// index on ties).  Returns the block of slot `lane`.
+// The candidates of a lane (blocks lane, lane+64, ...) are read once into NV registers; after every round only the
+// winner's lane rescans its registers, so a round costs one wave reduction instead of a dependent chain of LDS reads.
+template <int NV>
+NSA_DEVICE int select_blocks_regs(const float* imp, int t, int nb_cap, const NsaDecodeParams& p, int lane) {
+  static_assert(NV % 8 == 0, "candidates per lane come in groups of 8");
+  constexpr int NG = NV / 8;
+  const int nk = t >= 0 ? t / p.block_size : -1;
+  int result = p.ignore_index;
+  if (lane < p.num_init) {
+    if (lane <= nk) result = lane;
+  } else if (lane < p.num_init + p.num_local) {
+    if (lane <= nk) result = nk - (lane - p.num_init);
+  }
+  const int nsel = min(p.top_n, nk + 1);
+  const int jmax = min(nk, nb_cap - 1);
+  float v[NV];
+#pragma unroll
+  for (int k = 0; k < NV; k++) {
+    const int j = lane + 64 * k;
+    float x = j <= jmax ? imp[min(j, nb_cap - 1)] : -3.f;
+    if (j <= jmax && (j < p.num_init || j > nk - p.num_local)) x = -1.f;  // forced blocks: behind every real score
+    v[k] = x;
+  }
+  // best candidate of every group of 8 registers; a round only rescans the group the winner came from (the group
+  // number is wave-uniform, so that is one uniform branch)
+  float gbest[NG];
+  int gidx[NG];
+  auto rescan = [&](auto g_tag) {
+    constexpr int g = decltype(g_tag)::value;
+    float bs = -2.f;
+    int bi = 0x7fffffff;
+#pragma unroll
+    for (int k = g * 8; k < g * 8 + 8; k++)
+      if (v[k] > bs) { bs = v[k]; bi = lane + 64 * k; }
+    gbest[g] = bs;
+    gidx[g] = bi;
+  };
+  auto for_group = [&](int g, auto&& fn) {
+    if constexpr (NG == 1) { fn(std::integral_constant<int, 0>{}); }
+    else if constexpr (NG == 2) { if (g == 0) fn(std::integral_constant<int, 0>{}); else fn(std::integral_constant<int, 1>{}); }
+    else {
+      static_assert(NG == 4, "8, 16 or 32 candidates per lane");
+      if (g == 0) fn(std::integral_constant<int, 0>{});
+      else if (g == 1) fn(std::integral_constant<int, 1>{});
+      else if (g == 2) fn(std::integral_constant<int, 2>{});
+      else fn(std::integral_constant<int, 3>{});
+    }
+  };
+#pragma unroll
+  for (int g = 0; g < NG; g++) for_group(g, rescan);
+  for (int slot = p.num_init + p.num_local; slot < nsel; slot++) {
+    float best = -2.f;
+    int bj = 0x7fffffff;
+#pragma unroll
+    for (int g = 0; g < NG; g++)
+      if (gbest[g] > best) { best = gbest[g]; bj = gidx[g]; }
+    const int w = wave_argmax_lowest(best, bj, bj != 0x7fffffff);
+    if (lane == slot) result = w;
+    if (w > jmax) continue;  // wave-uniform: no candidate left
+    const bool mine = (w & 63) == lane;
+    const int kk = w >> 6;
+    for_group(kk >> 3, [&](auto g_tag) {  // take the winner out of its group, then rescan that group only
+      constexpr int g = decltype(g_tag)::value;
+#pragma unroll
+      for (int k = g * 8; k < g * 8 + 8; k++)
+        if (mine && k == kk) v[k] = -1.f;
+      rescan(g_tag);
+    });
+  }
+  return result;
+}
+
+// more than 2048 blocks: the same selection with the scores rescanned in LDS every round (taken scores are
+// overwritten with -1)
+NSA_DEVICE int select_blocks_lds(float* imp, int t, int nb_cap, const NsaDecodeParams& p, int lane) {
   const int nk = t >= 0 ? t / p.block_size : -1;
   int result = p.ignore_index;
   if (lane == 0) {
@@ -286,6 +377,13 @@ NSA_DEVICE int select_blocks_wave(float* imp, int t, int nb_cap, const NsaDecode
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
   return result;
+}
+
+NSA_DEVICE int select_blocks_wave(float* imp, int t, int nb_cap, const NsaDecodeParams& p, int lane) {
+  if (nb_cap <= 512) return select_blocks_regs<8>(imp, t, nb_cap, p, lane);
+  if (nb_cap <= 1024) return select_blocks_regs<16>(imp, t, nb_cap, p, lane);
+  if (nb_cap <= 2048) return select_blocks_regs<32>(imp, t, nb_cap, p, lane);
+  return select_blocks_lds(imp, t, nb_cap, p, lane);
 }
 
 template <int D, int VD, bool KEEP>
@@ -346,20 +444,16 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_cmp_topk_kernel(NsaDeco
   uf.run(wave, NW, nu, 0, y - 1, [&](int u) { return u * UK; }, tab_s, page, kbase, p.k_sr, vbase, p.v_sr);
   uf.publish(part_m + wave * 16, part_l + wave * 16, reinterpret_cast<float*>(Vs_all + wave * SLOT));
   __syncthreads();
-  for (int idx = tid; idx < 16 * VD; idx += NW * 64) {
+  if (tid < 16) {
+    const float lse2 = merge_weights(part_m, part_l, NW, 16, tid, p.scale_log2);
+    lse_s[tid] = tid < G ? lse2 : 0.f;
+    if (tid < G && p.lse_out) p.lse_out[(int64_t)b * p.lse_st + (kh * G + tid) * p.lse_sh] = lse2;
+  }
+  __syncthreads();
+  for (int idx = tid; idx < G * VD; idx += NW * 64) {
     int h = idx / VD, d = idx - h * VD;
-    float lse2;
-    float o = merge_partials(part_m, part_l, reinterpret_cast<const float*>(Vs_all), NW, 16, SLOT / 2, h, d, VD,
-                             p.scale_log2, &lse2);
-    if (h < G) {
-      p.cmp_o[(int64_t)b * p.co_st + (int64_t)(kh * G + h) * p.co_sh + d] = (bf16_t)o;
-      if (d == 0) {
-        lse_s[h] = lse2;
-        if (p.lse_out) p.lse_out[(int64_t)b * p.lse_st + (kh * G + h) * p.lse_sh] = lse2;
-      }
-    } else if (d == 0) {
-      lse_s[h] = 0.f;
-    }
+    float o = merge_value(part_l, reinterpret_cast<const float*>(Vs_all), NW, 16, SLOT / 2, h, d, VD);
+    p.cmp_o[(int64_t)b * p.co_st + (int64_t)(kh * G + h) * p.co_sh + d] = (bf16_t)o;
   }
   __syncthreads();
 
@@ -453,6 +547,12 @@ __global__ __launch_bounds__(SPLIT_WAVES * 64) void decode_cmp_partial_kernel(Ns
 
   UF uf;
   uf.init(p.q + (int64_t)b * p.q_st + (int64_t)head * p.q_sh, p.scale_log2, lane, Vs_all + wave * SLOT);
+  if (p.sp_keep_p != nullptr) {  // spill the un-normalised probabilities of every unit for the final kernel
+    const int nuc = (p.y_cap + UK - 1) / UK;
+    uf.keep_ld = 0;  // unit-major: a wave writes the 1 KB of a unit as whole cache lines
+    uf.keep_p = p.sp_keep_p + ((int64_t)b * p.KH + kh) * 16 * nuc * UK;
+    uf.keep_m = p.sp_keep_m + ((int64_t)b * p.KH + kh) * nuc * 16;
+  }
   const int nu = (y + UK - 1) / UK;
   uf.run(sp * NW + wave, NW * nsplit, nu, 0, y - 1, [&](int u) { return u * UK; }, tab_s, page, kbase, p.k_sr,
          vbase, p.v_sr);
@@ -590,7 +690,7 @@ template <int D, int VD>
 __global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecodeParams p) {
   using UF = UnitFlash<D, VD>;
   constexpr int NW = DEC_WAVES;
-  constexpr int NW_SLC = 5;  // waves on the selected blocks, the rest on the window
+  constexpr int NT = NW * 64;
   extern __shared__ __attribute__((aligned(16))) unsigned char dyn_raw[];
   constexpr int SLOT = UF::SLOT;
   static_assert(SLOT * 2 >= 16 * VD * 4, "a wave's slot must hold its partial output");
@@ -609,7 +709,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecod
   const int t = L - 1;
   const int32_t* tab = p.table + (int64_t)b * p.table_stride;
   const int page = p.page_size;
-  for (int i = tid; i < (L + page - 1) / page; i += NW * 64) tab_s[i] = tab[i];
+  for (int i = tid; i < (L + page - 1) / page; i += NT) tab_s[i] = tab[i];
   const bf16_t* kbase = p.k + (int64_t)kh * p.k_sh;
   const bf16_t* vbase = p.v + (int64_t)kh * p.v_sh;
   const int l16 = lane & 15;
@@ -617,54 +717,145 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecod
   const int head = kh * G + g;
   const int Bs = p.block_size;
   const int nvalid = t >= 0 ? min(p.top_n, t / Bs + 1) : 0;
-  if (p.pg != nullptr) {
-    // selection prologue: fold the head-summed probabilities of the compressed keys into block scores (held in the
-    // not-yet-used V staging area), force the initial/local blocks, then repeated arg-max by wave 0
-    float* imp = reinterpret_cast<float*>(Vs_all);
+  const int nb = min(L > 0 ? (L - 1) / Bs + 1 : 0, p.nb_cap);
+  __shared__ float sp_lse_s[16], sp_m_s[16], sp_l_s[16];
+  __shared__ float sp_w_s[64 * 16];  // weights of the parts of the compressed branch (nsplit <= 64)
+  constexpr int OPT = 16 * VD / NT;  // output values per thread
+  static_assert((16 * VD) % NT == 0, "output values must divide over the threads");
+  float ocmp_pre[OPT];               // split path: merged compressed-branch output of this thread's values
+  float* imp = nullptr;              // block scores, when the selection runs here
+  const bool select_here = p.sp_keep_p != nullptr || p.pg != nullptr;
+  if (p.sp_keep_p != nullptr) {
+    // Prologue of the two-launch split path: merge the statistics of the parts of the compressed branch, turn the
+    // spilled fp16 probabilities into head-summed probabilities (over the not-yet-used staging slots) and fold them
+    // into block scores.  The same arithmetic as the one-launch kernel.
+    typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+    const int y = L >= p.kernel_size ? min((L - p.kernel_size) / p.stride + 1, p.y_cap) : 0;
+    const int nuc = (p.y_cap + UK - 1) / UK, keep_ld = nuc * UK;
+    const int nsplit = p.nsplit;
+    float* pgs = reinterpret_cast<float*>(Vs_all);
+    imp = reinterpret_cast<float*>(tab_s + ((p.table_stride + 3) & ~3));
+    float* fac = imp + ((p.nb_cap + 3) & ~3);
+    const int64_t sp_base = ((int64_t)b * p.KH + kh) * nsplit * 16;
+    const _Float16* keep_p = p.sp_keep_p + ((int64_t)b * p.KH + kh) * 16 * keep_ld;
+    const float* keep_m = p.sp_keep_m + ((int64_t)b * p.KH + kh) * nuc * 16;
+    // all (m, l) of the parts in one round trip, then one thread per head
+    float* st_m = fac;
+    float* st_l = fac + 64 * 16;
+    for (int i = tid; i < nsplit * 16; i += NT) { st_m[i] = p.sp_m[sp_base + i]; st_l[i] = p.sp_l[sp_base + i]; }
+    __syncthreads();
+    if (tid < 16) {
+      float m = NSA_NEG_INF;
+      for (int s2 = 0; s2 < nsplit; s2++) m = fmaxf(m, st_m[s2 * 16 + tid]);
+      float l = 0.f;
+      for (int s2 = 0; s2 < nsplit; s2++) {
+        const float ms = st_m[s2 * 16 + tid];
+        const float a = (ms == NSA_NEG_INF) ? 0.f : fast_exp2((ms - m) * p.scale_log2);
+        sp_w_s[s2 * 16 + tid] = a;
+        l += a * st_l[s2 * 16 + tid];
+      }
+      const float inv = l > 0.f ? 1.f / l : 0.f;
+      for (int s2 = 0; s2 < nsplit; s2++) sp_w_s[s2 * 16 + tid] *= inv;
+      const float lse2 = (m != NSA_NEG_INF && l > 0.f) ? m * p.scale_log2 + fast_log2(l) : 0.f;
+      sp_lse_s[tid] = lse2;
+      if (tid < G && p.lse_out) p.lse_out[(int64_t)b * p.lse_st + (kh * G + tid) * p.lse_sh] = lse2;
+    }
+    __syncthreads();
+    // merge of the parts' outputs: independent loads, issued here so that they overlap the rest of the prologue
+#pragma unroll
+    for (int r = 0; r < OPT; r++) {
+      const int idx = tid + r * NT;
+      const int h = idx / VD, d = idx - h * VD;
+      float o = 0.f;
+      for (int s2 = 0; s2 < nsplit; s2++) o += sp_w_s[s2 * 16 + h] * p.sp_o[(sp_base + s2 * 16 + h) * VD + d];
+      ocmp_pre[r] = o;
+    }
+    const int nu = (y + UK - 1) / UK;
+    for (int i = tid; i < nu * 16; i += NT) {
+      const int h = i & 15;
+      fac[i] = h < G ? fast_exp2(__builtin_fmaf(keep_m[i], p.scale_log2, -sp_lse_s[h])) : 0.f;
+    }
+    __syncthreads();
+    for (int k4 = tid * 4; k4 < y; k4 += NT * 4) {
+      const float* f = fac + (k4 / UK) * 16;
+      h4 v[16];
+#pragma unroll
+      for (int h = 0; h < 16; h++)
+        v[h] = *reinterpret_cast<const h4*>(keep_p + (k4 / UK) * (16 * UK) + h * UK + (k4 % UK));
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int h = 0; h < 16; h++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc[e] += (float)v[h][e] * f[h];
+      *reinterpret_cast<f32x4*>(pgs + k4) = acc;
+    }
+    __syncthreads();
+    fold_block_scores(pgs, imp, y, nb, nb, p, tid, NT);
+  } else if (p.pg != nullptr) {
+    // fold the head-summed probabilities of the compressed keys (computed by the importance kernel) into block
+    // scores; they live behind the page table, the staging slots belong to the window waves
+    imp = reinterpret_cast<float*>(tab_s + ((p.table_stride + 3) & ~3));
     const float* pg = p.pg + ((int64_t)b * p.KH + kh) * p.y_cap;
     const int y = L >= p.kernel_size ? min((L - p.kernel_size) / p.stride + 1, p.y_cap) : 0;
-    const int nb = min(L > 0 ? (L - 1) / Bs + 1 : 0, p.nb_cap);
-    fold_block_scores(pg, imp, y, nb, nb, p, tid, NW * 64);
-    __syncthreads();
-    if (wave == 0) {
-      const int result = select_blocks_wave(imp, t, nb, p, lane);
-      blk_s[lane] = lane < nvalid ? max(result, 0) : 0;
-      if (lane < p.top_n) p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + lane] = result;
-    }
+    fold_block_scores(pg, imp, y, nb, nb, p, tid, NT);
   } else if (tid < 64) {
-    blk_s[tid] = tid < nvalid ? p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + tid] : 0;
+    blk_s[tid] = tid < nvalid ? max(p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + tid], 0) : 0;
   }
   __syncthreads();
 
+  // ---- window attention; when the selection runs here, wave 0 selects meanwhile ----
   UF uf;
   uf.init(p.q + (int64_t)b * p.q_st + (int64_t)head * p.q_sh, p.scale_log2, lane, Vs_all + wave * SLOT);
-  if (t >= 0) {
-    if (wave < NW_SLC) {
-      const int upb = Bs / UK;
-      uf.run(wave, NW_SLC, nvalid * upb, 0, t,
-             [&](int u) { int slot = u / upb; return max(blk_s[slot], 0) * Bs + (u - slot * upb) * UK; }, tab_s, page,
-             kbase, p.k_sr, vbase, p.v_sr);
-    } else {
+  const int w_first = select_here ? 1 : 0;
+  if (wave < w_first) {
+    const int result = select_blocks_wave(imp, t, nb, p, lane);
+    blk_s[lane] = lane < nvalid ? max(result, 0) : 0;
+    if (p.topk && lane < p.top_n) p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + lane] = result;
+  } else {
+    if (t >= 0) {
       const int klo = max(0, t - p.window);
       const int k0 = (klo / UK) * UK;
       const int nu = (t - k0) / UK + 1;
-      uf.run(wave - NW_SLC, NW - NW_SLC, nu, klo, t, [&](int u) { return k0 + u * UK; }, tab_s, page, kbase, p.k_sr,
+      uf.run(wave - w_first, NW - w_first, nu, klo, t, [&](int u) { return k0 + u * UK; }, tab_s, page, kbase, p.k_sr,
              vbase, p.v_sr);
     }
+    uf.publish(part_m + wave * 16, part_l + wave * 16, reinterpret_cast<float*>(Vs_all + wave * SLOT));
+  }
+  __syncthreads();
+  const float* part_o = reinterpret_cast<const float*>(Vs_all);
+  if (tid < 16) merge_weights(part_m + w_first * 16, part_l + w_first * 16, NW - w_first, 16, tid, p.scale_log2);
+  __syncthreads();
+  float o_swa_pre[OPT];
+#pragma unroll
+  for (int r = 0; r < OPT; r++) {
+    const int idx = tid + r * NT;
+    const int h = idx / VD, d = idx - h * VD;
+    o_swa_pre[r] = merge_value(part_l + w_first * 16, part_o + w_first * (SLOT / 2), NW - w_first, 16, SLOT / 2, h, d, VD);
+  }
+  __syncthreads();  // the slots are staging space again
+
+  // ---- selected blocks, all waves ----
+  uf.reset();
+  if (t >= 0) {
+    const int upb = Bs / UK;
+    uf.run(wave, NW, nvalid * upb, 0, t,
+           [&](int u) { int slot = u / upb; return blk_s[slot] * Bs + (u - slot * upb) * UK; }, tab_s, page, kbase,
+           p.k_sr, vbase, p.v_sr);
   }
   uf.publish(part_m + wave * 16, part_l + wave * 16, reinterpret_cast<float*>(Vs_all + wave * SLOT));
   __syncthreads();
-  const float* part_o = reinterpret_cast<const float*>(Vs_all);
-  for (int idx = tid; idx < 16 * VD; idx += NW * 64) {
-    int h = idx / VD, d = idx - h * VD;
+  if (tid < 16) merge_weights(part_m, part_l, NW, 16, tid, p.scale_log2);
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < OPT; r++) {
+    const int idx = tid + r * NT;
+    const int h = idx / VD, d = idx - h * VD;
     if (h >= G) continue;
     const int hq = kh * G + h;
-    float o_slc = merge_partials(part_m, part_l, part_o, NW_SLC, 16, SLOT / 2, h, d, VD, p.scale_log2, nullptr);
-    float o_swa = merge_partials(part_m + NW_SLC * 16, part_l + NW_SLC * 16, part_o + NW_SLC * (SLOT / 2),
-                                 NW - NW_SLC, 16, SLOT / 2, h, d, VD, p.scale_log2, nullptr);
+    float o_slc = merge_value(part_l, part_o, NW, 16, SLOT / 2, h, d, VD);
     // branch outputs are rounded to bf16 before the gated sum, as the three-kernel path stores them
     o_slc = (float)(bf16_t)o_slc;
-    o_swa = (float)(bf16_t)o_swa;
+    const float o_swa = (float)(bf16_t)o_swa_pre[r];
     if (p.slc_o) p.slc_o[(int64_t)b * p.co_st + (int64_t)hq * p.co_sh + d] = (bf16_t)o_slc;
     if (p.swa_o) p.swa_o[(int64_t)b * p.co_st + (int64_t)hq * p.co_sh + d] = (bf16_t)o_swa;
     if (p.out) {
@@ -672,7 +863,14 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecod
       float s0 = 1.f / (1.f + __expf(-(float)wp[0]));
       float s1 = 1.f / (1.f + __expf(-(float)wp[1]));
       float s2 = 1.f / (1.f + __expf(-(float)wp[2]));
-      float o_cmp = (float)p.cmp_o[(int64_t)b * p.co_st + (int64_t)hq * p.co_sh + d];
+      float o_cmp;
+      if (p.sp_keep_p != nullptr) {  // merged in the prologue
+        const float o = ocmp_pre[r];
+        if (p.cmp_o) p.cmp_o[(int64_t)b * p.co_st + (int64_t)hq * p.co_sh + d] = (bf16_t)o;
+        o_cmp = (float)(bf16_t)o;
+      } else {
+        o_cmp = (float)p.cmp_o[(int64_t)b * p.co_st + (int64_t)hq * p.co_sh + d];
+      }
       p.out[(int64_t)b * p.o_st + (int64_t)hq * p.o_sh + d] = (bf16_t)(o_cmp * s0 + o_slc * s1 + o_swa * s2);
     }
   }
@@ -798,20 +996,20 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_fused_kernel(NsaDecodeP
   uf.run(wave, NW, nu, 0, y - 1, [&](int u) { return u * UK; }, ctab_s, page, kbase, p.k_sr, vbase, p.v_sr);
   uf.publish(part_m + wave * 16, part_l + wave * 16, reinterpret_cast<float*>(slots + wave * SLOT));
   __syncthreads();
+  if (tid < 16) {
+    const float lse2 = merge_weights(part_m, part_l, NW, 16, tid, p.scale_log2);
+    lse_s[tid] = tid < G ? lse2 : 0.f;
+    if (tid < G && p.lse_out) p.lse_out[(int64_t)b * p.lse_st + (kh * G + tid) * p.lse_sh] = lse2;
+  }
+  __syncthreads();
   float o_cmp[OPT];
 #pragma unroll
   for (int r = 0; r < OPT; r++) {
     const int idx = tid + r * NTHREADS;
     const int h = idx / VD, d = idx - h * VD;
-    float lse2;
-    float o = merge_partials(part_m, part_l, reinterpret_cast<const float*>(slots), NW, 16, SLOT / 2, h, d, VD,
-                             p.scale_log2, &lse2);
+    const float o = merge_value(part_l, reinterpret_cast<const float*>(slots), NW, 16, SLOT / 2, h, d, VD);
     o_cmp[r] = (float)(bf16_t)o;  // the staged path stores the branch output as bf16 before the gated sum
-    if (d == 0) lse_s[h] = h < G ? lse2 : 0.f;
-    if (h < G) {
-      if (p.cmp_o) p.cmp_o[(int64_t)b * p.co_st + (int64_t)(kh * G + h) * p.co_sh + d] = (bf16_t)o;
-      if (d == 0 && p.lse_out) p.lse_out[(int64_t)b * p.lse_st + (kh * G + h) * p.lse_sh] = lse2;
-    }
+    if (h < G && p.cmp_o) p.cmp_o[(int64_t)b * p.co_st + (int64_t)(kh * G + h) * p.co_sh + d] = (bf16_t)o;
   }
   __syncthreads();
   // ---- probabilities p = kept exp2((s - m_unit)*c) * exp2(m_unit*c - lse), summed over the heads ----
@@ -860,15 +1058,17 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_fused_kernel(NsaDecodeP
   }
   uf.publish(part_m + wave * 16, part_l + wave * 16, reinterpret_cast<float*>(slots + wave * SLOT));
   __syncthreads();
+  if (tid < 16) merge_weights(part_m, part_l, NW, 16, tid, p.scale_log2);
+  else if (tid < 32) merge_weights(swa_m + 16, swa_l + 16, NW - 1, 16, tid - 16, p.scale_log2);
+  __syncthreads();
 #pragma unroll
   for (int r = 0; r < OPT; r++) {
     const int idx = tid + r * NTHREADS;
     const int h = idx / VD, d = idx - h * VD;
     if (h >= G) continue;
     const int hq = kh * G + h;
-    float o_slc = merge_partials(part_m, part_l, reinterpret_cast<const float*>(slots), NW, 16, SLOT / 2, h, d, VD,
-                                 p.scale_log2, nullptr);
-    float o_swa = merge_partials(swa_m + 16, swa_l + 16, swa_o, NW - 1, 16, 16 * VD, h, d, VD, p.scale_log2, nullptr);
+    float o_slc = merge_value(part_l, reinterpret_cast<const float*>(slots), NW, 16, SLOT / 2, h, d, VD);
+    float o_swa = merge_value(swa_l + 16, swa_o, NW - 1, 16, 16 * VD, h, d, VD);
     o_slc = (float)(bf16_t)o_slc;
     o_swa = (float)(bf16_t)o_swa;
     if (p.slc_o) p.slc_o[(int64_t)b * p.co_st + (int64_t)hq * p.co_sh + d] = (bf16_t)o_slc;
@@ -933,7 +1133,8 @@ int nsa_decode_cmp_topk_launch(const NsaDecodeParams& p, int B, int D, int VD, h
 int nsa_decode_slc_swa_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream) {
   if (B <= 0) return NSA_OK;
   dim3 grid(B, p.KH);
-  size_t extra = (size_t)(2 * DEC_WAVES * 16 + 64 + p.table_stride) * sizeof(float);
+  size_t extra = (size_t)(2 * DEC_WAVES * 16 + 64 + ((p.table_stride + 3) & ~3)) * sizeof(float);
+  if (p.pg != nullptr) extra += (size_t)((p.nb_cap + 3) & ~3) * sizeof(float);  // block scores
   if (D == 128 && VD == 128)
     return launch_dyn(decode_slc_swa_kernel<128, 128>, grid, slot_bytes<128, 128>() + extra, p, stream,
                       "decode_slc_swa_kernel");
@@ -967,6 +1168,47 @@ int nsa_decode_cmp_split_launch(const NsaDecodeParams& p, int B, int nsplit, int
     decode_importance_kernel<64, 64><<<grid, SPLIT_WAVES * 64, dyn2, stream>>>(p);
   }
   return nsa_check_launch("decode_importance_kernel");
+}
+
+// ---- two-launch split path: partial kernel with the probability spill, then the final kernel ----
+template <int D, int VD>
+static size_t split_final_lds(const NsaDecodeParams& p) {
+  const size_t slots = slot_bytes<D, VD>();
+  if ((size_t)((p.y_cap + UK - 1) / UK) * UK * 4 > slots) return 0;  // head-summed probabilities overlay the slots
+  const size_t nuc = (size_t)(p.y_cap + UK - 1) / UK;
+  const size_t total = slots + (size_t)(2 * DEC_WAVES * 16 + 64 + ((p.table_stride + 3) & ~3)) * 4 +
+                       (size_t)(((p.nb_cap + 3) & ~3) + (nuc * 16 > 2 * 64 * 16 ? nuc * 16 : 2 * 64 * 16)) * 4;  // factors, or the parts' (m, l)
+  return total <= 160 * 1024 ? total : 0;
+}
+
+int nsa_decode_split_lds_bytes(const NsaDecodeParams& p, int D, int VD) {
+  if (D == 128 && VD == 128) return (int)split_final_lds<128, 128>(p);
+  if (D == 64 && VD == 64) return (int)split_final_lds<64, 64>(p);
+  return 0;
+}
+
+int nsa_decode_split_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream) {
+  if (B <= 0) return NSA_OK;
+  const int lds2 = nsa_decode_split_lds_bytes(p, D, VD);
+  if (lds2 == 0) {
+    nsa_set_error("decode_split: head dims %d/%d or fixed_y_maxlen %d / fixed_num_slc_blocks %d / table width %d do "
+                  "not fit the final kernel's LDS", D, VD, p.y_cap, p.nb_cap, p.table_stride);
+    return NSA_ERR_UNSUPPORTED;
+  }
+  dim3 grid1(B, p.KH, p.nsplit), grid2(B, p.KH);
+  const int ntab = (p.y_cap + p.page_size - 1) / p.page_size;
+  const size_t dyn1 = (size_t)SPLIT_WAVES * (D == 128 ? UnitFlash<128, 128>::SLOT : UnitFlash<64, 64>::SLOT) * 2 +
+                      (size_t)(2 * SPLIT_WAVES * 16 + ntab) * 4;
+  if (D == 128) {
+    decode_cmp_partial_kernel<128, 128><<<grid1, SPLIT_WAVES * 64, dyn1, stream>>>(p);
+    int rc = nsa_check_launch("decode_cmp_partial_kernel");
+    if (rc) return rc;
+    return launch_dyn(decode_slc_swa_kernel<128, 128>, grid2, (size_t)lds2, p, stream, "decode_slc_swa_kernel");
+  }
+  decode_cmp_partial_kernel<64, 64><<<grid1, SPLIT_WAVES * 64, dyn1, stream>>>(p);
+  int rc = nsa_check_launch("decode_cmp_partial_kernel");
+  if (rc) return rc;
+  return launch_dyn(decode_slc_swa_kernel<64, 64>, grid2, (size_t)lds2, p, stream, "decode_slc_swa_kernel");
 }
 
 // LDS of the one-launch decode kernel; 0 when it does not fit (the caller then takes the two-launch path)

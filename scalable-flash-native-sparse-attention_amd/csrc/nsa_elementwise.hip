@@ -317,10 +317,30 @@ __global__ void paged_pool_decode_kernel(bf16_t* kc, int64_t k_sr, int64_t k_sh,
   const int st = ((L - K) / S) * S;
   const int32_t* tb = table + (int64_t)b * table_stride;
   float a[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  for (int r = 0; r < K; r++) {
-    int n = st + r;
-    int64_t row = (int64_t)tb[n / page] * page + (n % page);
-    acc8(a, ld_global_b128(cache + row * c_sr + (int64_t)h * c_sh + c * 8));
+  if (K <= page) {
+    // the window touches at most two pages: both table entries are read up front, then the rows are fetched eight at
+    // a time (independent loads) and added in row order
+    const int p0 = st / page, r0 = st - p0 * page;
+    const int64_t base0 = (int64_t)tb[p0] * page + r0;
+    const int64_t base1 = r0 + K > page ? (int64_t)tb[p0 + 1] * page + r0 - page : base0;
+    const bf16_t* col = cache + (int64_t)h * c_sh + c * 8;
+    for (int r = 0; r < K; r += 8) {
+      bf16x8 x[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        const int rr = min(r + u, K - 1);
+        x[u] = ld_global_b128(col + ((r0 + rr < page ? base0 : base1) + rr) * c_sr);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; u++)
+        if (r + u < K) acc8(a, x[u]);
+    }
+  } else {
+    for (int r = 0; r < K; r++) {
+      int n = st + r;
+      int64_t row = (int64_t)tb[n / page] * page + (n % page);
+      acc8(a, ld_global_b128(cache + row * c_sr + (int64_t)h * c_sh + c * 8));
+    }
   }
   float inv = 1.f / (float)K;
   *reinterpret_cast<bf16x8*>(cache + (int64_t)slot * c_sr + (int64_t)h * c_sh + c * 8) =

@@ -7,7 +7,7 @@ from .stages import (mean_pooling_prefill, kv_mean_pooling_decode, cmp_attn_pref
                      topk_decode, slc_attn_prefill, fused_slc_swa_attn_decode, swa_prefill, combine_prefill,
                      combine_decode, mean_pooling_decode, slc_attn_decode, fused_decode_supported, decode_cmp_topk,
                      decode_slc_swa_combine, decode_cmp_split, decode_one_launch, decode_one_launch_fits,
-                     store_kvcache, store_kvcache_and_pool_prefill)
+                     store_kvcache, store_kvcache_and_pool_prefill, decode_split, decode_split_fits)
 from .paging import PageTableBuilder, allocate_kv_pools
 
 
@@ -49,18 +49,35 @@ def nsa_prefill(q, k, v, w, x_cu_seqlens, y_cu_seqlens, x_maxlen, y_maxlen, cont
     return combine_prefill(cmp_o, slc_o, swa_o, w)
 
 
+def auto_cmp_splits(batch, num_kv_heads, fixed_y_maxlen, num_cus=256):
+    """Parts the compressed branch of a decode step is cut into per (request, kv head).  One workgroup per pair
+    fills the GPU from about one pair per CU on; a small batch of long contexts (>= 2048 compressed rows, i.e. 32K
+    tokens) is cut so that there are again about num_cus workgroups (measured on MI355X, 4 kv heads: 32 requests of
+    64K tokens 153 -> 117 us with 2 parts, 16 requests of 128K tokens 222 -> 118 us with 4)."""
+    pairs = batch * num_kv_heads
+    if fixed_y_maxlen <= 2048 or pairs * 2 > num_cus:
+        return 1
+    n = 2
+    while n < 8 and pairs * n * 2 <= num_cus:
+        n *= 2
+    return n
+
+
 def nsa_decode(q, k, v, w, context_lens, block_tables, cmp_slot_mapping, cmp_block_tables, cmp_num_splits=0,
                slc_num_splits=0, fixed_y_maxlen=8192, fixed_num_slc_blocks=2048, kernel_size=32, stride=16,
                block_size=64, top_n=16, num_init_blocks=1, num_local_blocks=2, window_size=512, sm_scale=None,
                new_k=None, new_v=None, slot_mapping=None):
     """One query token per request.  q [B,QH,D]; w [B,QH,3]; cmp_slot_mapping [B] (-1: no compressed row completes
     at this step).  Rows with context_lens == 0 (graph padding) produce zeros.  Returns o [B,QH,VD].
+    cmp_num_splits: 0 = chosen from the batch size and fixed_y_maxlen (auto_cmp_splits), 1 = never split.
     As upstream, the newest token's K/V are expected in the pools already; alternatively pass them as new_k / new_v
     [B,KH,*] with their flat pool rows slot_mapping [B] (-1: padding) and the cache write happens here (inside the
     single decode launch when that path is taken)."""
     assert k.size(1) % 64 == 0, "page size must be a multiple of 64"
     if sm_scale is None:
         sm_scale = q.size(-1) ** -0.5
+    if cmp_num_splits == 0:
+        cmp_num_splits = auto_cmp_splits(q.size(0), k.size(2), fixed_y_maxlen)
     one_launch = (fused_decode_supported(q, k, v) and cmp_num_splits <= 1 and
                   decode_one_launch_fits(q, k, v, block_tables, fixed_y_maxlen, fixed_num_slc_blocks))
     if one_launch:
@@ -84,8 +101,15 @@ def nsa_decode(q, k, v, w, context_lens, block_tables, cmp_slot_mapping, cmp_blo
                                           num_inital=num_init_blocks, num_local=num_local_blocks, sm_scale=sm_scale)
             return decode_slc_swa_combine(q, k, v, w, topk, cmp_o, block_tables, context_lens, block_size=block_size,
                                           top_n=top_n, window_size=window_size, sm_scale=sm_scale)
-        # cmp_num_splits > 1: the compressed branch is cut in that many key-interleaved parts per (request, kv head)
-        # (three launches); pays off when a few very long contexts sit in a batch of short ones
+        # cmp_num_splits > 1: the compressed branch is cut in that many key-interleaved parts per (request, kv head);
+        # pays off for small batches of long contexts and when a few very long contexts sit in a batch of short ones
+        if decode_split_fits(q, k, v, block_tables, fixed_y_maxlen, fixed_num_slc_blocks):
+            return decode_split(q, k, v, w, block_tables, cmp_block_tables, context_lens, nsplit=cmp_num_splits,
+                                fixed_y_maxlen=fixed_y_maxlen, fixed_num_slc_blocks=fixed_num_slc_blocks,
+                                kernel_size=kernel_size, stride=stride, block_size=block_size, top_n=top_n,
+                                num_inital=num_init_blocks, num_local=num_local_blocks, window_size=window_size,
+                                sm_scale=sm_scale)
+        # capacities beyond the LDS of that path: three launches, the probabilities recomputed from the keys
         cmp_o, pg = decode_cmp_split(q, k, v, cmp_block_tables, context_lens, nsplit=cmp_num_splits,
                                      fixed_y_maxlen=fixed_y_maxlen, kernel_size=kernel_size, stride=stride,
                                      sm_scale=sm_scale)

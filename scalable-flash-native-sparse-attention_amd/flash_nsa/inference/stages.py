@@ -323,6 +323,49 @@ def decode_cmp_split(q, k, v, cmp_block_tables, context_lens, nsplit=4, fixed_y_
     return cmp_o, pg
 
 
+def decode_split_fits(q, k, v, block_tables, fixed_y_maxlen, fixed_num_slc_blocks):
+    """True when decode_split's second kernel holds its tables and scores in LDS for these capacities."""
+    return bool(_lib.value("nsa_decode_split_fits", q.size(-1), v.size(-1), int(fixed_y_maxlen),
+                           int(fixed_num_slc_blocks), block_tables.size(1)))
+
+
+def decode_split(q, k, v, w, block_tables, cmp_block_tables, context_lens, nsplit=4, fixed_y_maxlen=8192,
+                 fixed_num_slc_blocks=2048, kernel_size=32, stride=16, block_size=64, top_n=16, num_inital=1,
+                 num_local=2, window_size=512, sm_scale=None, return_parts=False):
+    """The decode step in two launches, for small batches of long contexts: the compressed branch cut into `nsplit`
+    parts per (request, kv head) so that it fills the GPU, then one workgroup per pair for the merge, the block
+    selection, selected + window attention and the gated combine.  -> o [B,QH,VD]
+    (return_parts: also cmp_o, slc_o, swa_o, topk [KH,B,top_n], lse [B,QH])."""
+    check_bf16(q)
+    page, KH, D, ksr, ksh = _pool_args(k)
+    _, _, VD, vsr, vsh = _pool_args(v)
+    B, QH, _ = q.shape
+    sm_scale = q.size(-1) ** -0.5 if sm_scale is None else sm_scale
+    dev = q.device
+    out = torch.empty(B, QH, VD, device=dev, dtype=q.dtype)
+    parts = [torch.empty_like(out) for _ in range(3)] if return_parts else [None] * 3
+    topk = torch.empty(KH, B, top_n, device=dev, dtype=torch.int32) if return_parts else None
+    lse = torch.empty(B, QH, device=dev, dtype=torch.float32) if return_parts else None
+    ycap32 = (int(fixed_y_maxlen) + 31) // 32 * 32
+    sp_ml = torch.empty(2, B, KH, nsplit, 16, device=dev, dtype=torch.float32)
+    sp_o = torch.empty(B, KH, nsplit, 16, VD, device=dev, dtype=torch.float32)
+    keep_p = torch.empty(B, KH, 16, ycap32, device=dev, dtype=torch.float16)
+    keep_m = torch.empty(B, KH, ycap32 // 32, 16, device=dev, dtype=torch.float32)
+    _lib.call("nsa_decode_split", q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), ksr, ksh, v.data_ptr(), vsr,
+              vsh, w.data_ptr(), w.stride(0), w.stride(1), out.data_ptr(), out.stride(0), out.stride(1),
+              _lib.ptr(parts[0]), _lib.ptr(parts[1]), _lib.ptr(parts[2]), out.stride(0), out.stride(1),
+              _lib.ptr(lse), lse.stride(0) if return_parts else 0, lse.stride(1) if return_parts else 0,
+              _lib.ptr(topk), topk.stride(0) if return_parts else 0, topk.stride(1) if return_parts else 0,
+              sp_ml[0].data_ptr(), sp_ml[1].data_ptr(), sp_o.data_ptr(), keep_p.data_ptr(), keep_m.data_ptr(), nsplit,
+              _i32(context_lens).data_ptr(), _i32(block_tables).data_ptr(), block_tables.stride(0),
+              _i32(cmp_block_tables).data_ptr(), cmp_block_tables.stride(0), page, B, QH, KH, D, VD,
+              int(fixed_y_maxlen), int(fixed_num_slc_blocks), kernel_size, stride, block_size, top_n, num_inital,
+              num_local, -1, window_size, sm_scale, _lib.stream_ptr())
+    if return_parts:
+        return out, parts[0], parts[1], parts[2], topk, lse
+    return out
+
+
 def decode_slc_swa_combine(q, k, v, w, topk, cmp_o, block_tables, context_lens, block_size=64, top_n=16,
                            window_size=512, sm_scale=None, return_branches=False, pg=None, fixed_num_slc_blocks=2048,
                            kernel_size=32, stride=16, num_inital=1, num_local=2):

@@ -268,6 +268,51 @@ def test_one_launch_decode_matches_two_launch_and_staged(device, QH, KH, D):
     assert torch.equal(out, out2), "optional outputs must not change the result"
 
 
+@pytest.mark.parametrize("QH,KH,D", [(64, 4, 128), (16, 1, 128), (12, 2, 64)])
+@pytest.mark.parametrize("nsplit", [1, 3, 4])
+def test_split_decode_matches_one_launch(device, QH, KH, D, nsplit):
+    """The two-launch decode for small batches of long contexts (compressed branch in `nsplit` parts with spilled
+    fp16 probabilities, then merge + selection + selected/window attention + combine) against the one-launch kernel:
+    same lse and selection (both fold the same fp16 probabilities), branch outputs and output to bf16 rounding."""
+    from flash_nsa.inference import decode_one_launch, decode_split, decode_split_fits
+    ctx = [4096, 333, 48, 31, 1, 777, 2999, 640, 1024, 65, 0, 513, 514]
+    case = build_pool([max(c, 1) for c in ctx], KH, D, D, page=128, seed=51)
+    prepool(case, [max(c, 1) for c in ctx])
+    B = len(ctx)
+    d = to_dev(case, device)
+    q = randn_bf16(B, QH, D, seed=52).to(device)
+    w = randn_bf16(B, QH, 3, seed=53).to(device)
+    ctx_t = torch.tensor(ctx, dtype=torch.int32, device=device)
+    assert decode_split_fits(q, d["k"], d["v"], d["bt"], 512, 64)
+    assert not decode_split_fits(q, d["k"], d["v"], d["bt"], 32768, 8192)
+    kw = dict(top_n=8, window_size=200)
+    r_out, r_cmp, r_slc, r_swa, r_topk, r_lse = decode_one_launch(q, d["k"], d["v"], w, d["bt"], d["cbt"], ctx_t, 512,
+                                                                  64, return_parts=True, **kw)
+    out, cmp_o, slc_o, swa_o, topk, lse = decode_split(q, d["k"], d["v"], w, d["bt"], d["cbt"], ctx_t, nsplit=nsplit,
+                                                       fixed_y_maxlen=512, fixed_num_slc_blocks=64,
+                                                       return_parts=True, **kw)
+    live = ctx_t > 0
+    assert_close(lse[live], r_lse[live], "lse", atol=1e-4, rtol=1e-5)
+    assert_close(cmp_o[live], r_cmp[live], "cmp_o", atol=4e-3, rtol=1e-2)
+    # the parts change the order of the fp32 sums behind the scores: selections may differ only at score ties
+    nv = torch.clamp((ctx_t - 1) // 64 + 1, max=8).cpu()
+    a, r = topk.cpu(), r_topk.cpu()
+    same = [(b, kh) for b in range(B) if ctx[b] > 0 for kh in range(KH)
+            if sorted(a[kh, b, :nv[b]].tolist()) == sorted(r[kh, b, :nv[b]].tolist())]
+    n_pairs = sum(1 for c in ctx if c > 0) * KH
+    assert len(same) >= n_pairs - max(1, n_pairs // 50), f"{n_pairs - len(same)} of {n_pairs} selections differ"
+    G = QH // KH
+    for b, kh in same:
+        hs = slice(kh * G, (kh + 1) * G)
+        assert_close(slc_o[b, hs], r_slc[b, hs], "slc_o", atol=4e-3, rtol=1e-2)
+        assert_close(swa_o[b, hs], r_swa[b, hs], "swa_o", atol=4e-3, rtol=1e-2)
+        assert_close(out[b, hs], r_out[b, hs], "o", atol=8e-3, rtol=1e-2)
+    assert float(out[~live].abs().max()) == 0.0, "a padded request (context 0) must give zeros"
+    out2 = decode_split(q, d["k"], d["v"], w, d["bt"], d["cbt"], ctx_t, nsplit=nsplit, fixed_y_maxlen=512,
+                        fixed_num_slc_blocks=64, **kw)
+    assert torch.equal(out, out2), "optional outputs must not change the result"
+
+
 def test_one_launch_decode_pools_the_new_row_itself(device):
     """nsa_decode's one-launch kernel with a slot mapping == pooling kernel followed by the same kernel without:
     the pools end bit-identical and so do the outputs."""
