@@ -10,6 +10,7 @@
 // arg-max (lowest index on ties) -- only the int32 indices leave the CU (plus the fp32 scores on request).
 #include "nsa_common.h"
 #include "nsa_api_internal.h"
+#include <type_traits>
 
 namespace {
 
@@ -43,6 +44,8 @@ NSA_DEVICE int select_row(float* imp, int t, int nb_max, const NsaTopkParams& p,
     if (lane <= nk) result = nk - (lane - p.num_init);
   }
   if (REGS) {
+    // candidates in two groups of 8 registers with their best kept aside: a round marks and rescans only the group
+    // the winner came from (its number is wave-uniform)
     float v[16];
 #pragma unroll
     for (int k = 0; k < 16; k++) {
@@ -51,23 +54,37 @@ NSA_DEVICE int select_row(float* imp, int t, int nb_max, const NsaTopkParams& p,
       if (j <= jmax && (j < p.num_init || j > nk - p.num_local)) x = -1.f;
       v[k] = x;
     }
-    float best = -2.f;
-    int bj = 0x7fffffff;
+    float gbest[2];
+    int gidx[2];
+    auto rescan = [&](auto g_tag) {
+      constexpr int g = decltype(g_tag)::value;
+      float bs = -2.f;
+      int bi = 0x7fffffff;
 #pragma unroll
-    for (int k = 0; k < 16; k++)
-      if (v[k] > best) { best = v[k]; bj = lane + 64 * k; }
+      for (int k = g * 8; k < g * 8 + 8; k++)
+        if (v[k] > bs) { bs = v[k]; bi = lane + 64 * k; }
+      gbest[g] = bs;
+      gidx[g] = bi;
+    };
+    rescan(std::integral_constant<int, 0>{});
+    rescan(std::integral_constant<int, 1>{});
     for (int slot = p.num_init + p.num_local; slot < nsel; slot++) {
-      const int w = wave_argmax_lowest(best, bj, bj != 0x7fffffff);
+      const bool second = gbest[1] > gbest[0];
+      const int w = wave_argmax_lowest(second ? gbest[1] : gbest[0], second ? gidx[1] : gidx[0],
+                                       (second ? gidx[1] : gidx[0]) != 0x7fffffff);
       if (lane == slot) result = w;
-      const bool mine = (w & 63) == lane && w <= jmax;
+      if (w > jmax) continue;  // wave-uniform: no candidate left
+      const bool mine = (w & 63) == lane;
       const int kk = w >> 6;
-      best = -2.f;
-      bj = 0x7fffffff;
+      auto take = [&](auto g_tag) {
+        constexpr int g = decltype(g_tag)::value;
 #pragma unroll
-      for (int k = 0; k < 16; k++) {
-        if (mine && k == kk) v[k] = -1.f;
-        if (v[k] > best) { best = v[k]; bj = lane + 64 * k; }
-      }
+        for (int k = g * 8; k < g * 8 + 8; k++)
+          if (mine && k == kk) v[k] = -1.f;
+        rescan(g_tag);
+      };
+      if (kk < 8) take(std::integral_constant<int, 0>{});
+      else take(std::integral_constant<int, 1>{});
     }
     return result;
   }
