@@ -77,7 +77,9 @@ def nsa_decode(q, k, v, w, context_lens, block_tables, cmp_slot_mapping, cmp_blo
     if sm_scale is None:
         sm_scale = q.size(-1) ** -0.5
     if cmp_num_splits == 0:
-        cmp_num_splits = auto_cmp_splits(q.size(0), k.size(2), fixed_y_maxlen)
+        # the split kernels exist for the shapes of the fused decode kernels (head dims 128/128 or 64/64, at most 16
+        # q-heads per kv head)
+        cmp_num_splits = auto_cmp_splits(q.size(0), k.size(2), fixed_y_maxlen) if fused_decode_supported(q, k, v) else 1
     one_launch = (fused_decode_supported(q, k, v) and cmp_num_splits <= 1 and
                   decode_one_launch_fits(q, k, v, block_tables, fixed_y_maxlen, fixed_num_slc_blocks))
     if one_launch:

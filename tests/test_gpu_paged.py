@@ -363,3 +363,28 @@ def test_decode_qk192_v128_equals_training_last_row(device):
         with torch.no_grad():
             full = core(qs.to(device), ks, vs, ws.to(device), torch.tensor([0, L], dtype=torch.int32, device=device))
         assert_close(o[b], full[-1], f"decode vs training row (request {b})", atol=1e-2, rtol=1e-2)
+
+
+def test_decode_small_batch_long_context_takes_the_split_path(device):
+    """nsa_decode with its defaults on 2 requests of 40K tokens (fixed_y_maxlen 4096): the compressed branch is cut
+    into parts by itself; the result equals the two-launch path without parts up to ties of the selection, and head
+    dims the split kernels are not built for (192/128) are not routed there."""
+    from flash_nsa import nsa_decode
+    from flash_nsa.inference import auto_cmp_splits, decode_cmp_topk, decode_slc_swa_combine
+    assert auto_cmp_splits(2, 4, 4096) == 8 and auto_cmp_splits(64, 4, 4096) == 1 and auto_cmp_splits(2, 4, 2048) == 1
+    QH, KH, D = 64, 4, 128
+    ctx = [40000, 33333]
+    case = build_pool(ctx, KH, D, D, page=256, seed=61)
+    prepool(case, ctx)
+    d = to_dev(case, device)
+    q, w = randn_bf16(2, QH, D, seed=62).to(device), randn_bf16(2, QH, 3, seed=63).to(device)
+    ctx_t = torch.tensor(ctx, dtype=torch.int32, device=device)
+    none = torch.full((2,), -1, dtype=torch.int32, device=device)
+    kw = dict(fixed_y_maxlen=4096, fixed_num_slc_blocks=1024)
+    o = nsa_decode(q, d["k"], d["v"], w, ctx_t, d["bt"], none, d["cbt"], **kw)
+    cmp_o, topk = decode_cmp_topk(q, d["k"], d["v"], d["cbt"], ctx_t, **kw)
+    ref = decode_slc_swa_combine(q, d["k"], d["v"], w, topk, cmp_o, d["bt"], ctx_t)
+    err = (o.float() - ref.float()).abs().view(2, KH, -1).amax(-1)           # per (request, kv head)
+    assert int((err > 1e-2).sum()) <= 1, err
+    o1 = nsa_decode(q, d["k"], d["v"], w, ctx_t, d["bt"], none, d["cbt"], cmp_num_splits=1, **kw)
+    assert_close(o1, ref, "no parts", atol=8e-3, rtol=1e-2)
