@@ -11,7 +11,7 @@ import torch
 PEAK_HBM_GBS = 8000.0
 # bytes per step crossing the L2 <-> memory-side boundary (rocprofv3 --pmc FETCH_SIZE x2.000 + WRITE_SIZE x1.000, the
 # factors being what the counters read for a 1 GiB copy), measured for the default case of build_case()
-MEASURED_TRAFFIC_DEFAULT_CASE = 333.8e6
+MEASURED_TRAFFIC_DEFAULT_CASE = 334.2e6
 
 
 def build_case(dev, B=64, QH=64, KH=4, D=128, page=256, lo=4096, hi=32768, seed=3):
