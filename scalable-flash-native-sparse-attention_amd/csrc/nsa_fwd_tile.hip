@@ -27,8 +27,10 @@ __global__ __launch_bounds__(256, MINB) void fwd_tile_kernel(NsaFwdTileParams p)
   constexpr int KT = 64;
   constexpr int KLD = D + NSA_LDS_PAD;
   constexpr int VLD = VD + NSA_LDS_PAD;
-  __shared__ __attribute__((aligned(16))) bf16_t Ks[KT * KLD];
-  __shared__ __attribute__((aligned(16))) bf16_t Vs[KT * VLD];
+  // two K/V tile buffers: the tile after the one being computed is stored while the other waves may still read the
+  // current one, so a tile costs one barrier
+  __shared__ __attribute__((aligned(16))) bf16_t Ks2[2][KT * KLD];
+  __shared__ __attribute__((aligned(16))) bf16_t Vs2[2][KT * VLD];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -138,7 +140,7 @@ __global__ __launch_bounds__(256, MINB) void fwd_tile_kernel(NsaFwdTileParams p)
   };
 
   // one 64-key tile for one row set
-  auto process = [&](bool masked, auto rs_tag, int kt) {
+  auto process = [&](bool masked, auto rs_tag, int kt, const bf16_t* Ks, const bf16_t* Vs) {
     constexpr int rs = decltype(rs_tag)::value;
     // ---- S^T = K Q^T : two 32-key sub tiles, interleaved accumulators ----
     f32x16 sacc[2];
@@ -215,22 +217,31 @@ __global__ __launch_bounds__(256, MINB) void fwd_tile_kernel(NsaFwdTileParams p)
     }
   };
 
-  if (key_begin < key_end) gload(key_begin);
-
-  for (int kt = key_begin; kt < key_end; kt += KT) {
-    __syncthreads();
+  auto stage = [&](int buf) {
 #pragma unroll
     for (int j = 0; j < KJ; j++) {
       int pc = tid + j * 256;
-      *reinterpret_cast<bf16x8*>(&Ks[(pc / KP) * KLD + (pc % KP) * 8]) = kreg[j];
+      *reinterpret_cast<bf16x8*>(&Ks2[buf][(pc / KP) * KLD + (pc % KP) * 8]) = kreg[j];
     }
 #pragma unroll
     for (int j = 0; j < VJ; j++) {
       int pc = tid + j * 256;
-      *reinterpret_cast<bf16x8*>(&Vs[(pc / VP) * VLD + (pc % VP) * 8]) = vreg[j];
+      *reinterpret_cast<bf16x8*>(&Vs2[buf][(pc / VP) * VLD + (pc % VP) * 8]) = vreg[j];
     }
-    __syncthreads();
-    if (kt + KT < key_end) gload(kt + KT);
+  };
+  if (key_begin < key_end) {
+    gload(key_begin);
+    stage(0);
+    if (key_begin + KT < key_end) gload(key_begin + KT);
+  }
+
+  int buf = 0;
+  for (int kt = key_begin; kt < key_end; kt += KT, buf ^= 1) {
+    __syncthreads();  // tile kt is visible; nobody reads the other buffer (tile kt - KT) any more
+    if (kt + KT < key_end) {
+      stage(buf ^ 1);
+      if (kt + 2 * KT < key_end) gload(kt + 2 * KT);
+    }
     if (!wave_active) continue;
 
     // wave-uniform visibility classification of this tile
@@ -243,8 +254,8 @@ __global__ __launch_bounds__(256, MINB) void fwd_tile_kernel(NsaFwdTileParams p)
       full_vis = (kt + KT - 1 <= tw_lo) && (kt >= tw_hi - p.window);
     }
     if (!any_vis) continue;
-    process(!full_vis, std::integral_constant<int, 0>{}, kt);
-    if constexpr (RS > 1) process(!full_vis, std::integral_constant<int, RS - 1>{}, kt);
+    process(!full_vis, std::integral_constant<int, 0>{}, kt, Ks2[buf], Vs2[buf]);
+    if constexpr (RS > 1) process(!full_vis, std::integral_constant<int, RS - 1>{}, kt, Ks2[buf], Vs2[buf]);
   }
 
   // ---- epilogue ----
