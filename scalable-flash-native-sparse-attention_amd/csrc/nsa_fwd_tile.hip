@@ -19,14 +19,24 @@ namespace {
 constexpr int MODE_CMP = 0;
 constexpr int MODE_SWA = 1;
 
-template <int D, int VD, int MODE, bool PAGED, int RS, int MINB>
+typedef __attribute__((address_space(1))) const void* nsa_gptr_t;
+typedef __attribute__((address_space(3))) void* nsa_lptr_t;
+
+// position swizzle of the 16-byte chunks of row r in an unpadded LDS tile with CP chunks per row: chunk c sits at
+// position c ^ swz(r), which spreads the rows that a fragment read touches over all banks
+template <int CP>
+NSA_DEVICE constexpr int swz(int r) { return CP % 16 == 0 ? (r & 15) : ((r >> 1) & 7); }
+
+// ASYNC: the K/V tiles go from global memory straight into LDS (global_load_lds, 16 bytes per lane, no staging
+// registers, no ds_write); the tiles are then unpadded and swizzled instead of padded.
+template <int D, int VD, int MODE, bool PAGED, int RS, int MINB, bool ASYNC>
 __global__ __launch_bounds__(256, MINB) void fwd_tile_kernel(NsaFwdTileParams p) {
   static_assert(RS == 1 || RS == 2, "one or two 32-row sets per wave");
   constexpr int ROWS_W = 32 * RS;
   constexpr int ROWS_WG = 4 * ROWS_W;
   constexpr int KT = 64;
-  constexpr int KLD = D + NSA_LDS_PAD;
-  constexpr int VLD = VD + NSA_LDS_PAD;
+  constexpr int KLD = ASYNC ? D : D + NSA_LDS_PAD;
+  constexpr int VLD = ASYNC ? VD : VD + NSA_LDS_PAD;
   // two K/V tile buffers: the tile after the one being computed is stored while the other waves may still read the
   // current one, so a tile costs one barrier
   __shared__ __attribute__((aligned(16))) bf16_t Ks2[2][KT * KLD];
@@ -140,18 +150,53 @@ __global__ __launch_bounds__(256, MINB) void fwd_tile_kernel(NsaFwdTileParams p)
   };
 
   // one 64-key tile for one row set
+  // Fragment addresses.  Padded tiles: row * stride + column, the compiler folds everything but the lane part into
+  // immediates.  Swizzled tiles with a power-of-two row size: byte address = lane part XOR (index << 5 or 6) +
+  // compile-time row offset, with the lane parts computed once (kx, vxa, vxb), so a read costs at most one v_xor.
+  constexpr bool POW2 = (D == 64 || D == 128) && (VD == 64 || VD == 128);
+  int kx = 0, vxa = 0, vxb = 0;
+  if constexpr (ASYNC && POW2) {
+    const int s0 = swz<D / 8>(l32);
+    kx = (l32 * D * 2 + ((hl ^ (s0 & 1)) << 4)) ^ ((s0 >> 1) << 5);
+    const int sl = hl * 4 + (i16 >> 2);                 // row of the fragment inside its group of 16 rows
+    const int cl = (g16 & 1) * 2 + ((i16 & 3) >> 1);    // chunk inside its group of 4 chunks
+    const int sa = swz<VD / 8>(sl), sb = swz<VD / 8>(sl + 8);
+    vxa = (sl * VD * 2 + ((cl ^ (sa & 3)) << 4) + (i16 & 1) * 8) ^ ((sa >> 2) << 6);
+    vxb = ((sl + 8) * VD * 2 + ((cl ^ (sb & 3)) << 4) + (i16 & 1) * 8) ^ ((sb >> 2) << 6);
+  }
+  // K fragment: rows l32 + 32*half, chunk 2*kc + hl
+  auto kfrag = [&](const bf16_t* Ks, int half, int kc) -> bf16x8 {
+    if constexpr (ASYNC && POW2)
+      return *reinterpret_cast<const bf16x8*>(reinterpret_cast<const char*>(Ks) + half * 32 * D * 2 + (kx ^ (kc << 5)));
+    else if constexpr (ASYNC)
+      return *reinterpret_cast<const bf16x8*>(
+          Ks + ((l32 + 32 * half) * (D / 8) + ((2 * kc + hl) ^ swz<D / 8>(l32))) * 8);
+    else
+      return *reinterpret_cast<const bf16x8*>(Ks + (l32 + 32 * half) * KLD + (2 * kc + hl) * 8);
+  };
+  // transposed V fragment piece: row kb + (i16 >> 2) (kb a multiple of 16, plus 8 for the second piece), columns
+  // dt*32 + (g16&1)*16 + 4*(i16&3) ..
+  auto vfrag = [&](const bf16_t* Vs, int kb16, int second, int dt) -> bf16x4 {
+    if constexpr (ASYNC && POW2) {
+      const int x = (second ? vxb : vxa) ^ (dt << 6);
+      return lds_read_tr(reinterpret_cast<const bf16_t*>(reinterpret_cast<const char*>(Vs) + kb16 * VD * 2 + x));
+    } else {
+      const int row = kb16 + second * 8 + hl * 4 + (i16 >> 2);
+      const int col = dt * 32 + (g16 & 1) * 16 + 4 * (i16 & 3);
+      if constexpr (ASYNC) return lds_read_tr(Vs + (row * (VD / 8) + ((col >> 3) ^ swz<VD / 8>(row))) * 8 + (col & 7));
+      else return lds_read_tr(Vs + row * VLD + col);
+    }
+  };
   auto process = [&](bool masked, auto rs_tag, int kt, const bf16_t* Ks, const bf16_t* Vs) {
     constexpr int rs = decltype(rs_tag)::value;
     // ---- S^T = K Q^T : two 32-key sub tiles, interleaved accumulators ----
     f32x16 sacc[2];
 #pragma unroll
     for (int i = 0; i < 16; i++) { sacc[0][i] = 0.f; sacc[1][i] = 0.f; }
-    const bf16_t* kp0 = &Ks[l32 * KLD + hl * 8];
-    const bf16_t* kp1 = kp0 + 32 * KLD;
 #pragma unroll
     for (int kc = 0; kc < D / 16; kc++) {
-      bf16x8 k0 = *reinterpret_cast<const bf16x8*>(kp0 + kc * 16);
-      bf16x8 k1 = *reinterpret_cast<const bf16x8*>(kp1 + kc * 16);
+      bf16x8 k0 = kfrag(Ks, 0, kc);
+      bf16x8 k1 = kfrag(Ks, 1, kc);
       sacc[0] = mfma32(k0, qf[rs][kc], sacc[0]);
       sacc[1] = mfma32(k1, qf[rs][kc], sacc[1]);
     }
@@ -205,13 +250,11 @@ __global__ __launch_bounds__(256, MINB) void fwd_tile_kernel(NsaFwdTileParams p)
       const int nt = c >> 1, ch = c & 1;
       bf16x8 pf = pack8(sacc[nt][ch * 8 + 0], sacc[nt][ch * 8 + 1], sacc[nt][ch * 8 + 2], sacc[nt][ch * 8 + 3],
                         sacc[nt][ch * 8 + 4], sacc[nt][ch * 8 + 5], sacc[nt][ch * 8 + 6], sacc[nt][ch * 8 + 7]);
-      const int kb0 = nt * 32 + (2 * ch) * 8 + hl * 4;
-      const int kb1 = kb0 + 8;
+      const int kb16 = nt * 32 + ch * 16;  // the lane's rows: kb16 + hl*4 + (i16>>2) and 8 further
 #pragma unroll
       for (int dt = 0; dt < VD / 32; dt++) {
-        const int col = dt * 32 + (g16 & 1) * 16 + 4 * (i16 & 3);
-        bf16x4 v0 = lds_read_tr(&Vs[(kb0 + (i16 >> 2)) * VLD + col]);
-        bf16x4 v1 = lds_read_tr(&Vs[(kb1 + (i16 >> 2)) * VLD + col]);
+        bf16x4 v0 = vfrag(Vs, kb16, 0, dt);
+        bf16x4 v1 = vfrag(Vs, kb16, 1, dt);
         oacc[rs][dt] = mfma32(cat4(v0, v1), pf, oacc[rs][dt]);
       }
     }
@@ -229,18 +272,76 @@ __global__ __launch_bounds__(256, MINB) void fwd_tile_kernel(NsaFwdTileParams p)
       *reinterpret_cast<bf16x8*>(&Vs2[buf][(pc / VP) * VLD + (pc % VP) * 8]) = vreg[j];
     }
   };
+  // ASYNC staging: lane L of a wave's j-th load fills LDS piece j*256 + wave*64 + L (row = piece / chunks per row,
+  // position = piece % chunks per row), i.e. it fetches the chunk that the swizzle puts at that position
+  // per-lane byte offsets of its pieces from the first row of a tile (the same for every full tile)
+  int goffk[KJ], goffv[VJ];
+  if constexpr (ASYNC) {
+#pragma unroll
+    for (int j = 0; j < KJ; j++) {
+      const int pc = tid + j * 256, row = pc / KP;
+      goffk[j] = (int)((row * p.k_sr + ((pc % KP) ^ swz<KP>(row)) * 8) * 2);
+    }
+#pragma unroll
+    for (int j = 0; j < VJ; j++) {
+      const int pc = tid + j * 256, row = pc / VP;
+      goffv[j] = (int)((row * p.v_sr + ((pc % VP) ^ swz<VP>(row)) * 8) * 2);
+    }
+  }
+  auto stage_async = [&](int kt, int buf) {
+    int64_t row0;
+    if (PAGED) row0 = (int64_t)table[kt / p.page_size] * p.page_size + (kt % p.page_size);
+    else row0 = (int64_t)kbase + kt;
+    const int last = key_end - 1 - kt;  // >= 0; rows past it repeat it (masked)
+    const char* kb = reinterpret_cast<const char*>(p.k + row0 * p.k_sr + (int64_t)kh * p.k_sh);
+    const char* vb = reinterpret_cast<const char*>(p.v + row0 * p.v_sr + (int64_t)kh * p.v_sh);
+    if (last >= KT - 1) {  // wave-uniform
+#pragma unroll
+      for (int j = 0; j < KJ; j++)
+        __builtin_amdgcn_global_load_lds((nsa_gptr_t)(kb + goffk[j]),
+                                         (nsa_lptr_t)&Ks2[buf][(j * 256 + wave * 64) * 8], 16, 0, 0);
+#pragma unroll
+      for (int j = 0; j < VJ; j++)
+        __builtin_amdgcn_global_load_lds((nsa_gptr_t)(vb + goffv[j]),
+                                         (nsa_lptr_t)&Vs2[buf][(j * 256 + wave * 64) * 8], 16, 0, 0);
+    } else {
+#pragma unroll
+      for (int j = 0; j < KJ; j++) {
+        const int pc = tid + j * 256;
+        const int row = pc / KP, c = (pc % KP) ^ swz<KP>(row);
+        __builtin_amdgcn_global_load_lds((nsa_gptr_t)(kb + ((int64_t)min(row, last) * p.k_sr + c * 8) * 2),
+                                         (nsa_lptr_t)&Ks2[buf][(j * 256 + wave * 64) * 8], 16, 0, 0);
+      }
+#pragma unroll
+      for (int j = 0; j < VJ; j++) {
+        const int pc = tid + j * 256;
+        const int row = pc / VP, c = (pc % VP) ^ swz<VP>(row);
+        __builtin_amdgcn_global_load_lds((nsa_gptr_t)(vb + ((int64_t)min(row, last) * p.v_sr + c * 8) * 2),
+                                         (nsa_lptr_t)&Vs2[buf][(j * 256 + wave * 64) * 8], 16, 0, 0);
+      }
+    }
+  };
   if (key_begin < key_end) {
-    gload(key_begin);
-    stage(0);
-    if (key_begin + KT < key_end) gload(key_begin + KT);
+    if constexpr (ASYNC) {
+      stage_async(key_begin, 0);
+    } else {
+      gload(key_begin);
+      stage(0);
+      if (key_begin + KT < key_end) gload(key_begin + KT);
+    }
   }
 
   int buf = 0;
   for (int kt = key_begin; kt < key_end; kt += KT, buf ^= 1) {
+    if constexpr (ASYNC) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's pieces of tile kt have landed
     __syncthreads();  // tile kt is visible; nobody reads the other buffer (tile kt - KT) any more
     if (kt + KT < key_end) {
-      stage(buf ^ 1);
-      if (kt + 2 * KT < key_end) gload(kt + 2 * KT);
+      if constexpr (ASYNC) {
+        stage_async(kt + KT, buf ^ 1);
+      } else {
+        stage(buf ^ 1);
+        if (kt + 2 * KT < key_end) gload(kt + 2 * KT);
+      }
     }
     if (!wave_active) continue;
 
@@ -284,16 +385,24 @@ __global__ __launch_bounds__(256, MINB) void fwd_tile_kernel(NsaFwdTileParams p)
 template <int D, int VD, int MODE, bool PAGED>
 int launch_fwd_tile(const NsaFwdTileParams& p, int B, int max_q_len, hipStream_t stream) {
   if (B <= 0 || max_q_len <= 0) return NSA_OK;
-  static const int variant = nsa_tuning_knob("NSA_FWD_VARIANT", 1);
-  if (variant == 1) {
-    dim3 grid(cdiv_i(max_q_len * p.G, 128), B, p.KH);
-    fwd_tile_kernel<D, VD, MODE, PAGED, 1, 2><<<grid, 256, 0, stream>>>(p);
-  } else if (variant == 2) {
+  // 0 (default): direct-to-LDS staging for the compressed branch with power-of-two head dims (4.5 % faster there;
+  // the window branch, with its short key loops, and d=192, whose swizzled addresses cost registers, are faster with
+  // register staging); 1..4 force one variant for experiments
+  static const int variant = nsa_tuning_knob("NSA_FWD_VARIANT", 0);
+  constexpr bool pow2 = (D == 64 || D == 128) && (VD == 64 || VD == 128);
+  const bool async = variant == 4 || (variant == 0 && MODE == MODE_CMP && pow2);
+  if (variant == 2) {
     dim3 grid(cdiv_i(max_q_len * p.G, 256), B, p.KH);
-    fwd_tile_kernel<D, VD, MODE, PAGED, 2, 1><<<grid, 256, 0, stream>>>(p);
+    fwd_tile_kernel<D, VD, MODE, PAGED, 2, 1, false><<<grid, 256, 0, stream>>>(p);
+  } else if (variant == 3) {
+    dim3 grid(cdiv_i(max_q_len * p.G, 128), B, p.KH);
+    fwd_tile_kernel<D, VD, MODE, PAGED, 1, 1, false><<<grid, 256, 0, stream>>>(p);
+  } else if (async) {
+    dim3 grid(cdiv_i(max_q_len * p.G, 128), B, p.KH);
+    fwd_tile_kernel<D, VD, MODE, PAGED, 1, 2, true><<<grid, 256, 0, stream>>>(p);
   } else {
     dim3 grid(cdiv_i(max_q_len * p.G, 128), B, p.KH);
-    fwd_tile_kernel<D, VD, MODE, PAGED, 1, 1><<<grid, 256, 0, stream>>>(p);
+    fwd_tile_kernel<D, VD, MODE, PAGED, 1, 2, false><<<grid, 256, 0, stream>>>(p);
   }
   return nsa_check_launch("fwd_tile_kernel");
 }
