@@ -63,8 +63,8 @@ def test_prefill_with_cached_prefix(device, QH, KH, D):
 def test_chunked_prefill_equals_one_shot(device):
     from flash_nsa import nsa_prefill
     QH, KH, D = 16, 1, 128
-    ctx = [1000, 777]
-    kw = dict(top_n=6, window_size=100, fixed_y_maxlen=256, fixed_num_slc_blocks=32)
+    ctx = [5000, 777]
+    kw = dict(top_n=6, window_size=100, fixed_y_maxlen=512, fixed_num_slc_blocks=128)
     q_all = [randn_bf16(L, QH, D, seed=10 + i) for i, L in enumerate(ctx)]
     w_all = [randn_bf16(L, QH, 3, seed=20 + i) for i, L in enumerate(ctx)]
 
@@ -96,6 +96,15 @@ def test_chunked_prefill_equals_one_shot(device):
     for b in range(len(ctx)):
         assert torch.equal(one[b], four[b]), f"request {b}: chunked prefill differs from one-shot"
     assert torch.equal(d1["k"], d4["k"]) and torch.equal(d1["v"], d4["v"]), "pooled cache rows differ"
+    # the paged block selector working segment by segment (as it does for contexts whose score rows do not fit LDS)
+    import os
+    os.environ["NSA_TOPK_SEG_BLOCKS"] = "32"
+    try:
+        seg, _ = run(4)
+    finally:
+        os.environ.pop("NSA_TOPK_SEG_BLOCKS", None)
+    for b in range(len(ctx)):
+        assert torch.equal(one[b], seg[b]), f"request {b}: segmented block selection changed the prefill"
 
 
 @pytest.mark.parametrize("QH,KH,D", [(16, 1, 128), (64, 4, 128)])
