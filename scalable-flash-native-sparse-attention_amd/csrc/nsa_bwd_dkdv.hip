@@ -505,12 +505,9 @@ int launch(const NsaBwdTileParams& p0, int mode, int B, int max_q_len, int max_k
     if (kb_cmp == 2) {
       dim3 grid(cdiv_i(max_k_len, 256), B, p.KH);
       bwd_dkdv_kernel<D, VD, MODE_SWA, 4, 2><<<grid, 256, 0, stream>>>(p);
-    } else if ((int64_t)cdiv_i(max_k_len, 128) * B * p.KH >= 512) {
+    } else {
       dim3 grid(cdiv_i(max_k_len, 128), B, p.KH);
       bwd_dkdv_kernel<D, VD, MODE_SWA, 4, 1><<<grid, 256, 0, stream>>>(p);
-    } else {  // short batches: 64 keys per workgroup, twice the workgroups
-      dim3 grid(cdiv_i(max_k_len, 64), B, p.KH);
-      bwd_dkdv_kernel<D, VD, MODE_SWA, 2, 1><<<grid, 128, 0, stream>>>(p);
     }
   } else {
     if (n_items_bound <= 0) return NSA_OK;
