@@ -231,12 +231,34 @@ int nsa_cmp_attn_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void*
   rc = check_nsa_sizes("cmp_attn_bwd_dkdv", kernel_size, stride, 0);
   if (rc) return rc;
   if (q_chunk_tokens <= 0) {
-    // Largest power of two in [128, 2048] that still cuts the launch into about four workgroups per CU:
-    // (128-key tiles) x (query chunks that see them, about half) x kv heads x sequences.
-    const int64_t tiles = (y_maxlen + 127) / 128;
-    const int64_t want = (int64_t)B * KH * tiles * x_maxlen / (2 * 1024);
-    q_chunk_tokens = 128;
-    while (q_chunk_tokens < 2048 && q_chunk_tokens * 2 <= want) q_chunk_tokens *= 2;
+    // The kernel keeps one workgroup per CU, so a launch takes about
+    //   ceil(workgroups / CUs) * (fixed cost of a workgroup + its 64-row tiles * time per tile);
+    // a workgroup is one (128-key tile, query chunk that sees it, kv head, sequence).  The chunk (a power of two in
+    // [128, 2048]) that minimises this for the longest sequence is taken.  The constants (90 us, 2.4 us per tile
+    // at d = dv = 128) were fitted on MI355X to sweeps over one to eight sequences of 4K to 64K tokens, where the
+    // choice is within 1 % of the best chunk.
+    static int num_cus = 0;
+    if (num_cus == 0) {
+      int dev = 0;
+      hipDeviceProp_t prop;
+      num_cus = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+                 prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
+    }
+    const double tile_us = 2.4 * (D + VD) / 256.0, fixed_us = 90.0;
+    const int G = QH / KH;
+    double best = 0.0;
+    for (int chunk = 128; chunk <= 2048; chunk *= 2) {
+      const int64_t nch = (x_maxlen + chunk - 1) / chunk;
+      int64_t wgs = 0;
+      for (int64_t kt = 0; kt * 128 < y_maxlen; kt++) {
+        const int64_t fc = ((int64_t)stride * kt * 128 + kernel_size - 1) / chunk;
+        wgs += nch - (fc < nch ? fc : nch);
+      }
+      wgs *= (int64_t)B * KH;
+      const double rounds = (double)((wgs + num_cus - 1) / num_cus);
+      const double cost = rounds * (fixed_us + (double)chunk * G / 64.0 * tile_us);
+      if (q_chunk_tokens <= 0 || cost < best) { best = cost; q_chunk_tokens = chunk; }
+    }
   }
   BwdCommon c{q, q_st, q_sh, ck, ck_sr, ck_sh, cv, cv_sr, cv_sh, dO, do_st, do_sh, lse, lse_st, lse_sh, delta,
               delta_st, delta_sh};
