@@ -28,12 +28,17 @@ def test_c2_prefix_consistency_and_oracle_slice(device):
     qg = q.clone().requires_grad_()
     cu = torch.tensor([0, T], dtype=torch.int32, device=device)
     out = core(qg, k, v, w, cu)
-    out.backward(dev_randn((T, QH, D), 9, device))
+    do = dev_randn((T, QH, D), 9, device)
+    out.backward(do)
     assert torch.isfinite(out).all() and torch.isfinite(qg.grad).all()
-    with torch.no_grad():
-        short = core(q[:P].contiguous(), k[:P].contiguous(), v[:P].contiguous(), w[:P].contiguous(),
-                     torch.tensor([0, P], dtype=torch.int32, device=device))
+    qs_ = q[:P].clone().requires_grad_()
+    short = core(qs_, k[:P].contiguous(), v[:P].contiguous(), w[:P].contiguous(),
+                 torch.tensor([0, P], dtype=torch.int32, device=device))
     assert torch.equal(out[:P], short), "rows of the prefix changed when later tokens were appended"
+    # dq of a row depends on the keys at or before it only: the same property for the backward
+    short.backward(do[:P].contiguous())
+    assert torch.equal(qg.grad[:P], qs_.grad), "dq of the prefix changed when later tokens were appended"
+    short = short.detach()
     # oracle on a slice: first 1024 tokens, the 16 q-heads of kv head 0, device's own block selection
     n = 1024
     from flash_nsa import NSAHelper
@@ -49,9 +54,12 @@ def test_c2_prefix_consistency_and_oracle_slice(device):
         _, lse = cmp_attn_fwd(qs, ck, cv)
         topk, _ = slc_topk_indices(qs, ck, lse)
     assert torch.equal(o16, out[:n, :16]), "a kv group computed alone differs from the same group inside 4 groups"
-    ref = O.nsa_forward(qs.float().cpu(), ks.float().cpu(), vs.float().cpu(), ws.float().cpu(), [0, n],
+    qr = qs.float().cpu().requires_grad_()
+    ref = O.nsa_forward(qr, ks.float().cpu(), vs.float().cpu(), ws.float().cpu(), [0, n],
                         topk=topk.cpu(), round_dtype=torch.bfloat16)
     assert_close(o16, ref, "o (slice of the 64K run)")
+    ref.backward(do[:n, :16].float().cpu())
+    assert_close(qg.grad[:n, :16], qr.grad, "dq (slice of the 64K run)")
 
 
 def test_c2_recompute_and_learned_compression_full_size(device):
