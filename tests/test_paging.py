@@ -105,3 +105,19 @@ def test_oracle_store_kvcache_is_an_indexed_row_copy():
     want_k = torch.zeros(12, 2, 8).index_copy_(0, torch.tensor([7, 0, 11, 3]), key[[0, 2, 3, 4]])
     want_v = torch.zeros(12, 2, 4).index_copy_(0, torch.tensor([7, 0, 11, 3]), val[[0, 2, 3, 4]])
     assert torch.equal(kc.view(12, 2, 8), want_k) and torch.equal(vc.view(12, 2, 4), want_v)
+
+
+def test_decode_picks_parts_only_for_small_batches_of_long_contexts():
+    """auto_cmp_splits: one workgroup per (request, kv head) while those pairs fill the GPU or the contexts are short;
+    otherwise a power of two of parts, at most 8, that brings the workgroup count back to about the CU count."""
+    from flash_nsa.inference import auto_cmp_splits
+    assert auto_cmp_splits(64, 4, 4096) == 1          # 256 pairs: the GPU is full
+    assert auto_cmp_splits(33, 4, 4096) == 1          # more than half full
+    assert auto_cmp_splits(32, 4, 4096) == 2
+    assert auto_cmp_splits(16, 4, 8192) == 4
+    assert auto_cmp_splits(8, 4, 8192) == 8
+    assert auto_cmp_splits(1, 1, 8192) == 8           # never more than 8
+    assert auto_cmp_splits(1, 1, 2048) == 1           # up to 32K tokens per context: not worth two launches
+    for b in range(1, 80):
+        n = auto_cmp_splits(b, 4, 4096)
+        assert n in (1, 2, 4, 8) and (n == 1 or b * 4 * n <= 256)
