@@ -1,7 +1,7 @@
 // dQ of selected-block attention: one wave per (query token, kv head), 16 q-heads as the MFMA N dimension.
 //   S^T = K Q^T,  P^T = exp2(S^T*c - lse),  dP^T = V dO^T,  dS^T = P^T o (dP^T - delta),  dQ^T += K^T dS^T
-// K and V rows are staged row-major in wave-private LDS regions (K is read both as row fragments and, transposed,
-// through ds_read_b64_tr_b16; V as row fragments).
+// K rows are staged row-major in a wave-private LDS region (K is read both as row fragments and, transposed,
+// through ds_read_b64_tr_b16); V is only read as row fragments and comes from global memory in that layout.
 // Upstream: flash_nsa/ops/select_attn.py:336-437 (_dq_kernel).
 #include "nsa_common.h"
 #include "nsa_api_internal.h"
@@ -14,16 +14,13 @@ __global__ __launch_bounds__(256, 2) void slc_dq_kernel(NsaSlcBwdDqParams p) {
   // registers while unit u is computed out of wave-private LDS.
   constexpr int UK = 32;
   constexpr int KLD = D + NSA_LDS_PAD;
-  constexpr int VLD = VD + NSA_LDS_PAD;
   constexpr int KC = D / 32, VC = VD / 32;
-  constexpr int KJ = (UK * (D / 8)) / 64, VJ = (UK * (VD / 8)) / 64;
+  constexpr int KJ = (UK * (D / 8)) / 64, VJ = 2 * VC;
   __shared__ __attribute__((aligned(16))) bf16_t Ks_all[4 * UK * KLD];
-  __shared__ __attribute__((aligned(16))) bf16_t Vs_all[4 * UK * VLD];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   bf16_t* Ks = Ks_all + wave * UK * KLD;
-  bf16_t* Vs = Vs_all + wave * UK * VLD;
   const int l16 = lane & 15;
   const int kq = lane >> 4;
   const int b = blockIdx.y;
@@ -79,11 +76,10 @@ __global__ __launch_bounds__(256, 2) void slc_dq_kernel(NsaSlcBwdDqParams p) {
     int pc = lane + j * 64;
     koff[j] = (int64_t)(pc / (D / 8)) * p.k_sr + (pc % (D / 8)) * 8;
   }
+  // V is only needed as row fragments (dP^T = V dO^T): its rows are loaded straight in MFMA operand layout, lane
+  // (l16, kq) taking 16 bytes of row jt*16 + l16 at column kq*8 + kc*32 (16 rows x 64 contiguous bytes per load)
 #pragma unroll
-  for (int j = 0; j < VJ; j++) {
-    int pc = lane + j * 64;
-    voff[j] = (int64_t)(pc / (VD / 8)) * p.v_sr + (pc % (VD / 8)) * 8;
-  }
+  for (int j = 0; j < VJ; j++) voff[j] = (int64_t)((j / VC) * 16 + l16) * p.v_sr + kq * 8 + (j % VC) * 32;
   auto issue = [&](int key0, bf16x8 (&kr)[KJ], bf16x8 (&vr)[VJ]) {
     if (key0 < 0) return;
     const int64_t row0 = (int64_t)x0 + key0;
@@ -102,10 +98,8 @@ __global__ __launch_bounds__(256, 2) void slc_dq_kernel(NsaSlcBwdDqParams p) {
         kr[j] = ld_global_b128(kb + (int64_t)min(pc / (D / 8), kmax) * p.k_sr + (pc % (D / 8)) * 8);
       }
 #pragma unroll
-      for (int j = 0; j < VJ; j++) {
-        int pc = lane + j * 64;
-        vr[j] = ld_global_b128(vb + (int64_t)min(pc / (VD / 8), kmax) * p.v_sr + (pc % (VD / 8)) * 8);
-      }
+      for (int j = 0; j < VJ; j++)
+        vr[j] = ld_global_b128(vb + (int64_t)min((j / VC) * 16 + l16, kmax) * p.v_sr + kq * 8 + (j % VC) * 32);
     }
   };
   auto compute = [&](int key0, bf16x8 (&kr)[KJ], bf16x8 (&vr)[VJ]) {
@@ -114,11 +108,6 @@ __global__ __launch_bounds__(256, 2) void slc_dq_kernel(NsaSlcBwdDqParams p) {
     for (int j = 0; j < KJ; j++) {
       int pc = lane + j * 64;
       *reinterpret_cast<bf16x8*>(&Ks[(pc / (D / 8)) * KLD + (pc % (D / 8)) * 8]) = kr[j];
-    }
-#pragma unroll
-    for (int j = 0; j < VJ; j++) {
-      int pc = lane + j * 64;
-      *reinterpret_cast<bf16x8*>(&Vs[(pc / (VD / 8)) * VLD + (pc % (VD / 8)) * 8]) = vr[j];
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -132,10 +121,8 @@ __global__ __launch_bounds__(256, 2) void slc_dq_kernel(NsaSlcBwdDqParams p) {
 #pragma unroll
       for (int kc = 0; kc < KC; kc++)
         sacc[jt] = mfma16(*reinterpret_cast<const bf16x8*>(kp + kc * 32), qf[kc], sacc[jt]);
-      const bf16_t* vp = &Vs[(jt * 16 + l16) * VLD + kq * 8];
 #pragma unroll
-      for (int kc = 0; kc < VC; kc++)
-        pacc[jt] = mfma16(*reinterpret_cast<const bf16x8*>(vp + kc * 32), dof[kc], pacc[jt]);
+      for (int kc = 0; kc < VC; kc++) pacc[jt] = mfma16(vr[jt * VC + kc], dof[kc], pacc[jt]);
     }
     const int kmax = key_last - key0;
 #pragma unroll
