@@ -107,7 +107,7 @@ def staged_step(timer, q, k, v, w, wv, do, sm_scale):
     R("combine_fwd", lambda: combine_fwd(cmp_o, slc_o, swa_o, w))
 
     dcmp_o, dslc_o, dswa_o, dw, delta = R("combine_bwd", lambda: combine_bwd(cmp_o, slc_o, swa_o, w, do, True))
-    dq = torch.empty(q.shape, device=q.device, dtype=torch.float32)
+    dq = torch.zeros(q.shape, device=q.device, dtype=torch.float32)
     T, QH, D = q.shape
     _, KH, VD = v.shape
 
@@ -119,7 +119,8 @@ def staged_step(timer, q, k, v, w, wv, do, sm_scale):
     dk = torch.empty(T, KH, D, device=q.device, dtype=torch.float32)
     dv = torch.empty(T, KH, VD, device=q.device, dtype=torch.float32)
     cs = common(k, v, swa_lse, swa_lse.stride(0), swa_lse.stride(1), delta[2], dswa_o)
-    R("swa_dq", lambda: _lib.call("nsa_swa_bwd_dq", *cs, dq.data_ptr(), dq.stride(0), dq.stride(1), 1,
+    # dq modes as in the fused backward: the selected branch stores (1), the window branch adds (2)
+    R("swa_dq", lambda: _lib.call("nsa_swa_bwd_dq", *cs, dq.data_ptr(), dq.stride(0), dq.stride(1), 2,
                                   H.x_cu_seqlens.data_ptr(), H.batch, H.x_maxlen, QH, KH, D, VD, H.window_size,
                                   sm_scale, _lib.stream_ptr()))
     R("swa_dkdv", lambda: _lib.call("nsa_swa_bwd_dkdv", *cs, dk.data_ptr(), dk.stride(0), dk.stride(1),
@@ -127,7 +128,7 @@ def staged_step(timer, q, k, v, w, wv, do, sm_scale):
                                     H.x_maxlen, QH, KH, D, VD, H.window_size, sm_scale, _lib.stream_ptr()))
     cl = common(k, v, slc_lse, slc_lse.stride(0), slc_lse.stride(1), delta[1], dslc_o)
     R("slc_dq", lambda: _lib.call("nsa_slc_attn_bwd_dq", *cl, topk.data_ptr(), topk.stride(0), topk.stride(1),
-                                  dq.data_ptr(), dq.stride(0), dq.stride(1), 2, H.x_cu_seqlens.data_ptr(), H.batch,
+                                  dq.data_ptr(), dq.stride(0), dq.stride(1), 1, H.x_cu_seqlens.data_ptr(), H.batch,
                                   H.x_maxlen, QH, KH, D, VD, H.block_size, topk.size(-1), sm_scale, _lib.stream_ptr()))
     bind = R("inverse_index", lambda: get_bind_from_find(topk))
     R("slc_dkdv", lambda: _lib.call("nsa_slc_attn_bwd_dkdv", *cl, dk.data_ptr(), dk.stride(0), dk.stride(1),

@@ -140,10 +140,10 @@ class NSAFunction(torch.autograd.Function):
             main, side = torch.cuda.current_stream(), _side_stream(q.device)
             side.wait_stream(main)
             with torch.cuda.stream(side):
-                # dq chain: the window branch stores, the selected branch adds, the compressed branch adds and
-                # writes q's dtype
-                swa_bwd(q, k, v, swa_o, swa_lse, dswa_o, delta=delta[2], dq=_store_into(dq32), parts="dq", **kw)
-                slc_attn_bwd(q, k, v, topk, slc_o, slc_lse, dslc_o, dq32, delta=delta[1], parts="dq", **kw)
+                # dq chain: the selected branch (memory bound) stores, the window branch (matrix bound, with
+                # bandwidth to spare for the read-modify-write) adds, the compressed branch adds and writes q's dtype
+                slc_attn_bwd(q, k, v, topk, slc_o, slc_lse, dslc_o, _store_into(dq32), delta=delta[1], parts="dq", **kw)
+                swa_bwd(q, k, v, swa_o, swa_lse, dswa_o, delta=delta[2], dq=dq32, parts="dq", **kw)
                 dq, _, _ = cmp_attn_bwd(q, cmp_k, cmp_v, cmp_o, cmp_lse, dcmp_o, dq32, delta=delta[0],
                                         finalize_dq=True, parts="dq", **kw)
                 dq.record_stream(main)
@@ -154,10 +154,11 @@ class NSAFunction(torch.autograd.Function):
             _, dcmp_k, dcmp_v = cmp_attn_bwd(q, cmp_k, cmp_v, cmp_o, cmp_lse, dcmp_o, delta=delta[0], parts="dkdv",
                                              **kw)
         else:
-            # window branch first: it writes every element of dq / dk / dv, the other branches add to them
-            _, dk, dv = swa_bwd(q, k, v, swa_o, swa_lse, dswa_o, delta=delta[2], dq=_store_into(dq32), dkv_fp32=True,
-                                **kw)
-            slc_attn_bwd(q, k, v, topk, slc_o, slc_lse, dslc_o, dq32, dk, dv, delta=delta[1], **kw)
+            # the selected branch stores dq, the window branch adds to it and writes every element of dk / dv, to
+            # which the selected branch then adds
+            slc_attn_bwd(q, k, v, topk, slc_o, slc_lse, dslc_o, _store_into(dq32), delta=delta[1], parts="dq", **kw)
+            _, dk, dv = swa_bwd(q, k, v, swa_o, swa_lse, dswa_o, delta=delta[2], dq=dq32, dkv_fp32=True, **kw)
+            slc_attn_bwd(q, k, v, topk, slc_o, slc_lse, dslc_o, None, dk, dv, delta=delta[1], parts="dkdv", **kw)
             dq, dcmp_k, dcmp_v = cmp_attn_bwd(q, cmp_k, cmp_v, cmp_o, cmp_lse, dcmp_o, dq32, delta=delta[0],
                                               finalize_dq=True, **kw)
         _, dwk = compress_kv_bwd(k, cmp_k_weight, win_k, hid_k, dcmp_k, dk, k_method, helper)
