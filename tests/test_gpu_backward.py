@@ -163,6 +163,8 @@ def test_combine_bwd(device):
     ([400, 330], 16, 2, 128, ("mean", "mean")),       # groups of 8
     ([400, 330], 6, 3, 64, ("mean", "mean")),         # groups of 2
     ([400, 330], 12, 4, 64, ("mean", "mean")),        # groups of 3 (not a power of two)
+    # 48 ragged sequences, some empty or shorter than one compression window
+    ([(37 * i * i + 11 * i) % 257 for i in range(48)], 16, 2, 128, ("mean", "sigmoid-mul")),
 ])
 def test_nsa_core_fwd_bwd(device, core, lens, QH, KH, D, methods):
     """HFNSACore and NSACore against the composed oracle (upstream only compares them with each other)."""
@@ -201,7 +203,13 @@ def test_nsa_core_fwd_bwd(device, core, lens, QH, KH, D, methods):
     ro = O.nsa_forward(qr, kr, vr, wr, cu, ocfg, wk=wkr, wv=wvr, topk=topk.cpu())
     ro.backward(do.float())
     assert_close(out, ro, "o")
-    assert_close(qd.grad, qr.grad, "dq")
+    # The first tokens of a sequence attend one to four keys: their probabilities are near one-hot, dP and delta are
+    # both of order |dO||V| and cancel (at position 0 exactly: the fp32 dq is 0), and delta is formed from the bf16
+    # rounded output, as upstream forms it.  The rounding of that output, not the kernels' arithmetic, sets the
+    # error there (up to 0.035 on values of 0.5 in the many-sequence case), so those rows get a wider absolute bound.
+    early = torch.cat([torch.arange(n) for n in lens]) < 4
+    assert_close(qd.grad[~early.to(device)], qr.grad[~early], "dq")
+    assert_close(qd.grad[early.to(device)], qr.grad[early], "dq of the first four tokens of a sequence", atol=5e-2)
     assert_close(kd.grad, kr.grad, "dk", row_scale=True)
     assert_close(vd.grad, vr.grad, "dv", row_scale=True)
     assert_close(wd.grad, wr.grad, "dw", atol=5e-2)
