@@ -219,6 +219,54 @@ def test_nsa_core_fwd_bwd(device, core, lens, QH, KH, D, methods):
         assert_close(wv.grad, wvr.grad, "dWv", atol=5e-2, rtol=2e-2, row_scale=True)
 
 
+@pytest.mark.parametrize("hp", [
+    dict(kernel_size=64, stride=32, block_size=128, top_n=4, window_size=256),
+    dict(kernel_size=64, stride=16, block_size=64, top_n=5, window_size=100),
+    dict(kernel_size=32, stride=8, block_size=64, top_n=16, window_size=512),
+    dict(kernel_size=16, stride=16, block_size=64, top_n=3, window_size=1, num_init_blocks=0, num_local_blocks=1),
+    dict(kernel_size=32, stride=16, block_size=64, top_n=8, window_size=64, num_init_blocks=2, num_local_blocks=3),
+])
+def test_nsa_core_other_hyperparameters(device, hp):
+    """Compression window / stride, selection block, top-n, forced blocks and window other than the defaults
+    (upstream NSAHelper.set_hyperparameters, flash_nsa/utils.py:180-214): selection identical to the oracle's on the
+    device's compressed keys, forward and backward against the composed oracle."""
+    from flash_nsa import NSAConfig, NSACore, NSAHelper
+    from flash_nsa.ops.compress_attn import cmp_attn_fwd
+    from flash_nsa.ops.topk import slc_topk_indices
+    from flash_nsa.modules.megatron_level_nsa import compress_kv_fwd
+    lens, QH, KH, D = [1500, 700, 90], 8, 2, 128
+    cu = make_cu(lens)
+    T = int(cu[-1])
+    q, k, v, w = make_qkvw(T, QH, KH, D, seed=71)
+    do = randn_bf16(T, QH, D, seed=76)
+    try:
+        mod = NSACore(NSAConfig(head_dim=D, num_heads=QH, num_kv_heads=KH, **hp)).to(device=device, dtype=torch.bfloat16)
+        qd, kd, vd, wd = [t.to(device).requires_grad_() for t in (q, k, v, w)]
+        out = mod(qd, kd, vd, wd, cu.to(device))
+        out.backward(do.to(device))
+        with torch.no_grad():
+            ck = compress_kv_fwd(kd.detach(), None, "mean")[2]
+            cv = compress_kv_fwd(vd.detach(), None, "mean")[2]
+            _, lse = cmp_attn_fwd(qd.detach(), ck, cv)
+            topk, _ = slc_topk_indices(qd.detach(), ck, lse)
+    finally:
+        NSAHelper.set_hyperparameters()
+    ocfg = O.OracleConfig(**hp)
+    rt, imps = O.slc_topk(q.float(), ck.float().cpu(), None, cu, ocfg, return_importance=True)
+    n_rows, n_diff, n_bad = O.topk_mismatch_report(topk.cpu(), rt, imps, cu, ocfg.block_size, ocfg.top_n, tie_tol=1e-3)
+    assert n_bad == 0 and n_diff <= max(1, n_rows // 200), (n_rows, n_diff, n_bad)
+    qr, kr, vr, wr = leaf(q), leaf(k), leaf(v), leaf(w)
+    ro = O.nsa_forward(qr, kr, vr, wr, cu, ocfg, topk=topk.cpu())
+    ro.backward(do.float())
+    assert_close(out, ro, "o")
+    early = torch.cat([torch.arange(n) for n in lens]) < 4  # see test_nsa_core_fwd_bwd
+    assert_close(qd.grad[~early.to(device)], qr.grad[~early], "dq")
+    assert_close(qd.grad[early.to(device)], qr.grad[early], "dq of the first four tokens of a sequence", atol=5e-2)
+    assert_close(kd.grad, kr.grad, "dk", row_scale=True)
+    assert_close(vd.grad, vr.grad, "dv", row_scale=True)
+    assert_close(wd.grad, wr.grad, "dw", atol=5e-2)
+
+
 def test_nsa_core_qk192_v128(device):
     """Dqk = 192, Dv = 128 (the head shape upstream's inference notebook exercises), forward + backward."""
     from flash_nsa import NSAConfig, NSACore
