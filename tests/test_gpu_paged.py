@@ -107,6 +107,51 @@ def test_chunked_prefill_equals_one_shot(device):
         assert torch.equal(one[b], seg[b]), f"request {b}: segmented block selection changed the prefill"
 
 
+@pytest.mark.parametrize("hp", [
+    dict(kernel_size=64, stride=32, block_size=128, top_n=4, window_size=256),
+    dict(kernel_size=64, stride=16, block_size=64, top_n=5, window_size=100),
+    dict(kernel_size=32, stride=8, block_size=64, top_n=16, window_size=512),
+    dict(kernel_size=16, stride=16, block_size=64, top_n=3, window_size=1, num_init_blocks=0, num_local_blocks=1),
+])
+def test_decode_other_hyperparameters_equals_training_row(device, hp):
+    """Decode with compression, block, top-n, forced-block and window settings other than the defaults: every
+    request's output is the last row of the training forward on its gathered sequence, and the one-launch path agrees
+    with the stage-by-stage one."""
+    from flash_nsa import nsa_decode, NSAConfig, NSACore, NSAHelper
+    from flash_nsa.inference import nsa_decode_staged
+    QH, KH, D = 16, 2, 128
+    ctx = [1024, 333, 130, 64, 65, 1, 777, 2000, 640]
+    ks, st = hp["kernel_size"], hp["stride"]
+    case = build_pool(ctx, KH, D, D, page=128, seed=7, kernel=ks, stride=st)
+    prepool(case, [L - 1 for L in ctx], kernel=ks, stride=st)
+    slots = decode_slot_mapping(case, kernel=ks, stride=st)
+    B = len(ctx)
+    q, w = randn_bf16(B, QH, D, seed=8), randn_bf16(B, QH, 3, seed=9)
+    d = to_dev(case, device)
+    ctx_t = torch.tensor(ctx, dtype=torch.int32).to(device)
+    try:
+        o = nsa_decode(q.to(device), d["k"], d["v"], w.to(device), ctx_t, d["bt"], slots.to(device), d["cbt"],
+                       fixed_y_maxlen=256, fixed_num_slc_blocks=32, **hp)
+        o2 = nsa_decode_staged(q.to(device), d["k"], d["v"], w.to(device), ctx_t, d["bt"], d["cbt"],
+                               fixed_y_maxlen=256, fixed_num_slc_blocks=32, **hp)
+        assert_close(o, o2, "one-launch vs stage-by-stage decode", atol=1e-2, rtol=1e-2)
+        core = NSACore(NSAConfig(head_dim=D, num_heads=QH, num_kv_heads=KH, **hp))
+        for b in range(B):
+            L = ctx[b]
+            ks_ = O.gather_rows(case["k"], case["bt"][b], L).to(device)
+            vs_ = O.gather_rows(case["v"], case["bt"][b], L).to(device)
+            qs = randn_bf16(L, QH, D, seed=100 + b)
+            qs[-1] = q[b]
+            ws = randn_bf16(L, QH, 3, seed=200 + b)
+            ws[-1] = w[b]
+            with torch.no_grad():
+                full = core(qs.to(device), ks_, vs_, ws.to(device),
+                            torch.tensor([0, L], dtype=torch.int32, device=device))
+            assert_close(o[b], full[-1], f"decode vs training row (request {b})", atol=1e-2, rtol=1e-2)
+    finally:
+        NSAHelper.set_hyperparameters()
+
+
 @pytest.mark.parametrize("QH,KH,D", [(16, 1, 128), (64, 4, 128)])
 def test_decode_vs_oracle_and_training_forward(device, QH, KH, D):
     from flash_nsa import nsa_decode, NSAConfig, NSACore
