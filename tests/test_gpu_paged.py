@@ -108,6 +108,48 @@ def test_chunked_prefill_equals_one_shot(device):
 
 
 @pytest.mark.parametrize("hp", [
+    dict(kernel_size=32, stride=16, block_size=64, top_n=16, window_size=512),
+    dict(kernel_size=64, stride=32, block_size=128, top_n=4, window_size=256),
+    dict(kernel_size=32, stride=8, block_size=64, top_n=16, window_size=512),
+    dict(kernel_size=16, stride=16, block_size=64, top_n=3, window_size=1, num_init_blocks=0, num_local_blocks=1),
+])
+def test_prefill_with_cached_prefix_equals_training_rows(device, hp):
+    """Prefill of new tokens behind a cached prefix, default and other compression / block / top-n / window settings:
+    the output rows are bit-equal to the same rows of the training forward on the gathered sequence."""
+    from flash_nsa import nsa_prefill, NSAConfig, NSACore, NSAHelper
+    QH, KH, D = 16, 2, 128
+    cached = [0, 37, 512, 1000, 130, 64]
+    new = [300, 200, 64, 17, 1, 700]
+    ctx = [c + n for c, n in zip(cached, new)]
+    ks, st = hp["kernel_size"], hp["stride"]
+    case = build_pool(ctx, KH, D, D, page=128, seed=3, kernel=ks, stride=st)
+    prepool(case, cached, kernel=ks, stride=st)
+    slots, ycu = prefill_slot_mapping(case, cached, kernel=ks, stride=st)
+    xcu = make_cu(new)
+    d = to_dev(case, device)
+    ctx_t = torch.tensor(ctx, dtype=torch.int32)
+    qs = [randn_bf16(L, QH, D, seed=100 + b) for b, L in enumerate(ctx)]
+    ws = [randn_bf16(L, QH, 3, seed=200 + b) for b, L in enumerate(ctx)]
+    q = torch.cat([qs[b][cached[b]:] for b in range(len(ctx))])
+    w = torch.cat([ws[b][cached[b]:] for b in range(len(ctx))])
+    try:
+        o = nsa_prefill(q.to(device), d["k"], d["v"], w.to(device), xcu.to(device), ycu.to(device), max(new),
+                        max(case["ys"]), ctx_t.to(device), d["bt"], slots.to(device), d["cbt"], fixed_y_maxlen=256,
+                        fixed_num_slc_blocks=32, **hp)
+        core = NSACore(NSAConfig(head_dim=D, num_heads=QH, num_kv_heads=KH, **hp))
+        for b, L in enumerate(ctx):
+            ks_ = O.gather_rows(case["k"], case["bt"][b], L).to(device)
+            vs_ = O.gather_rows(case["v"], case["bt"][b], L).to(device)
+            with torch.no_grad():
+                full = core(qs[b].to(device), ks_, vs_, ws[b].to(device),
+                            torch.tensor([0, L], dtype=torch.int32, device=device))
+            a, e = int(xcu[b]), int(xcu[b + 1])
+            assert torch.equal(o[a:e], full[cached[b]:]), f"request {b} (cached {cached[b]}, new {new[b]})"
+    finally:
+        NSAHelper.set_hyperparameters()
+
+
+@pytest.mark.parametrize("hp", [
     dict(kernel_size=64, stride=32, block_size=128, top_n=4, window_size=256),
     dict(kernel_size=64, stride=16, block_size=64, top_n=5, window_size=100),
     dict(kernel_size=32, stride=8, block_size=64, top_n=16, window_size=512),
