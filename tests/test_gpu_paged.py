@@ -116,13 +116,23 @@ def test_chunked_prefill_equals_one_shot(device):
 def test_prefill_with_cached_prefix_equals_training_rows(device, hp):
     """Prefill of new tokens behind a cached prefix, default and other compression / block / top-n / window settings:
     the output rows are bit-equal to the same rows of the training forward on the gathered sequence."""
+    _prefill_equals_training_rows(device, 16, 2, 128, 128, [0, 37, 512, 1000, 130, 64], [300, 200, 64, 17, 1, 700], hp)
+
+
+@pytest.mark.parametrize("QH,KH,D,page", [(16, 2, 128, 64), (16, 2, 128, 512), (6, 2, 128, 128), (5, 1, 128, 128),
+                                          (7, 7, 128, 128), (64, 2, 128, 128), (8, 2, 64, 256)])
+def test_prefill_head_groups_and_page_sizes_equal_training_rows(device, QH, KH, D, page):
+    """The same for pages of 64 / 256 / 512 rows (prefixes and chunks on and around page boundaries) and for groups of
+    1, 3, 5 and 32 q-heads per kv head."""
+    _prefill_equals_training_rows(device, QH, KH, D, page, [0, 37, 512, 1000, 130, 64, page, page - 1, 3 * page + 5],
+                                  [300, 200, 64, 17, 1, 700, page, page + 1, 2 * page], {})
+
+
+def _prefill_equals_training_rows(device, QH, KH, D, page, cached, new, hp):
     from flash_nsa import nsa_prefill, NSAConfig, NSACore, NSAHelper
-    QH, KH, D = 16, 2, 128
-    cached = [0, 37, 512, 1000, 130, 64]
-    new = [300, 200, 64, 17, 1, 700]
     ctx = [c + n for c, n in zip(cached, new)]
-    ks, st = hp["kernel_size"], hp["stride"]
-    case = build_pool(ctx, KH, D, D, page=128, seed=3, kernel=ks, stride=st)
+    ks, st = hp.get("kernel_size", 32), hp.get("stride", 16)
+    case = build_pool(ctx, KH, D, D, page=page, seed=3, kernel=ks, stride=st)
     prepool(case, cached, kernel=ks, stride=st)
     slots, ycu = prefill_slot_mapping(case, cached, kernel=ks, stride=st)
     xcu = make_cu(new)
@@ -134,8 +144,8 @@ def test_prefill_with_cached_prefix_equals_training_rows(device, hp):
     w = torch.cat([ws[b][cached[b]:] for b in range(len(ctx))])
     try:
         o = nsa_prefill(q.to(device), d["k"], d["v"], w.to(device), xcu.to(device), ycu.to(device), max(new),
-                        max(case["ys"]), ctx_t.to(device), d["bt"], slots.to(device), d["cbt"], fixed_y_maxlen=256,
-                        fixed_num_slc_blocks=32, **hp)
+                        max(case["ys"]), ctx_t.to(device), d["bt"], slots.to(device), d["cbt"], fixed_y_maxlen=512,
+                        fixed_num_slc_blocks=128, **hp)
         core = NSACore(NSAConfig(head_dim=D, num_heads=QH, num_kv_heads=KH, **hp))
         for b, L in enumerate(ctx):
             ks_ = O.gather_rows(case["k"], case["bt"][b], L).to(device)
