@@ -225,6 +225,9 @@ def test_nsa_core_fwd_bwd(device, core, lens, QH, KH, D, methods):
     dict(kernel_size=32, stride=8, block_size=64, top_n=16, window_size=512),
     dict(kernel_size=16, stride=16, block_size=64, top_n=3, window_size=1, num_init_blocks=0, num_local_blocks=1),
     dict(kernel_size=32, stride=16, block_size=64, top_n=8, window_size=64, num_init_blocks=2, num_local_blocks=3),
+    dict(top_n=64, window_size=64),                                   # more slots than most tokens have blocks
+    dict(top_n=1, num_init_blocks=0, num_local_blocks=1),             # the token's own block only
+    dict(top_n=2, num_init_blocks=1, num_local_blocks=1, window_size=0),  # window = the token itself
 ])
 def test_nsa_core_other_hyperparameters(device, hp):
     """Compression window / stride, selection block, top-n, forced blocks and window other than the defaults
