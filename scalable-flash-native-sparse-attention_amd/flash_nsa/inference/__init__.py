@@ -51,11 +51,13 @@ def nsa_prefill(q, k, v, w, x_cu_seqlens, y_cu_seqlens, x_maxlen, y_maxlen, cont
 
 def auto_cmp_splits(batch, num_kv_heads, fixed_y_maxlen, num_cus=256):
     """Parts the compressed branch of a decode step is cut into per (request, kv head).  One workgroup per pair
-    fills the GPU from about one pair per CU on; a small batch of long contexts (>= 2048 compressed rows, i.e. 32K
-    tokens) is cut so that there are again about num_cus workgroups (measured on MI355X, 4 kv heads: 32 requests of
-    64K tokens 153 -> 117 us with 2 parts, 16 requests of 128K tokens 222 -> 118 us with 4)."""
+    fills the GPU from about one pair per CU on; a small batch of contexts of 16K tokens or more (>= 1024 compressed
+    rows of capacity) is cut so that there are again about num_cus workgroups (measured on MI355X, 4 kv heads: 32
+    requests of 64K tokens 153 -> 117 us with 2 parts, 16 requests of 128K tokens 222 -> 118 us with 4, one request of
+    32K tokens 56 -> 46 us with 8; when the actual contexts are much shorter than the capacity the second launch costs
+    1-2 us)."""
     pairs = batch * num_kv_heads
-    if fixed_y_maxlen <= 2048 or pairs * 2 > num_cus:
+    if fixed_y_maxlen < 1024 or pairs * 2 > num_cus:
         return 1
     n = 2
     while n < 8 and pairs * n * 2 <= num_cus:

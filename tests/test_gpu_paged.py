@@ -535,7 +535,7 @@ def test_decode_small_batch_long_context_takes_the_split_path(device):
     dims the split kernels are not built for (192/128) are not routed there."""
     from flash_nsa import nsa_decode
     from flash_nsa.inference import auto_cmp_splits, decode_cmp_topk, decode_slc_swa_combine
-    assert auto_cmp_splits(2, 4, 4096) == 8 and auto_cmp_splits(64, 4, 4096) == 1 and auto_cmp_splits(2, 4, 2048) == 1
+    assert auto_cmp_splits(2, 4, 4096) == 8 and auto_cmp_splits(64, 4, 4096) == 1 and auto_cmp_splits(2, 4, 512) == 1
     QH, KH, D = 64, 4, 128
     ctx = [40000, 33333]
     case = build_pool(ctx, KH, D, D, page=256, seed=61)

@@ -108,8 +108,9 @@ def test_oracle_store_kvcache_is_an_indexed_row_copy():
 
 
 def test_decode_picks_parts_only_for_small_batches_of_long_contexts():
-    """auto_cmp_splits: one workgroup per (request, kv head) while those pairs fill the GPU or the contexts are short;
-    otherwise a power of two of parts, at most 8, that brings the workgroup count back to about the CU count."""
+    """auto_cmp_splits: one workgroup per (request, kv head) while those pairs fill the GPU or the capacity is below
+    16K tokens; otherwise a power of two of parts, at most 8, that brings the workgroup count back to about the CU
+    count."""
     from flash_nsa.inference import auto_cmp_splits
     assert auto_cmp_splits(64, 4, 4096) == 1          # 256 pairs: the GPU is full
     assert auto_cmp_splits(33, 4, 4096) == 1          # more than half full
@@ -117,7 +118,8 @@ def test_decode_picks_parts_only_for_small_batches_of_long_contexts():
     assert auto_cmp_splits(16, 4, 8192) == 4
     assert auto_cmp_splits(8, 4, 8192) == 8
     assert auto_cmp_splits(1, 1, 8192) == 8           # never more than 8
-    assert auto_cmp_splits(1, 1, 2048) == 1           # up to 32K tokens per context: not worth two launches
+    assert auto_cmp_splits(1, 1, 2048) == 8           # 32K tokens of capacity: worth the second launch
+    assert auto_cmp_splits(1, 1, 1000) == 1           # below 16K tokens of capacity: one launch
     for b in range(1, 80):
         n = auto_cmp_splits(b, 4, 4096)
         assert n in (1, 2, 4, 8) and (n == 1 or b * 4 * n <= 256)
