@@ -253,8 +253,9 @@ int nsa_decode_cmp_split(const void* q, int64_t q_st, int64_t q_sh, const void* 
 /* The decode step of flash_nsa/inference/__init__.py:207-257 for small batches of long contexts, in two launches:
  * (1) the compressed branch cut into nsplit key-interleaved parts per (request, kv head) -- partial (m, l, o) and the
  * un-normalised fp16 probabilities of every compressed key go to scratch; (2) per (request, kv head): merge of the
- * parts, block scores, selection, selected-block + window attention, gated combine.  The pooled row of the newest
- * compressed key must be in the pool (nsa_paged_pool_decode).  Scratch, all caller-allocated, contents undefined:
+ * parts, block scores, selection, selected-block + window attention, gated combine.  cmp_slot_mapping [B] (-1: no
+ * compressed row completes at this step) makes launch (1) pool the newest compressed row, as nsa_paged_pool_decode
+ * would; null: the row must be in the pool already.  Scratch, all caller-allocated, contents undefined:
  *   sp_m, sp_l [B,KH,nsplit,16] fp32; sp_o [B,KH,nsplit,16,VD] fp32;
  *   sp_keep_p [B,KH,Y/32,16,32] fp16 and sp_keep_m [B,KH,Y/32,16] fp32 with Y = fixed_y_maxlen rounded up to 32.
  * cmp_o / slc_o / swa_o / lse / topk are optional outputs (null: not written).
@@ -265,11 +266,11 @@ int nsa_decode_split(const void* q, int64_t q_st, int64_t q_sh, const void* k_ca
                      void* out, int64_t o_st, int64_t o_sh, void* cmp_o, void* slc_o, void* swa_o, int64_t co_st,
                      int64_t co_sh, float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk, int64_t tk_sh,
                      int64_t tk_st, float* sp_m, float* sp_l, float* sp_o, void* sp_keep_p, float* sp_keep_m,
-                     int nsplit, const int32_t* context_lens, const int32_t* block_tables, int table_stride,
-                     const int32_t* cmp_block_tables, int cmp_table_stride, int page_size, int B, int QH, int KH,
-                     int D, int VD, int fixed_y_maxlen, int fixed_num_slc_blocks, int kernel_size, int stride,
-                     int block_size, int top_n, int num_init, int num_local, int ignore_index, int window,
-                     float sm_scale, void* stream);
+                     int nsplit, const int32_t* cmp_slot_mapping, const int32_t* context_lens,
+                     const int32_t* block_tables, int table_stride, const int32_t* cmp_block_tables,
+                     int cmp_table_stride, int page_size, int B, int QH, int KH, int D, int VD, int fixed_y_maxlen,
+                     int fixed_num_slc_blocks, int kernel_size, int stride, int block_size, int top_n, int num_init,
+                     int num_local, int ignore_index, int window, float sm_scale, void* stream);
 /* Replaces flash_nsa/inference/select_attn.py:655-787 (fused_slc_swa_attn_decode) + inference/combine.py:104-127
  * (combine_decode): selected-block and window attention; slc_o / swa_o (optional, same strides as cmp_o) receive the
  * branch outputs; out (optional) = cmp_o*sig(w0) + slc_o*sig(w1) + swa_o*sig(w2).

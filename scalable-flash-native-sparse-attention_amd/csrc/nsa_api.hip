@@ -577,11 +577,11 @@ int nsa_decode_split(const void* q, int64_t q_st, int64_t q_sh, const void* k_ca
                      void* out, int64_t o_st, int64_t o_sh, void* cmp_o, void* slc_o, void* swa_o, int64_t co_st,
                      int64_t co_sh, float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk, int64_t tk_sh,
                      int64_t tk_st, float* sp_m, float* sp_l, float* sp_o, void* sp_keep_p, float* sp_keep_m,
-                     int nsplit, const int32_t* context_lens, const int32_t* block_tables, int table_stride,
-                     const int32_t* cmp_block_tables, int cmp_table_stride, int page_size, int B, int QH, int KH,
-                     int D, int VD, int fixed_y_maxlen, int fixed_num_slc_blocks, int kernel_size, int stride,
-                     int block_size, int top_n, int num_init, int num_local, int ignore_index, int window,
-                     float sm_scale, void* stream) {
+                     int nsplit, const int32_t* cmp_slot_mapping, const int32_t* context_lens,
+                     const int32_t* block_tables, int table_stride, const int32_t* cmp_block_tables,
+                     int cmp_table_stride, int page_size, int B, int QH, int KH, int D, int VD, int fixed_y_maxlen,
+                     int fixed_num_slc_blocks, int kernel_size, int stride, int block_size, int top_n, int num_init,
+                     int num_local, int ignore_index, int window, float sm_scale, void* stream) {
   int rc = check_heads("decode_split", QH, KH, D, VD);
   if (rc) return rc;
   rc = check_nsa_sizes("decode_split", kernel_size, stride, block_size);
@@ -611,6 +611,7 @@ int nsa_decode_split(const void* q, int64_t q_st, int64_t q_sh, const void* k_ca
   p.sp_m = sp_m; p.sp_l = sp_l; p.sp_o = sp_o;
   p.sp_keep_p = (_Float16*)sp_keep_p; p.sp_keep_m = sp_keep_m; p.nsplit = nsplit;
   p.ctx_lens = context_lens;
+  p.cmp_slots = cmp_slot_mapping;
   p.table = block_tables;
   p.cmp_table = cmp_block_tables; p.cmp_table_stride = cmp_table_stride; p.page_size = page_size;
   p.G = QH / KH; p.KH = KH;

@@ -539,6 +539,34 @@ __global__ __launch_bounds__(SPLIT_WAVES * 64) void decode_cmp_partial_kernel(Ns
   const int32_t* ctab = p.cmp_table + (int64_t)b * p.cmp_table_stride;
   const int page = p.page_size;
   for (int i = tid; i < (y + page - 1) / page; i += NW * 64) tab_s[i] = ctab[i];
+  // The compressed row that the newest token completes (mean of the last kernel_size raw rows, fp32 sums in row
+  // order like nsa_paged_pool_decode; flash_nsa/inference/compress_kv.py:253-287 upstream) is written by the part
+  // that attends it -- the one whose waves own the last unit -- wave 0 for K and wave 1 for V, one 16-byte piece per
+  // lane.  Only this workgroup reads it back in this launch, so a workgroup-scope release and the barrier suffice.
+  {
+    const int cmp_slot = p.cmp_slots != nullptr ? p.cmp_slots[b] : -1;
+    const int last_unit = y > 0 ? (y - 1) / UK : 0;
+    if (cmp_slot >= 0 && L >= p.kernel_size && sp == (last_unit % (NW * nsplit)) / NW && wave < 2) {
+      bf16_t* cache = const_cast<bf16_t*>(wave == 0 ? p.k : p.v);
+      const int64_t c_sr = wave == 0 ? p.k_sr : p.v_sr, c_sh = wave == 0 ? p.k_sh : p.v_sh;
+      if (lane < (wave == 0 ? D : VD) / 8) {
+        const int32_t* tab = p.table + (int64_t)b * p.table_stride;
+        const int st = ((L - p.kernel_size) / p.stride) * p.stride;
+        float a[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (int r = 0; r < p.kernel_size; r++) {
+          const int n = st + r;
+          const int64_t row = (int64_t)tab[n / page] * page + (n % page);
+          const bf16x8 x = ld_global_b128(cache + row * c_sr + (int64_t)kh * c_sh + lane * 8);
+#pragma unroll
+          for (int e = 0; e < 8; e++) a[e] += (float)x[e];
+        }
+        const float inv = 1.f / (float)p.kernel_size;
+        *reinterpret_cast<bf16x8*>(cache + (int64_t)cmp_slot * c_sr + (int64_t)kh * c_sh + lane * 8) =
+            pack8(a[0] * inv, a[1] * inv, a[2] * inv, a[3] * inv, a[4] * inv, a[5] * inv, a[6] * inv, a[7] * inv);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    }
+  }
   __syncthreads();
   const bf16_t* kbase = p.k + (int64_t)kh * p.k_sh;
   const bf16_t* vbase = p.v + (int64_t)kh * p.v_sh;

@@ -94,6 +94,21 @@ def nsa_decode(q, k, v, w, context_lens, block_tables, cmp_slot_mapping, cmp_blo
                                  slot_mapping=slot_mapping)
     if new_k is not None:
         store_kvcache(new_k, new_v, k, v, slot_mapping)
+    if (fused_decode_supported(q, k, v) and cmp_num_splits > 1 and
+            decode_split_fits(q, k, v, block_tables, fixed_y_maxlen, fixed_num_slc_blocks)):
+        # small batches of long contexts: the compressed branch is cut in that many key-interleaved parts per
+        # (request, kv head); two launches.  From 8 requests on the first of them also pools the newest compressed
+        # row (2 us less than the pooling launch at 16-32 requests); below that the pooling, which sits in front of
+        # the one workgroup that owns the last unit, costs more than its launch (46 -> 49 us for one request).
+        fuse_pool = q.size(0) >= 8
+        if not fuse_pool:
+            kv_mean_pooling_decode(k, v, block_table=block_tables, slot_mapping=cmp_slot_mapping,
+                                   context_lens=context_lens, kernel_size=kernel_size, stride=stride)
+        return decode_split(q, k, v, w, block_tables, cmp_block_tables, context_lens, nsplit=cmp_num_splits,
+                            fixed_y_maxlen=fixed_y_maxlen, fixed_num_slc_blocks=fixed_num_slc_blocks,
+                            kernel_size=kernel_size, stride=stride, block_size=block_size, top_n=top_n,
+                            num_inital=num_init_blocks, num_local=num_local_blocks, window_size=window_size,
+                            sm_scale=sm_scale, cmp_slot_mapping=cmp_slot_mapping if fuse_pool else None)
     kv_mean_pooling_decode(k, v, block_table=block_tables, slot_mapping=cmp_slot_mapping, context_lens=context_lens,
                            kernel_size=kernel_size, stride=stride)
     if fused_decode_supported(q, k, v):
@@ -105,15 +120,8 @@ def nsa_decode(q, k, v, w, context_lens, block_tables, cmp_slot_mapping, cmp_blo
                                           num_inital=num_init_blocks, num_local=num_local_blocks, sm_scale=sm_scale)
             return decode_slc_swa_combine(q, k, v, w, topk, cmp_o, block_tables, context_lens, block_size=block_size,
                                           top_n=top_n, window_size=window_size, sm_scale=sm_scale)
-        # cmp_num_splits > 1: the compressed branch is cut in that many key-interleaved parts per (request, kv head);
-        # pays off for small batches of long contexts and when a few very long contexts sit in a batch of short ones
-        if decode_split_fits(q, k, v, block_tables, fixed_y_maxlen, fixed_num_slc_blocks):
-            return decode_split(q, k, v, w, block_tables, cmp_block_tables, context_lens, nsplit=cmp_num_splits,
-                                fixed_y_maxlen=fixed_y_maxlen, fixed_num_slc_blocks=fixed_num_slc_blocks,
-                                kernel_size=kernel_size, stride=stride, block_size=block_size, top_n=top_n,
-                                num_inital=num_init_blocks, num_local=num_local_blocks, window_size=window_size,
-                                sm_scale=sm_scale)
-        # capacities beyond the LDS of that path: three launches, the probabilities recomputed from the keys
+        # parts with capacities beyond the LDS of the two-launch path: three launches after the pooling, the
+        # probabilities recomputed from the keys
         cmp_o, pg = decode_cmp_split(q, k, v, cmp_block_tables, context_lens, nsplit=cmp_num_splits,
                                      fixed_y_maxlen=fixed_y_maxlen, kernel_size=kernel_size, stride=stride,
                                      sm_scale=sm_scale)

@@ -331,11 +331,13 @@ def decode_split_fits(q, k, v, block_tables, fixed_y_maxlen, fixed_num_slc_block
 
 def decode_split(q, k, v, w, block_tables, cmp_block_tables, context_lens, nsplit=4, fixed_y_maxlen=8192,
                  fixed_num_slc_blocks=2048, kernel_size=32, stride=16, block_size=64, top_n=16, num_inital=1,
-                 num_local=2, window_size=512, sm_scale=None, return_parts=False):
+                 num_local=2, window_size=512, sm_scale=None, return_parts=False, cmp_slot_mapping=None):
     """The decode step in two launches, for small batches of long contexts: the compressed branch cut into `nsplit`
     parts per (request, kv head) so that it fills the GPU, then one workgroup per pair for the merge, the block
     selection, selected + window attention and the gated combine.  -> o [B,QH,VD]
-    (return_parts: also cmp_o, slc_o, swa_o, topk [KH,B,top_n], lse [B,QH])."""
+    (return_parts: also cmp_o, slc_o, swa_o, topk [KH,B,top_n], lse [B,QH]).
+    cmp_slot_mapping [B] (-1: none): the first launch also pools the compressed row that the newest token completes;
+    None: that row is in the pool already."""
     check_bf16(q)
     page, KH, D, ksr, ksh = _pool_args(k)
     _, _, VD, vsr, vsh = _pool_args(v)
@@ -357,7 +359,7 @@ def decode_split(q, k, v, w, block_tables, cmp_block_tables, context_lens, nspli
               _lib.ptr(lse), lse.stride(0) if return_parts else 0, lse.stride(1) if return_parts else 0,
               _lib.ptr(topk), topk.stride(0) if return_parts else 0, topk.stride(1) if return_parts else 0,
               sp_ml[0].data_ptr(), sp_ml[1].data_ptr(), sp_o.data_ptr(), keep_p.data_ptr(), keep_m.data_ptr(), nsplit,
-              _i32(context_lens).data_ptr(), _i32(block_tables).data_ptr(), block_tables.stride(0),
+              _lib.ptr(None if cmp_slot_mapping is None else _i32(cmp_slot_mapping)), _i32(context_lens).data_ptr(), _i32(block_tables).data_ptr(), block_tables.stride(0),
               _i32(cmp_block_tables).data_ptr(), cmp_block_tables.stride(0), page, B, QH, KH, D, VD,
               int(fixed_y_maxlen), int(fixed_num_slc_blocks), kernel_size, stride, block_size, top_n, num_inital,
               num_local, -1, window_size, sm_scale, _lib.stream_ptr())

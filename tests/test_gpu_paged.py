@@ -500,6 +500,37 @@ def test_one_launch_decode_pools_the_new_row_itself(device):
     assert torch.equal(o1, o2)
 
 
+@pytest.mark.parametrize("nsplit", [2, 8])
+def test_split_decode_pools_the_new_row_itself(device, nsplit):
+    """The two-launch decode with a slot mapping == pooling kernel followed by the same path without: the pools end
+    bit-identical and so do the outputs (the part that owns the last unit pools the row before it attends it), and
+    nsa_decode takes that route when asked for parts."""
+    from flash_nsa import nsa_decode
+    from flash_nsa.inference import decode_split, kv_mean_pooling_decode
+    QH, KH, D = 64, 4, 128
+    ctx = [1024, 48, 32, 31, 2001, 656, 645, 4099, 4128, 2064]   # six of them complete a compressed row at this step
+    case = build_pool(ctx, KH, D, D, page=128, seed=41)
+    prepool(case, [L - 1 for L in ctx])
+    slots = decode_slot_mapping(case)
+    assert int((slots >= 0).sum()) == 6
+    B = len(ctx)
+    q, w = randn_bf16(B, QH, D, seed=42).to(device), randn_bf16(B, QH, 3, seed=43).to(device)
+    ctx_t = torch.tensor(ctx, dtype=torch.int32, device=device)
+    d1, d2, d3 = to_dev(case, device), to_dev(case, device), to_dev(case, device)
+    for d in (d2, d3):
+        d["k"], d["v"] = d["k"].clone(), d["v"].clone()
+    kw = dict(fixed_y_maxlen=512, fixed_num_slc_blocks=128)
+    kv_mean_pooling_decode(d1["k"], d1["v"], block_table=d1["bt"], slot_mapping=slots.to(device), context_lens=ctx_t)
+    o1 = decode_split(q, d1["k"], d1["v"], w, d1["bt"], d1["cbt"], ctx_t, nsplit=nsplit, **kw)
+    o2 = decode_split(q, d2["k"], d2["v"], w, d2["bt"], d2["cbt"], ctx_t, nsplit=nsplit,
+                      cmp_slot_mapping=slots.to(device), **kw)
+    assert torch.equal(d1["k"], d2["k"]) and torch.equal(d1["v"], d2["v"])
+    assert torch.equal(o1, o2)
+    o3 = nsa_decode(q, d3["k"], d3["v"], w, ctx_t, d3["bt"], slots.to(device), d3["cbt"], cmp_num_splits=nsplit, **kw)
+    assert torch.equal(d1["k"], d3["k"]) and torch.equal(d1["v"], d3["v"])
+    assert torch.equal(o1, o3)
+
+
 def test_decode_qk192_v128_equals_training_last_row(device):
     """Dqk = 192, Dv = 128, 2 kv heads (the head shape of upstream's inference notebook, cell 43): nsa_decode takes
     the stage-by-stage kernels here; its output equals the last row of the training forward on the gathered
