@@ -500,6 +500,49 @@ def test_one_launch_decode_pools_the_new_row_itself(device):
     assert torch.equal(o1, o2)
 
 
+@pytest.mark.parametrize("B", [3, 9])
+def test_split_decode_graph_replay_equals_eager(device, B):
+    """The two-launch path (with the pooling as a launch of its own for 3 requests, inside the first launch for 9)
+    captured in a HIP graph: every replay, with eager work and synchronisations in between, equals the eager result,
+    also after the static inputs change."""
+    from flash_nsa import nsa_decode
+    QH, KH, D = 64, 4, 128
+    ctx = [2064, 1000, 0, 333, 4128, 640, 2049, 48, 1][:B]
+    case = build_pool([max(c, 1) for c in ctx], KH, D, D, page=128, seed=11)
+    case["ctx"] = ctx
+    case["ys"] = [max((L - 32) // 16 + 1, 0) for L in ctx]
+    prepool(case, [max(L - 1, 0) for L in ctx])
+    slots = decode_slot_mapping(case)
+    d = to_dev(case, device)
+    q = randn_bf16(B, QH, D, seed=12).to(device)
+    w = randn_bf16(B, QH, 3, seed=13).to(device)
+    ctx_t = torch.tensor(ctx, dtype=torch.int32, device=device)
+    args = (q, d["k"], d["v"], w, ctx_t, d["bt"], slots.to(device), d["cbt"])
+    kw = dict(fixed_y_maxlen=512, fixed_num_slc_blocks=128, cmp_num_splits=4)
+    eager = nsa_decode(*args, **kw).clone()
+    assert torch.isfinite(eager).all() and (eager[2] == 0).all()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        nsa_decode(*args, **kw)
+    torch.cuda.current_stream().wait_stream(side)
+    with torch.cuda.graph(graph):
+        out = nsa_decode(*args, **kw)
+    for it in range(4):
+        out.zero_()
+        junk = torch.randn(1 << 20, device=device).sum()  # the program's own eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {it} differs from eager"
+    q.copy_(randn_bf16(B, QH, D, seed=14).to(device))
+    eager2 = nsa_decode(*args, **kw).clone()
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out, eager2)
+
+
 @pytest.mark.parametrize("nsplit", [2, 8])
 def test_split_decode_pools_the_new_row_itself(device, nsplit):
     """The two-launch decode with a slot mapping == pooling kernel followed by the same path without: the pools end
