@@ -261,6 +261,8 @@ int nsa_decode_cmp_split(const void* q, int64_t q_st, int64_t q_sh, const void* 
  * cmp_o / slc_o / swa_o / lse / topk are optional outputs (null: not written).
  * nsa_decode_split_fits: 1 when fixed_y_maxlen / fixed_num_slc_blocks / the raw table width fit the LDS of (2). */
 int nsa_decode_split_fits(int D, int VD, int fixed_y_maxlen, int fixed_num_slc_blocks, int table_stride);
+/* LDS bytes of launch (2), dynamic + statically declared, for these capacities; 0 when they do not fit 160 KB */
+int nsa_decode_split_lds_total(int D, int VD, int fixed_y_maxlen, int fixed_num_slc_blocks, int table_stride);
 int nsa_decode_split(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr, int64_t k_sh,
                      const void* v_cache, int64_t v_sr, int64_t v_sh, const void* w, int64_t w_st, int64_t w_sh,
                      void* out, int64_t o_st, int64_t o_sh, void* cmp_o, void* slc_o, void* swa_o, int64_t co_st,

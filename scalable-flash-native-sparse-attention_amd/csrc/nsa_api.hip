@@ -572,6 +572,13 @@ int nsa_decode_split_fits(int D, int VD, int fixed_y_maxlen, int fixed_num_slc_b
   return nsa_decode_split_lds_bytes(p, D, VD) > 0 ? 1 : 0;
 }
 
+int nsa_decode_split_lds_total(int D, int VD, int fixed_y_maxlen, int fixed_num_slc_blocks, int table_stride) {
+  NsaDecodeParams p{};
+  fill_decode_split(p, fixed_y_maxlen, fixed_num_slc_blocks, table_stride);
+  const int dyn = nsa_decode_split_lds_bytes(p, D, VD);
+  return dyn > 0 ? dyn + nsa_decode_split_static_lds_bytes() : 0;
+}
+
 int nsa_decode_split(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr, int64_t k_sh,
                      const void* v_cache, int64_t v_sr, int64_t v_sh, const void* w, int64_t w_st, int64_t w_sh,
                      void* out, int64_t o_st, int64_t o_sh, void* cmp_o, void* slc_o, void* swa_o, int64_t co_st,

@@ -141,4 +141,5 @@ int nsa_decode_fused_launch(const NsaDecodeParams& p, int B, int D, int VD, hipS
 int nsa_decode_fused_lds_bytes(const NsaDecodeParams& p, int D, int VD);  // 0: does not fit
 int nsa_decode_cmp_split_launch(const NsaDecodeParams& p, int B, int nsplit, int D, int VD, hipStream_t stream);
 int nsa_decode_split_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream);
-int nsa_decode_split_lds_bytes(const NsaDecodeParams& p, int D, int VD);  // final kernel; 0: does not fit
+int nsa_decode_split_lds_bytes(const NsaDecodeParams& p, int D, int VD);  // final kernel, dynamic part; 0: does not fit
+int nsa_decode_split_static_lds_bytes();                                   // final kernel, statically declared part

@@ -18,6 +18,9 @@
 namespace {
 
 constexpr int DEC_WAVES = 8;
+// static LDS of decode_slc_swa_kernel (statistics and weights of up to 64 parts of the compressed branch); the host
+// adds it to the dynamic size when it decides whether a launch fits the 160 KB of a CU
+constexpr size_t SLC_SWA_STATIC_LDS = (3 * 16 + 64 * 16) * sizeof(float);
 constexpr int UK = 32;  // keys per unit
 
 // One wave's flash-attention state over units of 32 keys for the 16 heads of a kv group.
@@ -748,6 +751,8 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecod
   const int nb = min(L > 0 ? (L - 1) / Bs + 1 : 0, p.nb_cap);
   __shared__ float sp_lse_s[16], sp_m_s[16], sp_l_s[16];
   __shared__ float sp_w_s[64 * 16];  // weights of the parts of the compressed branch (nsplit <= 64)
+  static_assert(sizeof(sp_lse_s) + sizeof(sp_m_s) + sizeof(sp_l_s) + sizeof(sp_w_s) == SLC_SWA_STATIC_LDS,
+                "the host-side LDS budget must count this kernel's static arrays");
   constexpr int OPT = 16 * VD / NT;  // output values per thread
   static_assert((16 * VD) % NT == 0, "output values must divide over the threads");
   float ocmp_pre[OPT];               // split path: merged compressed-branch output of this thread's values
@@ -1112,9 +1117,11 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_fused_kernel(NsaDecodeP
 }  // namespace
 
 template <class K>
-static int launch_dyn(K kern, dim3 grid, size_t dyn, const NsaDecodeParams& p, hipStream_t stream, const char* name) {
-  if (dyn > 160 * 1024) {
-    nsa_set_error("%s: %zu bytes of LDS needed (fixed_y_maxlen / fixed_num_slc_blocks too large)", name, dyn);
+static int launch_dyn(K kern, dim3 grid, size_t dyn, const NsaDecodeParams& p, hipStream_t stream, const char* name,
+                      size_t static_lds = 0) {
+  if (dyn + static_lds > 160 * 1024) {
+    nsa_set_error("%s: %zu bytes of LDS needed (fixed_y_maxlen / fixed_num_slc_blocks too large)", name,
+                  dyn + static_lds);
     return NSA_ERR_UNSUPPORTED;
   }
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn);
@@ -1165,10 +1172,10 @@ int nsa_decode_slc_swa_launch(const NsaDecodeParams& p, int B, int D, int VD, hi
   if (p.pg != nullptr) extra += (size_t)((p.nb_cap + 3) & ~3) * sizeof(float);  // block scores
   if (D == 128 && VD == 128)
     return launch_dyn(decode_slc_swa_kernel<128, 128>, grid, slot_bytes<128, 128>() + extra, p, stream,
-                      "decode_slc_swa_kernel");
+                      "decode_slc_swa_kernel", SLC_SWA_STATIC_LDS);
   if (D == 64 && VD == 64)
     return launch_dyn(decode_slc_swa_kernel<64, 64>, grid, slot_bytes<64, 64>() + extra, p, stream,
-                      "decode_slc_swa_kernel");
+                      "decode_slc_swa_kernel", SLC_SWA_STATIC_LDS);
   nsa_set_error("decode: unsupported head dims D=%d VD=%d (built: 128/128, 64/64)", D, VD);
   return NSA_ERR_UNSUPPORTED;
 }
@@ -1206,7 +1213,7 @@ static size_t split_final_lds(const NsaDecodeParams& p) {
   const size_t nuc = (size_t)(p.y_cap + UK - 1) / UK;
   const size_t total = slots + (size_t)(2 * DEC_WAVES * 16 + 64 + ((p.table_stride + 3) & ~3)) * 4 +
                        (size_t)(((p.nb_cap + 3) & ~3) + (nuc * 16 > 2 * 64 * 16 ? nuc * 16 : 2 * 64 * 16)) * 4;  // factors, or the parts' (m, l)
-  return total <= 160 * 1024 ? total : 0;
+  return total + SLC_SWA_STATIC_LDS <= 160 * 1024 ? total : 0;
 }
 
 int nsa_decode_split_lds_bytes(const NsaDecodeParams& p, int D, int VD) {
@@ -1214,6 +1221,8 @@ int nsa_decode_split_lds_bytes(const NsaDecodeParams& p, int D, int VD) {
   if (D == 64 && VD == 64) return (int)split_final_lds<64, 64>(p);
   return 0;
 }
+
+int nsa_decode_split_static_lds_bytes() { return (int)SLC_SWA_STATIC_LDS; }
 
 int nsa_decode_split_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream) {
   if (B <= 0) return NSA_OK;
@@ -1231,12 +1240,14 @@ int nsa_decode_split_launch(const NsaDecodeParams& p, int B, int D, int VD, hipS
     decode_cmp_partial_kernel<128, 128><<<grid1, SPLIT_WAVES * 64, dyn1, stream>>>(p);
     int rc = nsa_check_launch("decode_cmp_partial_kernel");
     if (rc) return rc;
-    return launch_dyn(decode_slc_swa_kernel<128, 128>, grid2, (size_t)lds2, p, stream, "decode_slc_swa_kernel");
+    return launch_dyn(decode_slc_swa_kernel<128, 128>, grid2, (size_t)lds2, p, stream, "decode_slc_swa_kernel",
+                      SLC_SWA_STATIC_LDS);
   }
   decode_cmp_partial_kernel<64, 64><<<grid1, SPLIT_WAVES * 64, dyn1, stream>>>(p);
   int rc = nsa_check_launch("decode_cmp_partial_kernel");
   if (rc) return rc;
-  return launch_dyn(decode_slc_swa_kernel<64, 64>, grid2, (size_t)lds2, p, stream, "decode_slc_swa_kernel");
+  return launch_dyn(decode_slc_swa_kernel<64, 64>, grid2, (size_t)lds2, p, stream, "decode_slc_swa_kernel",
+                    SLC_SWA_STATIC_LDS);
 }
 
 // LDS of the one-launch decode kernel; 0 when it does not fit (the caller then takes the two-launch path)

@@ -97,3 +97,26 @@ def test_helper_does_not_confuse_a_new_tensor_with_the_registered_one():
     NSAHelper.init_cu_seqlens(b)
     assert (NSAHelper.x_maxlen, NSAHelper.y_len) == (400, 19 + 24)
     assert NSAHelper._host_cu == [0, 330, 730]
+
+
+def test_split_decode_lds_budget_counts_static_arrays():
+    """nsa_decode_split_fits must imply dynamic + statically declared LDS <= 160 KB for the second launch: a
+    capacity whose dynamic part alone fits but whose total does not has to be reported as not fitting, so that
+    nsa_decode falls back instead of failing at launch.  Host arithmetic only."""
+    from flash_nsa import _lib
+    limit = 160 * 1024
+    seen_near_limit = 0
+    for D in (128, 64):
+        for y in (512, 2048, 8192, 16384, 20000, 20480, 24576, 32768):
+            for nb in (64, 512, 2048, 4096, 8192):
+                prev_fit = True
+                for tw in list(range(8, 6000, 97)):
+                    fits = _lib.value("nsa_decode_split_fits", D, D, y, nb, tw)
+                    total = _lib.value("nsa_decode_split_lds_total", D, D, y, nb, tw)
+                    assert (total > 0) == bool(fits)
+                    if fits:
+                        assert 4288 < total <= limit, (D, y, nb, tw, total)
+                        assert prev_fit, "a wider table cannot fit where a narrower one did not"
+                        seen_near_limit += total > limit - 4288
+                    prev_fit = bool(fits)
+    assert seen_near_limit > 0, "the sweep must reach totals within the static part of the limit"
