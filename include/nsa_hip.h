@@ -273,6 +273,27 @@ int nsa_decode_split(const void* q, int64_t q_st, int64_t q_sh, const void* k_ca
                      int cmp_table_stride, int page_size, int B, int QH, int KH, int D, int VD, int fixed_y_maxlen,
                      int fixed_num_slc_blocks, int kernel_size, int stride, int block_size, int top_n, int num_init,
                      int num_local, int ignore_index, int window, float sm_scale, void* stream);
+/* nsa_decode_split without any allocation.  No counterpart upstream: it is for callers that cannot allocate device
+ * memory around the call (code under graph capture, tight serving loops, harnesses that forbid hipMalloc).  The
+ * arguments are those of nsa_decode_split minus the five scratch buffers, which are carved out of one file-scope
+ * device array of nsa_decode_split_static_capacity() bytes (32 MiB, held by every GPU the library runs on until the
+ * process ends).  nsa_decode_split_static_bytes gives the bytes a call needs (e.g. 21.6 MB for 16 requests x 4 kv
+ * heads x 8 parts at fixed_y_maxlen 8192); a call that needs more is refused with NSA_ERR_UNSUPPORTED.  All calls on
+ * one GPU share the array: calls that overlap there (other streams or threads) race.  Neither this entry point nor
+ * anything below it calls hipMalloc / hipFree. */
+int64_t nsa_decode_split_static_capacity(void);
+int64_t nsa_decode_split_static_bytes(int B, int KH, int VD, int nsplit, int fixed_y_maxlen);
+int nsa_decode_split_static(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr,
+                            int64_t k_sh, const void* v_cache, int64_t v_sr, int64_t v_sh, const void* w,
+                            int64_t w_st, int64_t w_sh, void* out, int64_t o_st, int64_t o_sh, void* cmp_o,
+                            void* slc_o, void* swa_o, int64_t co_st, int64_t co_sh, float* lse, int64_t lse_st,
+                            int64_t lse_sh, int32_t* topk, int64_t tk_sh, int64_t tk_st, int nsplit,
+                            const int32_t* cmp_slot_mapping, const int32_t* context_lens,
+                            const int32_t* block_tables, int table_stride, const int32_t* cmp_block_tables,
+                            int cmp_table_stride, int page_size, int B, int QH, int KH, int D, int VD,
+                            int fixed_y_maxlen, int fixed_num_slc_blocks, int kernel_size, int stride,
+                            int block_size, int top_n, int num_init, int num_local, int ignore_index, int window,
+                            float sm_scale, void* stream);
 /* Replaces flash_nsa/inference/select_attn.py:655-787 (fused_slc_swa_attn_decode) + inference/combine.py:104-127
  * (combine_decode): selected-block and window attention; slc_o / swa_o (optional, same strides as cmp_o) receive the
  * branch outputs; out (optional) = cmp_o*sig(w0) + slc_o*sig(w1) + swa_o*sig(w2).
