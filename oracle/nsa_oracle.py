@@ -27,6 +27,10 @@ Pinning status (see tests/test_oracle_*.py):
   select_blocks                   golden vectors of the upstream torch_topk (tests/golden) + brute force
   combine / activations           closed forms
   gradients                       torch.autograd of this dense restatement + fp64 gradcheck
+  nsa_forward_backward,           with no rounding: equal to torch.autograd through nsa_forward / cmp_attn /
+  branch_forward_backward         slc_attn / swa (fp64)
+  paged_pool_decode               last row of mean_pooling on the gathered sequence
+  topk_mismatch_report            hand-built cases (identical, tie-excused, wrong, out-of-range)
   swa                             parity unpinned against upstream: the upstream delegates to the external
                                   FlashAttention wheel and holds no vectors for it; pinned by the textbook
                                   band-mask definition only.
@@ -369,6 +373,177 @@ def nsa_forward(q, k, v, w, cu_seqlens, cfg: OracleConfig = OracleConfig(), wk=N
         return o, dict(cmp_k=ck, cmp_v=cv, cmp_o=cmp_o, cmp_lse=cmp_lse, topk=topk, slc_o=slc_o, slc_lse=slc_lse,
                        swa_o=swa_o, swa_lse=swa_lse)
     return o
+
+
+# ----------------------------------------------------------------------------------------------
+# forward + backward with the rounding points of a half-precision pipeline
+# ----------------------------------------------------------------------------------------------
+class _RoundBothWays(torch.autograd.Function):
+    """y = round(x) on the way forward, dx = round(dy) on the way back (a tensor that a pipeline stores in
+    half precision in both directions)."""
+
+    @staticmethod
+    def forward(ctx, x, dtype):
+        ctx.dtype = dtype
+        return x.to(dtype).to(x.dtype)
+
+    @staticmethod
+    def backward(ctx, g):
+        return g.to(ctx.dtype).to(g.dtype), None
+
+
+def _branch_backward(p, q, k, v, d_o, delta, scale, r_mma=lambda x: x):
+    """Softmax-attention backward of one branch of one sequence from its probabilities.
+    p [QH,L,M], q [L,QH,D], k [M,KH,D], v [M,KH,VD], d_o [L,QH,VD], delta [L,QH]
+    -> dq [L,QH,D], dk [M,KH,D], dv [M,KH,VD]   (dS = P * (dP - delta), the form every flash backward uses:
+    flash_nsa/ops/compress_attn.py:187-332, flash_nsa/ops/select_attn.py:142-330 upstream).
+    r_mma rounds the two computed matrix operands, P (for dV) and dS (for dQ and dK), the way a half-precision
+    matrix unit receives them (upstream casts them with .to(dtype) before tl.dot at the same places)."""
+    QH, KH = q.shape[1], k.shape[1]
+    G = QH // KH
+    M = k.shape[0]
+    ke, ve = k.repeat_interleave(G, 1), v.repeat_interleave(G, 1)
+    dp = torch.einsum("nhd,mhd->hnm", d_o, ve)
+    ds = r_mma(p * (dp - delta.transpose(0, 1)[..., None]))
+    dq = scale * torch.einsum("hnm,mhd->nhd", ds, ke)
+    dk = scale * torch.einsum("hnm,nhd->mhd", ds, q).reshape(M, KH, G, q.shape[-1]).sum(2)
+    dv = torch.einsum("hnm,nhd->mhd", r_mma(p), d_o).reshape(M, KH, G, d_o.shape[-1]).sum(2)
+    return dq, dk, dv
+
+
+def _masked_probs(q, k, mask, scale):
+    """q [Lq,QH,D], k [Lk,KH,D], mask [KH,Lq,Lk] -> softmax probabilities [QH,Lq,Lk] (rows without a key: 0)."""
+    G = q.shape[1] // k.shape[1]
+    s = torch.einsum("nhd,mhd->hnm", q, k.repeat_interleave(G, 1)) * scale
+    m = mask.repeat_interleave(G, 0)
+    s = s.masked_fill(~m, float("-inf"))
+    has = m.any(-1)
+    p = torch.softmax(torch.where(has[..., None], s, torch.zeros_like(s)), -1)
+    return torch.where(has[..., None], p, torch.zeros_like(p))
+
+
+def _branch_probs(kind, qs, ks, cfg, scale, topk_seq=None):
+    """Probabilities [QH,L,M] of one branch for one sequence; ks = compressed keys for "cmp", raw keys otherwise."""
+    L, KH = qs.shape[0], ks.shape[1]
+    t = torch.arange(L)
+    if kind == "cmp":
+        return _cmp_probs_one_seq(qs, ks, cfg.kernel_size, cfg.stride, scale)[0]
+    if kind == "slc":
+        return _masked_probs(qs, ks, _slc_mask_one_seq(topk_seq, t, L, cfg.block_size), scale)
+    d = t[:, None] - t[None, :]
+    return _masked_probs(qs, ks, ((d >= 0) & (d <= cfg.window_size))[None].expand(KH, L, L), scale)
+
+
+def branch_forward_backward(kind, q, k, v, d_o, cu_seqlens, cfg: OracleConfig = OracleConfig(), topk=None,
+                            scale=None, round_dtype: Optional[torch.dtype] = None, round_mma=False):
+    """One attention branch ("cmp": k, v are the compressed rows; "slc"; "swa") forward and backward the way a
+    flash backward computes it: o stored rounded, delta = rowsum(round(o) * d_o), dS = P (dP - delta), optionally
+    with P and dS rounded before the matrix products.  Without rounding it equals torch.autograd through
+    cmp_attn / slc_attn / swa.  -> dict(o, dq, dk, dv), gradients unrounded."""
+    scale = q.shape[-1] ** -0.5 if scale is None else scale
+    r = (lambda x: x) if round_dtype is None else (lambda x: x.to(round_dtype).to(x.dtype))
+    meta = seq_lengths(cu_seqlens, cfg.kernel_size, cfg.stride, cfg.block_size)
+    G = q.shape[1] // k.shape[1]
+    o = torch.zeros(q.shape[0], q.shape[1], v.shape[-1], dtype=q.dtype)
+    dq, dk, dv = torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)
+    for b, L in enumerate(meta["x_seqlens"]):
+        if L == 0:
+            continue
+        a, e = meta["x_cu"][b], meta["x_cu"][b + 1]
+        ka, ke = (meta["y_cu"][b], meta["y_cu"][b + 1]) if kind == "cmp" else (a, e)
+        p = _branch_probs(kind, q[a:e], k[ka:ke], cfg, scale, None if topk is None else topk[:, a:e])
+        o[a:e] = r(torch.einsum("hnm,mhd->nhd", p, v[ka:ke].repeat_interleave(G, 1)))
+        delta = (d_o[a:e] * o[a:e]).sum(-1)
+        dq[a:e], dk_i, dv_i = _branch_backward(p, q[a:e], k[ka:ke], v[ka:ke], d_o[a:e], delta, scale,
+                                               r if round_mma else (lambda x: x))
+        dk[ka:ke] += dk_i
+        dv[ka:ke] += dv_i
+    return dict(o=o, dq=dq, dk=dk, dv=dv)
+
+
+def nsa_forward_backward(q, k, v, w, d_out, cu_seqlens, cfg: OracleConfig = OracleConfig(), topk=None, wk=None,
+                         wv=None, scale=None, round_dtype: Optional[torch.dtype] = None, round_mma=False):
+    """Composed NSA forward and a hand-written backward that keeps the rounding points of the fused training node
+    (flash_nsa/modules/megatron_level_nsa.py:87-159 upstream stores exactly these tensors in q's dtype between
+    kernels): compressed K/V, the three branch outputs, the three branch output gradients d o_k = round(dy sig_k),
+    the correction term delta_k = rowsum(round(o_k) * round(d o_k)), the compressed-row gradients handed to the
+    compression backward, the learned compression's pre-activation and its gradient, and the final dq / dk / dv /
+    dw / dW.  Everything else is computed in the dtype of the inputs (fp32 or fp64); with round_mma the
+    probabilities and dS of the backward are rounded as well before they enter a matrix product.
+    With round_dtype=None nothing is rounded and the result must equal torch.autograd through nsa_forward: that
+    identity pins the backward formulas.
+    -> dict(o, dq, dk, dv, dw, dwk, dwv)"""
+    assert topk is not None, "pass the selection so that both sides attend the same blocks"
+    scale = q.shape[-1] ** -0.5 if scale is None else scale
+    r = (lambda x: x) if round_dtype is None else (lambda x: x.to(round_dtype).to(x.dtype))
+    rb = (lambda x: x) if round_dtype is None else (lambda x: _RoundBothWays.apply(x, round_dtype))
+    meta = seq_lengths(cu_seqlens, cfg.kernel_size, cfg.stride, cfg.block_size)
+    KH = k.shape[1]
+
+    # compression through autograd, with the tensors the pipeline stores rounded both ways
+    def compress_graph(x, weight, method):
+        xl = x.detach().clone().requires_grad_()
+        if method == "mean":
+            return xl, None, rb(mean_pooling(xl, cu_seqlens, cfg.kernel_size, cfg.stride))
+        wl = weight.detach().clone().requires_grad_()
+        win = rb(construct_block(xl, cu_seqlens, cfg.kernel_size, cfg.stride).flatten(-2, -1))
+        hid = rb(win @ wl.t())
+        out = hid if method == "linear" else rb(sigmoid_mul(hid) if method == "sigmoid-mul" else swiglu(hid))
+        return xl, wl, out
+
+    k_leaf, wk_leaf, ck_g = compress_graph(k, wk, cfg.cmp_k_method)
+    v_leaf, wv_leaf, cv_g = compress_graph(v, wv, cfg.cmp_v_method)
+    ck, cv = ck_g.detach(), cv_g.detach()
+
+    g = torch.sigmoid(w)
+    o = torch.zeros(q.shape[0], q.shape[1], v.shape[-1], dtype=q.dtype)
+    dq = torch.zeros_like(q)
+    dk = torch.zeros_like(k)
+    dv = torch.zeros_like(v)
+    dw = torch.zeros_like(w)
+    dck = torch.zeros_like(ck)
+    dcv = torch.zeros_like(cv)
+    for b, L in enumerate(meta["x_seqlens"]):
+        if L == 0:
+            continue
+        a, e = meta["x_cu"][b], meta["x_cu"][b + 1]
+        ya, ye = meta["y_cu"][b], meta["y_cu"][b + 1]
+        qs, ks, vs, gs, dys = q[a:e], k[a:e], v[a:e], g[a:e], d_out[a:e]
+        G = qs.shape[1] // KH
+        branches = (
+            (_branch_probs("cmp", qs, ck[ya:ye], cfg, scale), ck[ya:ye], cv[ya:ye]),
+            (_branch_probs("slc", qs, ks, cfg, scale, topk[:, a:e]), ks, vs),
+            (_branch_probs("swa", qs, ks, cfg, scale), ks, vs),
+        )
+        for i, (p, kk, vv) in enumerate(branches):
+            o_i = r(torch.einsum("hnm,mhd->nhd", p, vv.repeat_interleave(G, 1)))
+            o[a:e] += o_i * gs[..., i:i + 1]
+            dw[a:e, :, i] = gs[..., i] * (1 - gs[..., i]) * (dys * o_i).sum(-1)
+            d_oi = r(dys * gs[..., i:i + 1])
+            delta = (d_oi * o_i).sum(-1)
+            dq_i, dk_i, dv_i = _branch_backward(p, qs, kk, vv, d_oi, delta, scale, r if round_mma else (lambda x: x))
+            dq[a:e] += dq_i
+            if i == 0:
+                dck[ya:ye] += dk_i
+                dcv[ya:ye] += dv_i
+            else:
+                dk[a:e] += dk_i
+                dv[a:e] += dv_i
+    grads_k = torch.autograd.grad(ck_g, [k_leaf] + ([wk_leaf] if wk_leaf is not None else []), dck,
+                                  allow_unused=True) if ck.numel() else (torch.zeros_like(k), None)
+    grads_v = torch.autograd.grad(cv_g, [v_leaf] + ([wv_leaf] if wv_leaf is not None else []), dcv,
+                                  allow_unused=True) if cv.numel() else (torch.zeros_like(v), None)
+    dk = dk + (grads_k[0] if grads_k[0] is not None else 0)
+    dv = dv + (grads_v[0] if grads_v[0] is not None else 0)
+
+    def wgrad(leaf, grads):
+        if leaf is None:
+            return None
+        gw = grads[1] if len(grads) > 1 and grads[1] is not None else torch.zeros_like(leaf)
+        return r(gw)
+
+    return dict(o=r(o), dq=r(dq), dk=r(dk), dv=r(dv), dw=r(dw), dwk=wgrad(wk_leaf, grads_k),
+                dwv=wgrad(wv_leaf, grads_v))
 
 
 # ----------------------------------------------------------------------------------------------

@@ -202,8 +202,8 @@ __global__ void combine_fwd_kernel(const bf16_t* a, const bf16_t* bb, const bf16
       pack8(r[0], r[1], r[2], r[3], r[4], r[5], r[6], r[7]);
 }
 
-// backward: da,db,dc = dy*sig(w_k); dw_k = sig_k(1-sig_k) * sum_d dy*x_k; optional delta_k = sig_k * sum_d dy*x_k
-// (= rowsum(x_k * d x_k), the softmax-backward correction term of branch k), written as delta[k][T][H] fp32.
+// backward: da,db,dc = dy*sig(w_k); dw_k = sig_k(1-sig_k) * sum_d dy*x_k; optional delta_k = rowsum(x_k * d x_k)
+// with the stored (bf16) d x_k, the softmax-backward correction term of branch k, written as delta[k][T][H] fp32.
 // D/8 consecutive lanes share one (t,h); D/8 must be a power of two <= 64.
 __global__ void combine_bwd_kernel(const bf16_t* a, const bf16_t* bb, const bf16_t* c, int64_t i_st, int64_t i_sh,
                                    const bf16_t* w, int64_t w_st, int64_t w_sh, const bf16_t* dy, int64_t dy_st,
@@ -221,21 +221,29 @@ __global__ void combine_bwd_kernel(const bf16_t* a, const bf16_t* bb, const bf16
   int64_t off = t * i_st + (int64_t)h * i_sh + cc * 8;
   bf16x8 va = ld_global_b128(a + off), vb = ld_global_b128(bb + off), vc = ld_global_b128(c + off);
   bf16x8 g = ld_global_b128(dy + t * dy_st + (int64_t)h * dy_sh + cc * 8);
-  float ra[8], rb[8], rc[8], p0 = 0.f, p1 = 0.f, p2 = 0.f;
+  // p_k = sum_d dy * x_k (gate gradient); q_k = sum_d round(dy * sig_k) * x_k: the correction term is formed from
+  // the ROUNDED branch gradient, the one the attention backward kernels read, so that dP - delta cancels exactly
+  // where a row's probabilities are one-hot (upstream forms it the same way from the stored bf16 tensors,
+  // flash_nsa/ops/compress_attn.py:160-184)
+  float p0 = 0.f, p1 = 0.f, p2 = 0.f, q0 = 0.f, q1 = 0.f, q2 = 0.f;
+  bf16x8 ra, rb, rc;
 #pragma unroll
   for (int e = 0; e < 8; e++) {
     float gf = (float)g[e];
-    ra[e] = gf * s0; rb[e] = gf * s1; rc[e] = gf * s2;
-    p0 += gf * (float)va[e]; p1 += gf * (float)vb[e]; p2 += gf * (float)vc[e];
+    float xa = (float)va[e], xb = (float)vb[e], xc = (float)vc[e];
+    ra[e] = (bf16_t)(gf * s0); rb[e] = (bf16_t)(gf * s1); rc[e] = (bf16_t)(gf * s2);
+    p0 += gf * xa; p1 += gf * xb; p2 += gf * xc;
+    q0 += (float)ra[e] * xa; q1 += (float)rb[e] * xb; q2 += (float)rc[e] * xc;
   }
   for (int o = C >> 1; o > 0; o >>= 1) {
     p0 += __shfl_xor(p0, o, 64); p1 += __shfl_xor(p1, o, 64); p2 += __shfl_xor(p2, o, 64);
+    q0 += __shfl_xor(q0, o, 64); q1 += __shfl_xor(q1, o, 64); q2 += __shfl_xor(q2, o, 64);
   }
   if (!ok) return;
   int64_t ooff = (t * H + h) * (int64_t)D + cc * 8;  // grads are contiguous [T,H,D]
-  *reinterpret_cast<bf16x8*>(da + ooff) = pack8(ra[0], ra[1], ra[2], ra[3], ra[4], ra[5], ra[6], ra[7]);
-  *reinterpret_cast<bf16x8*>(db + ooff) = pack8(rb[0], rb[1], rb[2], rb[3], rb[4], rb[5], rb[6], rb[7]);
-  *reinterpret_cast<bf16x8*>(dc + ooff) = pack8(rc[0], rc[1], rc[2], rc[3], rc[4], rc[5], rc[6], rc[7]);
+  *reinterpret_cast<bf16x8*>(da + ooff) = ra;
+  *reinterpret_cast<bf16x8*>(db + ooff) = rb;
+  *reinterpret_cast<bf16x8*>(dc + ooff) = rc;
   if (cc == 0) {
     bf16_t* dwp = dw + (t * H + h) * 3;
     dwp[0] = (bf16_t)(s0 * (1.f - s0) * p0);
@@ -243,9 +251,9 @@ __global__ void combine_bwd_kernel(const bf16_t* a, const bf16_t* bb, const bf16
     dwp[2] = (bf16_t)(s2 * (1.f - s2) * p2);
     if (delta != nullptr) {
       int64_t TH = T * H;
-      delta[0 * TH + t * H + h] = s0 * p0;
-      delta[1 * TH + t * H + h] = s1 * p1;
-      delta[2 * TH + t * H + h] = s2 * p2;
+      delta[0 * TH + t * H + h] = q0;
+      delta[1 * TH + t * H + h] = q1;
+      delta[2 * TH + t * H + h] = q2;
     }
   }
 }

@@ -18,6 +18,145 @@ def dev_randn(shape, seed, device):
     return torch.randn(*shape, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
 
 
+def test_c1_exact(device):
+    """The reference's own CPU-runnable configuration at its own shape: one causal sequence of 4096 tokens, 16
+    q-heads on 1 kv head, d = 128, i.i.d. N(0,1) from seed 0, mean compression 32/16, blocks of 64, top-16 with 1
+    initial + 2 local forced blocks, window 512.  The device's selection is compared with the oracle's own (sets
+    identical except at score ties within 1e-3), the forward with the fp32 oracle, the backward with the oracle
+    that keeps the pipeline's rounding points; every element at 2e-2 + 1e-2 |ref| (dk / dv, sums over up to 4096 x 16
+    query rows: relative to max(|ref|, rms of the row))."""
+    from flash_nsa import NSAConfig, NSACore
+    from flash_nsa.ops.compress_kv import mean_pooling_fwd
+    from flash_nsa.ops.compress_attn import cmp_attn_fwd
+    from flash_nsa.ops.topk import slc_topk_indices
+    T, QH, KH, D = 4096, 16, 1, 128
+    g = torch.Generator().manual_seed(0)
+    q, k, v, w = [torch.randn(*s, generator=g).to(torch.bfloat16) for s in
+                  ((T, QH, D), (T, KH, D), (T, KH, D), (T, QH, 3))]
+    do = torch.randn(T, QH, D, generator=g).to(torch.bfloat16)
+    cu = torch.tensor([0, T], dtype=torch.int32)
+    core = NSACore(NSAConfig(head_dim=D, num_heads=QH, num_kv_heads=KH))
+    qd, kd, vd, wd = [t.to(device).requires_grad_() for t in (q, k, v, w)]
+    out = core(qd, kd, vd, wd, cu.to(device))
+    out.backward(do.to(device))
+    with torch.no_grad():
+        ck, cv = mean_pooling_fwd(kd.detach()), mean_pooling_fwd(vd.detach())
+        _, lse = cmp_attn_fwd(qd.detach(), ck, cv)
+        topk, _ = slc_topk_indices(qd.detach(), ck, lse)
+    cfg = O.OracleConfig()
+    rt, imps = O.slc_topk(q.float(), ck.float().cpu(), None, cu, cfg, return_importance=True)
+    n_rows, n_diff, n_bad = O.topk_mismatch_report(topk.cpu(), rt, imps, cu, 64, 16, tie_tol=1e-3)
+    assert n_rows == T and n_bad == 0 and n_diff <= 4, (n_rows, n_diff, n_bad)
+    # at 4096 tokens most rows have more than 16 blocks to choose from: the selection is a real choice
+    assert int((torch.arange(T) // 64 + 1 > 16).sum()) > T // 2
+    ref_o = O.nsa_forward(q.float(), k.float(), v.float(), w.float(), cu, cfg, topk=topk.cpu())
+    assert_close(out, ref_o, "o against the fp32 oracle")
+    ref = O.nsa_forward_backward(q.float(), k.float(), v.float(), w.float(), do.float(), cu, cfg, topk=topk.cpu(),
+                                 round_dtype=torch.bfloat16, round_mma=True)
+    assert_close(out, ref["o"], "o")
+    assert_close(qd.grad, ref["dq"], "dq")
+    assert_close(kd.grad, ref["dk"], "dk", row_scale=True)
+    assert_close(vd.grad, ref["dv"], "dv", row_scale=True)
+    assert_close(wd.grad, ref["dw"], "dw")
+
+
+def test_long_context_packed_batch_beyond_4gib_offsets(device):
+    """Upstream documents a single-GPU limit of 256K tokens from 32-bit pointer offsets (README.md:99).  A packed
+    batch of 3 x 131072 tokens (64q/4kv, d = 128) puts the third sequence beyond 2^32 bytes and 2^31 elements of q,
+    o, dO and dq: its output and dq must equal, bit for bit, the same sequence run alone; dk / dv to the order of
+    the fp32 atomic additions."""
+    from flash_nsa import NSAConfig, NSACore
+    L, QH, KH, D = 131072, 64, 4, 128
+    T = 3 * L
+    assert 2 * L * QH * D * 2 >= 2 ** 32 and 2 * L * QH * D >= 2 ** 31
+    core = NSACore(NSAConfig(head_dim=D, num_heads=QH, num_kv_heads=KH))
+    q, k, v, w, do = [dev_randn(s, 30 + i, device) for i, s in
+                      enumerate([(T, QH, D), (T, KH, D), (T, KH, D), (T, QH, 3), (T, QH, D)])]
+
+    def run(sl, cu):
+        ts = [t[sl].clone().requires_grad_() for t in (q, k, v, w)]
+        o = core(*ts, torch.tensor(cu, dtype=torch.int32, device=device))
+        o.backward(do[sl])
+        return [o.detach()] + [t.grad for t in ts]
+
+    packed = run(slice(0, T), [0, L, 2 * L, T])
+    assert all(torch.isfinite(t[2 * L:]).all() for t in packed)
+    third = [t[2 * L:].clone() for t in packed]
+    first = [t[:L].clone() for t in packed]
+    del packed
+    torch.cuda.empty_cache()
+    for name, got, sl in (("third", third, slice(2 * L, T)), ("first", first, slice(0, L))):
+        single = run(sl, [0, L])
+        assert torch.equal(got[0], single[0]), f"{name} sequence: forward differs from the sequence run alone"
+        assert torch.equal(got[1], single[1]), f"{name} sequence: dq differs"
+        assert_close(got[2], single[2], f"{name} sequence: dk", atol=2e-3, rtol=8e-3, row_scale=True)
+        assert_close(got[3], single[3], f"{name} sequence: dv", atol=2e-3, rtol=8e-3, row_scale=True)
+        assert torch.equal(got[4], single[4]), f"{name} sequence: dw differs"
+        del single
+        torch.cuda.empty_cache()
+
+
+def test_long_context_262144_tokens(device):
+    """One sequence of 262144 tokens (64q/4kv, d = 128) forward + backward: gradients finite, the first 4096 rows of
+    o and dq bit-equal to a 4096-token run (causality), the last 64 rows of kv group 0 against the oracle (their
+    selection compared with the oracle's own, their output with the device's selection), and the block selector
+    forced to work in short segments returns the same indices as the default at this length."""
+    import os
+    from flash_nsa import NSAConfig, NSACore, NSAHelper
+    from flash_nsa.ops.compress_kv import mean_pooling_fwd
+    from flash_nsa.ops.compress_attn import cmp_attn_fwd
+    from flash_nsa.ops.topk import slc_topk_indices
+    T, QH, KH, D, P, n = 262144, 64, 4, 128, 4096, 64
+    q, k, v, w, do = [dev_randn(s, 40 + i, device) for i, s in
+                      enumerate([(T, QH, D), (T, KH, D), (T, KH, D), (T, QH, 3), (T, QH, D)])]
+    core = NSACore(NSAConfig(head_dim=D, num_heads=QH, num_kv_heads=KH))
+    cu = torch.tensor([0, T], dtype=torch.int32, device=device)
+    ts = [t.clone().requires_grad_() for t in (q, k, v, w)]
+    out = core(*ts, cu)
+    out.backward(do)
+    for t in ts:
+        assert torch.isfinite(t.grad).all()
+    ps = [t[:P].clone().requires_grad_() for t in (q, k, v, w)]
+    short = core(*ps, torch.tensor([0, P], dtype=torch.int32, device=device))
+    short.backward(do[:P])
+    assert torch.equal(out[:P], short) and torch.equal(ts[0].grad[:P], ps[0].grad)
+    out = out.detach()
+    del ts, ps, short
+    torch.cuda.empty_cache()
+    # selection: default segmenting against forced short segments
+    NSAHelper.init_cu_seqlens(cu)
+    with torch.no_grad():
+        ck, cv = mean_pooling_fwd(k), mean_pooling_fwd(v)
+        _, lse = cmp_attn_fwd(q, ck, cv)
+        topk, _ = slc_topk_indices(q, ck, lse)
+        try:
+            os.environ["NSA_TOPK_SEG_BLOCKS"] = "512"
+            topk_seg, _ = slc_topk_indices(q, ck, lse)
+        finally:
+            os.environ.pop("NSA_TOPK_SEG_BLOCKS", None)
+    assert torch.equal(topk, topk_seg), "segment length changed the selection"
+    # the last n rows of kv group 0 against the oracle: the sequence laid out as a paged pool with identity tables
+    page = 256
+    y = ck.shape[0]
+    ypad = (y + page - 1) // page * page
+    kh0 = lambda t: t[:, :1].float().cpu()
+    pad = lambda t: torch.cat([t, t.new_zeros(ypad - y, 1, D)], 0)
+    kc = torch.cat([kh0(k), pad(kh0(ck))], 0).view(-1, page, 1, D)
+    vc = torch.cat([kh0(v), pad(kh0(cv))], 0).view(-1, page, 1, D)
+    bt = torch.arange(T // page, dtype=torch.int32)[None]
+    cbt = (T // page + torch.arange(ypad // page, dtype=torch.int32))[None]
+    qs, ws = q[T - n:, :16].float().cpu(), w[T - n:, :16].float().cpu()
+    tk_dev = topk[:1, T - n:].cpu()
+    xcu, ctx = torch.tensor([0, n]), torch.tensor([T])
+    ref_o, parts = O.nsa_paged_forward(qs, kc, vc, ws, xcu, ctx, bt, cbt, topk=tk_dev, round_dtype=torch.bfloat16,
+                                       return_parts=True)
+    assert_close(out[T - n:, :16], ref_o, "o (last rows of the 262144-token run)")
+    own = O.select_blocks(parts[0]["imp"], torch.arange(T - n, T), 64, 16, 1, 2, -1)
+    n_rows, n_diff, n_bad = O.topk_mismatch_report(tk_dev, own, [parts[0]["imp"]], [0, n], 64, 16, tie_tol=1e-3,
+                                                   t_offsets=[T - n])
+    assert n_rows == n and n_bad == 0, (n_rows, n_diff, n_bad)
+
+
 def test_c2_prefix_consistency_and_oracle_slice(device):
     """T = 65536, 64q/4kv heads, d = 128 (benchmark configuration): forward + backward run; the first 4096 rows of the
     forward equal a 4096-token run (causality), and the first 1024 rows of kv group 0 match the oracle."""

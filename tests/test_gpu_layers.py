@@ -60,9 +60,11 @@ def test_rope_strided_views_and_broadcast_table(device):
     assert_close(ke, want_k.to(torch.bfloat16).float(), "ke", atol=2e-6, rtol=8e-3)
 
 
-def _layer_reference(x, cos, sin, weights, cfg_kw, cu, QH, KH, D, topk):
-    """x [b,s,hidden] fp32 on the CPU; projections as fp32 matmuls on bf16-rounded activations (the device rounds
-    q/k/v/w and o to bf16 between the stages), oracle RoPE and core."""
+def _layer_reference(x, cos, sin, weights, cfg_kw, cu, QH, KH, D, topk, d_out):
+    """Forward and backward of the layer on the CPU in fp32 with the pipeline's rounding points: every tensor the
+    device stores in bf16 between two stages (projection outputs, rotated q / k, the core's output and gradients,
+    the gradients handed back through RoPE and the projections) is rounded, the arithmetic in between is fp32.
+    -> (layer output, d hidden_states)"""
     wq, wk, wv, ww, wo = weights
     r = lambda t: t.to(torch.bfloat16).float()
     b, s, _ = x.shape
@@ -70,10 +72,17 @@ def _layer_reference(x, cos, sin, weights, cfg_kw, cu, QH, KH, D, topk):
     k = r(F.linear(x, wk)).view(b, s, KH, D)
     v = r(F.linear(x, wv)).view(b, s, KH, D)
     w = r(F.linear(x, ww)).view(b, s, QH, 3)
-    q, k = r(O.rope(q, cos, sin)), r(O.rope(k, cos, sin))
-    o = O.nsa_forward(q.flatten(0, 1), k.flatten(0, 1), v.flatten(0, 1), w.flatten(0, 1), cu,
-                      O.OracleConfig(**cfg_kw), topk=topk)
-    return F.linear(r(o).view(b, s, -1), wo)
+    ql, kl = q.clone().requires_grad_(), k.clone().requires_grad_()
+    qe, ke = O.rope(ql, cos, sin), O.rope(kl, cos, sin)
+    d_core = r(d_out @ wo).view(b * s, QH, D)
+    core = O.nsa_forward_backward(r(qe.detach()).flatten(0, 1), r(ke.detach()).flatten(0, 1), v.flatten(0, 1),
+                                  w.flatten(0, 1), d_core, cu, O.OracleConfig(**cfg_kw), topk=topk,
+                                  round_dtype=torch.bfloat16, round_mma=True)
+    out = F.linear(core["o"].view(b, s, -1), wo)
+    dq, dk = torch.autograd.grad([qe, ke], [ql, kl], [core["dq"].view_as(qe), core["dk"].view_as(ke)])
+    gx = (r(dq).flatten(2) @ wq + r(dk).flatten(2) @ wk + core["dv"].view(b, s, -1) @ wv +
+          core["dw"].view(b, s, -1) @ ww)
+    return out, gx
 
 
 @pytest.mark.parametrize("kind", ["hf", "megatron"])
@@ -113,12 +122,10 @@ def test_attention_layers_forward_backward(device, kind):
         ck = mean_pooling_fwd(kd.flatten(0, 1))
         _, lse = cmp_attn_fwd(qd.flatten(0, 1), ck, ck)
         topk, _ = slc_topk_indices(qd.flatten(0, 1), ck, lse)
-    xr = x.float().requires_grad_()
-    ref = _layer_reference(xr, cos, sin, weights, cfg_kw, cu, QH, KH, D, topk.cpu())
-    assert_close(out, ref, "layer output", atol=3e-2, rtol=2e-2)
     do = randn_bf16(b, s, hidden, seed=12)
+    ref_out, ref_gx = _layer_reference(x.float(), cos, sin, weights, cfg_kw, cu, QH, KH, D, topk.cpu(), do.float())
+    assert_close(out, ref_out, "layer output")
     out.backward(do.to(device))
-    ref.backward(do.float())
     gx = xd.grad if kind == "hf" else xd.grad.transpose(0, 1)
-    assert_close(gx, xr.grad, "d hidden_states", atol=5e-2, rtol=5e-2, row_scale=True)
+    assert_close(gx, ref_gx, "d hidden_states")
     NSAHelper.set_hyperparameters()

@@ -120,3 +120,12 @@ def test_split_decode_lds_budget_counts_static_arrays():
                         seen_near_limit += total > limit - 4288
                     prev_fit = bool(fits)
     assert seen_near_limit > 0, "the sweep must reach totals within the static part of the limit"
+
+
+def test_inverse_index_refuses_more_blocks_than_its_histogram_holds():
+    """The inverse index counts per selection block in an LDS histogram of 16384 entries: a batch with more blocks
+    (more than 1048576 tokens at 64 per block) is refused with a message instead of launched."""
+    from flash_nsa import _lib
+    with pytest.raises(RuntimeError, match="exceed the LDS histogram"):
+        _lib.call("nsa_build_inverse_index", None, 0, 0, 16, None, None, 1, 1 << 21, 4, 16385, 64, 1024, None, None,
+                  None, None, 0, None)

@@ -288,3 +288,167 @@ def test_rope_is_a_rotation_of_channel_pairs():
                 a, bb = x[b, n, 1, e], x[b, n, 1, H + e]
                 assert abs(out[b, n, 1, e] - (a * c2[b, n, e] - bb * s2[b, n, e])) < 1e-12
                 assert abs(out[b, n, 1, H + e] - (bb * c2[b, n, H + e] + a * s2[b, n, H + e])) < 1e-12
+
+
+# ------------------------------------------------------------------ the hand-written backward
+@pytest.mark.parametrize("methods", [("mean", "mean"), ("linear", "swiglu"), ("mean", "sigmoid-mul")])
+def test_hand_written_backward_equals_autograd_when_nothing_is_rounded(methods):
+    """nsa_forward_backward derives every gradient by hand (it has to: autograd cannot place a rounding inside the
+    softmax backward).  With rounding off it must be torch.autograd through nsa_forward, which pins its formulas
+    (a wrong sign, transpose, scale or a dropped branch shows up at 1e-9)."""
+    cu = [0, 150, 150, 190, 287]
+    T, QH, KH, D = 287, 4, 2, 16
+    cfg = O.OracleConfig(top_n=3, window_size=20, cmp_k_method=methods[0], cmp_v_method=methods[1])
+    q, k, v, w, do = [rand(*s, seed=10 + i) for i, s in
+                      enumerate([(T, QH, D), (T, KH, D), (T, KH, D), (T, QH, 3), (T, QH, D)])]
+    rows = {"mean": 0, "linear": D, "swiglu": 2 * D, "sigmoid-mul": 2 * D}
+    wk = rand(rows[methods[0]], 32 * D, seed=20) * 0.05 if methods[0] != "mean" else None
+    wv = rand(rows[methods[1]], 32 * D, seed=21) * 0.05 if methods[1] != "mean" else None
+    topk = O.slc_topk(q, O.compress(k, cu, methods[0], wk), None, cu, cfg)
+    leaves = [t.clone().requires_grad_() for t in (q, k, v, w)]
+    wkl = wk.clone().requires_grad_() if wk is not None else None
+    wvl = wv.clone().requires_grad_() if wv is not None else None
+    ro = O.nsa_forward(*leaves, cu, cfg, wk=wkl, wv=wvl, topk=topk)
+    ro.backward(do)
+    res = O.nsa_forward_backward(q, k, v, w, do, cu, cfg, topk=topk, wk=wk, wv=wv)
+    want = dict(o=ro.detach(), dq=leaves[0].grad, dk=leaves[1].grad, dv=leaves[2].grad, dw=leaves[3].grad,
+                dwk=None if wkl is None else wkl.grad, dwv=None if wvl is None else wvl.grad)
+    for name, ref in want.items():
+        if ref is None:
+            assert res[name] is None
+        else:
+            assert torch.allclose(res[name], ref, atol=1e-9, rtol=1e-9), name
+            assert float(ref.abs().max()) > 1e-3, f"{name}: the case must exercise this gradient"
+
+
+@pytest.mark.parametrize("kind", ["cmp", "slc", "swa"])
+def test_single_branch_backward_equals_autograd_when_nothing_is_rounded(kind):
+    cu = [0, 130, 130, 200]
+    T, QH, KH, D = 200, 4, 2, 8
+    cfg = O.OracleConfig(top_n=2, num_local_blocks=1, window_size=17)
+    q, k, v, do = [rand(*s, seed=30 + i) for i, s in enumerate([(T, QH, D), (T, KH, D), (T, KH, D), (T, QH, D)])]
+    topk = None
+    if kind == "cmp":
+        k, v = O.mean_pooling(k, cu), O.mean_pooling(v, cu)
+    if kind == "slc":
+        topk = O.slc_topk(q, O.mean_pooling(k, cu), None, cu, cfg)
+    ql, kl, vl = [t.clone().requires_grad_() for t in (q, k, v)]
+    if kind == "cmp":
+        o = O.cmp_attn(ql, kl, vl, cu)[0]
+    elif kind == "slc":
+        o = O.slc_attn(ql, kl, vl, topk, cu, cfg.block_size)[0]
+    else:
+        o = O.swa(ql, kl, vl, cu, cfg.window_size)[0]
+    o.backward(do)
+    res = O.branch_forward_backward(kind, q, k, v, do, cu, cfg, topk=topk)
+    for name, ref in (("o", o.detach()), ("dq", ql.grad), ("dk", kl.grad), ("dv", vl.grad)):
+        assert torch.allclose(res[name], ref, atol=1e-10), (kind, name)
+
+
+def test_rounding_points_explain_what_the_fp32_reference_cannot():
+    """Why the GPU tests compare with the reference that keeps the pipeline's rounding points.  The two CPU
+    references compared here are both exact arithmetic on the same bf16 inputs and differ only in whether the
+    tensors a bf16 pipeline stores between kernels (compressed rows, branch outputs and their gradients, the
+    correction term formed from them, P and dS as matrix operands) are rounded.  On a batch of short sequences they
+    agree within the parity bar on o, dq and the gate gradient, but are further apart than the bar in dv and, ten
+    times over, in the gradient of the compression weight (a sum over every compressed row of rounded terms).  No
+    kernel arithmetic is involved: that distance is the cost of the storage format, which upstream shares, and a
+    device that is correct to the last bit would fail the bar against the unrounded reference there."""
+    lens = [(37 * i * i + 11 * i) % 97 + 3 for i in range(24)]
+    cu = np.concatenate([[0], np.cumsum(lens)])
+    T, QH, KH, D = int(cu[-1]), 8, 1, 64
+    bf = lambda t: t.to(torch.bfloat16).float()
+    q, k, v, w, do = [bf(rand(*s, seed=40 + i, dtype=torch.float32)) for i, s in
+                      enumerate([(T, QH, D), (T, KH, D), (T, KH, D), (T, QH, 3), (T, QH, D)])]
+    wv = bf(rand(2 * D, 32 * D, seed=50, dtype=torch.float32) * 0.02)
+    cfg = O.OracleConfig(top_n=4, window_size=64, cmp_v_method="sigmoid-mul")
+    topk = O.slc_topk(q, O.mean_pooling(k, cu), None, cu, cfg)
+    pure = O.nsa_forward_backward(q, k, v, w, do, cu, cfg, topk=topk, wv=wv)
+    kept = O.nsa_forward_backward(q, k, v, w, do, cu, cfg, topk=topk, wv=wv, round_dtype=torch.bfloat16,
+                                  round_mma=True)
+
+    def worst(name, row_scale=False):
+        a, b = kept[name], pure[name]
+        mag = b.abs()
+        if row_scale:  # the relative base the GPU tests use for sums over many rows (dk, dv, weight gradients)
+            mag = torch.maximum(mag, b.pow(2).mean(-1, keepdim=True).sqrt())
+        return float(((a - b).abs() / (2e-2 + 1e-2 * mag)).max())
+
+    assert worst("o") < 1.0 and worst("dq") < 1.0 and worst("dw") < 1.0 and worst("dk") < 1.0
+    assert worst("dv") > 1.0 and worst("dv", row_scale=True) < 1.0
+    assert worst("dwv") > 3.0 and worst("dwv", row_scale=True) > 1.0
+
+
+# ------------------------------------------------------------------ helpers that GPU tests use as checkers
+@pytest.mark.parametrize("L", [32, 47, 48, 64, 4096])
+def test_paged_pool_decode_is_the_last_row_of_mean_pooling(L):
+    """The decode-step pooling writes exactly one row: the last row of mean_pooling over the request's gathered
+    tokens; nothing else in the pool changes, and a slot of -1 or a context shorter than the window writes nothing."""
+    page, H, D = 64, 2, 4
+    npg = (L + page - 1) // page
+    P = npg + 3
+    perm = torch.randperm(P, generator=torch.Generator().manual_seed(L))
+    cache = rand(P, page, H, D, seed=L)
+    bt = perm[:npg][None].to(torch.int32)
+    slot = int(perm[npg]) * page + 5
+    before = cache.clone()
+    O.paged_pool_decode(cache, torch.tensor([L]), bt, torch.tensor([slot]))
+    xs = O.gather_rows(before, bt[0], L)
+    want = O.mean_pooling(xs, [0, L])[-1]
+    flat, flat0 = cache.view(-1, H, D), before.view(-1, H, D)
+    assert torch.allclose(flat[slot], want, atol=1e-12)
+    # brute force of the same row: the window ends at the last multiple of the stride that fits
+    st = ((L - 32) // 16) * 16
+    assert torch.allclose(flat[slot], xs[st:st + 32].mean(0), atol=1e-12)
+    keep = torch.ones(P * page, dtype=torch.bool)
+    keep[slot] = False
+    assert torch.equal(flat[keep], flat0[keep])
+    again = before.clone()
+    O.paged_pool_decode(again, torch.tensor([L]), bt, torch.tensor([-1]))
+    assert torch.equal(again, before)
+    O.paged_pool_decode(again, torch.tensor([31]), bt, torch.tensor([slot]))
+    assert torch.equal(again, before)
+
+
+def test_topk_mismatch_report_hand_cases():
+    """One sequence of 200 tokens, one kv head, top-3.  Rows are built by hand: identical sets in another order
+    (no difference), a swap between two blocks whose scores differ by 5e-4 (differing, excused), a swap between
+    blocks whose scores differ by 0.5 (unexcused), an index beyond the row's last visible block (unexcused), and
+    a difference in a slot past the row's valid count (ignored)."""
+    T, N = 200, 3
+    imp = torch.zeros(1, T, 4)
+    imp[0, :, 0], imp[0, :, 1], imp[0, :, 2], imp[0, :, 3] = 0.9, 0.4, 0.4005, 0.1
+    base = torch.full((1, T, N), -1, dtype=torch.int32)
+    for t in range(T):
+        nk = t // 64
+        row = [0, nk, max(nk - 1, 0)][:min(N, nk + 1)]
+        base[0, t, :len(row)] = torch.tensor(row, dtype=torch.int32)
+    cu = [0, T]
+    assert O.topk_mismatch_report(base, base.clone(), [imp], cu, 64, N) == (T, 0, 0)
+    a = base.clone()
+    a[0, 150] = torch.tensor([1, 0, 2], dtype=torch.int32)          # same set {0,1,2}, other order
+    assert O.topk_mismatch_report(a, base, [imp], cu, 64, N) == (T, 0, 0)
+    b1, b2 = base.clone(), base.clone()
+    b1[0, 199] = torch.tensor([0, 3, 1], dtype=torch.int32)         # t=199: blocks 0..3 visible
+    b2[0, 199] = torch.tensor([0, 3, 2], dtype=torch.int32)         # differs in {1,2}: scores 0.4 vs 0.4005
+    assert O.topk_mismatch_report(b1, b2, [imp], cu, 64, N) == (T, 1, 0)
+    assert O.topk_mismatch_report(b1, b2, [imp], cu, 64, N, tie_tol=1e-4) == (T, 1, 1)
+    c = b1.clone()
+    c[0, 199] = torch.tensor([1, 3, 2], dtype=torch.int32)          # dropped block 0 (0.9) for block 2 (0.4005)
+    assert O.topk_mismatch_report(c, b1, [imp], cu, 64, N) == (T, 1, 1)
+    d = base.clone()
+    d[0, 100] = torch.tensor([0, 1, 3], dtype=torch.int32)          # t=100 sees blocks 0..1 only; block 3 is ahead
+    d[0, 100, 2] = 3
+    d2 = base.clone()
+    d2[0, 100, :2] = torch.tensor([0, 3], dtype=torch.int32)
+    assert O.topk_mismatch_report(d2, base, [imp], cu, 64, N) == (T, 1, 1)
+    e = base.clone()
+    e[0, 10, 1:] = 7                                                # t=10 has one valid slot; the rest is ignored
+    assert O.topk_mismatch_report(e, base, [imp], cu, 64, N) == (T, 0, 0)
+    f = base.clone()
+    f[0, 199, 1] = -1                                               # a negative index in a valid slot
+    assert O.topk_mismatch_report(f, base, [imp], cu, 64, N)[2] == 1
+    # with a prefix offset (paged prefill): local row 0 sits at position 130 and has three valid slots
+    off_a, off_b = base[:, 130:].clone(), base[:, 130:].clone()
+    off_b[0, 0] = torch.tensor([0, 2, 3], dtype=torch.int32)        # block 3 is beyond position 130
+    assert O.topk_mismatch_report(off_a, off_b, [imp[:, 130:]], [0, T - 130], 64, N, t_offsets=[130])[1:] == (1, 1)
