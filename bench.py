@@ -279,12 +279,31 @@ def cpu_baseline(min_seconds=12.0):
         fwd_s += t1 - t0
         bwd_s += t2 - t1
         reps += 1
+    # one more forward, stage by stage: the breakdown upstream prints with HFNSACore(bench=True)
+    # (flash_nsa/modules/hf_level_nsa.py:145-158): cmp_k, cmp_v, cmp_o, top_k, slc_o, swa_o, combine
+    stage_s = {}
+
+    def timed(name, fn):
+        t0 = time.perf_counter()
+        out = fn()
+        stage_s[name] = round(time.perf_counter() - t0, 4)
+        return out
+
+    with torch.no_grad():
+        cu, cfg = [0, T], O.OracleConfig()
+        ck = timed("cmp_k", lambda: O.mean_pooling(k, cu))
+        cv = timed("cmp_v", lambda: O.mean_pooling(v, cu))
+        cmp_o, cmp_lse = timed("cmp_o", lambda: O.cmp_attn(q, ck, cv, cu))
+        topk = timed("top_k", lambda: O.slc_topk(q, ck, cmp_lse, cu, cfg))
+        slc_o, _ = timed("slc_o", lambda: O.slc_attn(q, k, v, topk, cu))
+        swa_o, _ = timed("swa_o", lambda: O.swa(q, k, v, cu))
+        timed("combine", lambda: O.combine(cmp_o, slc_o, swa_o, w))
     fl = stage_flops([T], QH, D, D)
     total = (fl["fwd_total"] + fl["bwd_total"]) * reps
     return {"value": total / (fwd_s + bwd_s) / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
             "sample": f"{reps} forward+backward passes of the CPU oracle, T={T}, {QH}q/{KH}kv heads, d={D}, fp32, "
                       f"torch {torch.__version__} with {torch.get_num_threads()} threads",
-            "fwd_s": fwd_s / reps, "bwd_s": bwd_s / reps}
+            "fwd_s": fwd_s / reps, "bwd_s": bwd_s / reps, "fwd_stage_s": stage_s}
 
 
 def main():

@@ -10,58 +10,13 @@ import torch
 
 PEAK_HBM_GBS = 8000.0
 # bytes per step crossing the L2 <-> memory-side boundary (rocprofv3 --pmc FETCH_SIZE x2.000 + WRITE_SIZE x1.000, the
-# factors being what the counters read for a 1 GiB copy), measured for the default case of build_case()
+# factors being what the counters read for a 1 GiB copy), measured for the default case of build_decode_case()
 MEASURED_TRAFFIC_DEFAULT_CASE = 334.2e6
-
-
-def build_case(dev, B=64, QH=64, KH=4, D=128, page=256, lo=4096, hi=32768, seed=3):
-    g = torch.Generator().manual_seed(seed)
-    lens = torch.randint(lo, hi + 1, (B,), generator=g).tolist()
-    ys = [max((L - 32) // 16 + 1, 0) for L in lens]
-    n_raw = [(L + page - 1) // page for L in lens]
-    n_cmp = [max((y + page - 1) // page, 1) for y in ys]
-    P = sum(n_raw) + sum(n_cmp)
-    perm = torch.randperm(P, generator=g)
-    bt = torch.full((B, max(n_raw)), -1, dtype=torch.int32)
-    cbt = torch.full((B, max(n_cmp)), -1, dtype=torch.int32)
-    pos = 0
-    for b in range(B):
-        bt[b, :n_raw[b]] = perm[pos:pos + n_raw[b]].to(torch.int32)
-        pos += n_raw[b]
-        cbt[b, :n_cmp[b]] = perm[pos:pos + n_cmp[b]].to(torch.int32)
-        pos += n_cmp[b]
-    gd = torch.Generator(device=dev).manual_seed(seed)
-    k = torch.randn(P, page, KH, D, device=dev, generator=gd, dtype=torch.float32).to(torch.bfloat16)
-    v = torch.randn(P, page, KH, D, device=dev, generator=gd, dtype=torch.float32).to(torch.bfloat16)
-    q = torch.randn(B, QH, D, device=dev, generator=gd, dtype=torch.float32).to(torch.bfloat16)
-    w = torch.randn(B, QH, 3, device=dev, generator=gd, dtype=torch.float32).to(torch.bfloat16)
-    slots = []
-    for b, L in enumerate(lens):
-        if L >= 32 and (L - 32) % 16 == 0:
-            i = ys[b] - 1
-            slots.append(int(cbt[b, i // page]) * page + i % page)
-        else:
-            slots.append(-1)
-    ctx = torch.tensor(lens, dtype=torch.int32, device=dev)
-    return dict(q=q, k=k, v=v, w=w, ctx=ctx, bt=bt.to(dev), cbt=cbt.to(dev),
-                slots=torch.tensor(slots, dtype=torch.int32, device=dev), lens=lens, ys=ys, page=page)
 
 
 # Decode attention of one layer with a 4 GiB KV pool, batch = 4 GiB / (S * 4 kv heads * 2 (K,V) * 2 bytes * 128), every
 # request at context S, graph replay: microseconds the reference reports on one H800 (upstream README.md:291-300)
 REFERENCE_H800_DECODE_US = {4096: 689, 8192: 421, 16384: 279, 32768: 206, 65536: 172, 131072: 160}
-
-
-def pool_all_rows(c, dev):
-    """Pools every compressed row of the cached contexts of a build_case() dict (what earlier steps left behind)."""
-    from flash_nsa.inference import mean_pooling_prefill
-    B, page = len(c["lens"]), c["page"]
-    ycu = torch.zeros(B + 1, dtype=torch.int32)
-    ycu[1:] = torch.cumsum(torch.tensor(c["ys"]), 0)
-    slots = torch.cat([(c["cbt"][b].cpu()[torch.arange(y) // page].to(torch.int64) * page + torch.arange(y) % page)
-                       for b, y in enumerate(c["ys"])]).to(torch.int32).to(dev)
-    for cache in (c["k"], c["v"]):
-        mean_pooling_prefill(cache, ycu.to(dev), max(c["ys"]), c["bt"], slots)
 
 
 def decode_sweep(dev, lengths=(4096, 8192, 16384, 32768, 65536, 131072), reps=100):
@@ -72,9 +27,10 @@ def decode_sweep(dev, lengths=(4096, 8192, 16384, 32768, 65536, 131072), reps=10
     import json
     from flash_nsa import nsa_decode
     from flash_nsa.inference import auto_cmp_splits
+    from flash_nsa.inference.synthetic import build_decode_case, pool_all_rows
     for S in lengths:
         B = (4 << 30) // (S * 4 * 2 * 2 * 128)
-        c = build_case(dev, B=B, lo=S, hi=S, seed=5)
+        c = build_decode_case(dev, B=B, lo=S, hi=S, seed=5)
         pool_all_rows(c, dev)
         args = (c["q"], c["k"], c["v"], c["w"], c["ctx"], c["bt"], c["slots"], c["cbt"])
         kw = dict(fixed_y_maxlen=max(2048, (S // 16 + 255) // 256 * 256), fixed_num_slc_blocks=max(512, S // 64))
@@ -117,44 +73,56 @@ def algorithmic_bytes(lens, KH=4, D=128, VD=128, QH=64, top_n=16, block=64, wind
     return tot
 
 
-def decode_bench(dev, reps=200, warmup=20):
-    from flash_nsa import nsa_decode
-    from flash_nsa.inference import kv_mean_pooling_decode
-    c = build_case(dev)
-    args = (c["q"], c["k"], c["v"], c["w"], c["ctx"], c["bt"], c["slots"], c["cbt"])
-    kw = dict(fixed_y_maxlen=2048, fixed_num_slc_blocks=512)
-    # the compressed rows of the cached context are pooled once up front (every row, through the prefill pooling)
-    from flash_nsa.inference import mean_pooling_prefill
-    ycu = torch.zeros(len(c["lens"]) + 1, dtype=torch.int32)
-    ycu[1:] = torch.cumsum(torch.tensor(c["ys"]), 0)
-    page = c["page"]
-    all_slots = torch.cat([(c["cbt"][b].cpu()[torch.arange(y) // page].to(torch.int64) * page + torch.arange(y) % page)
-                           for b, y in enumerate(c["ys"])]).to(torch.int32).to(dev)
-    for cache in (c["k"], c["v"]):
-        mean_pooling_prefill(cache, ycu.to(dev), max(c["ys"]), c["bt"], all_slots)
-    eager = nsa_decode(*args, **kw)
-    torch.cuda.synchronize()
+def _capture(fn):
+    """Runs fn on a side stream (so that lazily created state exists), then captures it in a graph."""
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
         for _ in range(3):
-            nsa_decode(*args, **kw)
+            fn()
     torch.cuda.current_stream().wait_stream(side)
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-        out = nsa_decode(*args, **kw)
-    for _ in range(warmup):
-        graph.replay()
+        out = fn()
+    return graph, out
+
+
+def _time_replays(graphs, reps, warmup):
+    """Microseconds per replay, the graphs taken round-robin (one graph: every replay re-reads the same memory)."""
+    for i in range(warmup):
+        graphs[i % len(graphs)].replay()
     torch.cuda.synchronize()
     s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     s.record()
-    for _ in range(reps):
-        graph.replay()
+    for i in range(reps):
+        graphs[i % len(graphs)].replay()
     e.record()
     torch.cuda.synchronize()
-    us = s.elapsed_time(e) * 1e3 / reps
+    return s.elapsed_time(e) * 1e3 / reps
+
+
+def decode_bench(dev, reps=200, warmup=20, cold_copies=6):
+    """Hot: one graph replayed over one batch (its 342 MB of K/V can stay partly in the 256 MB memory-side cache between
+    replays).  Cold: `cold_copies` copies of the batch in disjoint memory, one graph each, replayed round-robin, so
+    that (cold_copies - 1) x 342 MB of other K/V pass through the caches before a copy is read again: every replay
+    streams its K/V from HBM."""
+    from flash_nsa import nsa_decode
+    from flash_nsa.inference.synthetic import build_decode_case, pool_all_rows
+    c = build_decode_case(dev)
+    pool_all_rows(c, dev)  # the compressed rows of the cached context, as earlier steps left them
+    kw = dict(fixed_y_maxlen=2048, fixed_num_slc_blocks=512)
+
+    def args_of(case):
+        return (case["q"], case["k"], case["v"], case["w"], case["ctx"], case["bt"], case["slots"], case["cbt"])
+
+    args = args_of(c)
+    eager = nsa_decode(*args, **kw)
+    torch.cuda.synchronize()
+    graph, out = _capture(lambda: nsa_decode(*args, **kw))
+    us = _time_replays([graph], reps, warmup)
     same = bool(torch.equal(out, eager))
     # eager (no graph) for comparison
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     s.record()
     for _ in range(20):
         nsa_decode(*args, **kw)
@@ -168,34 +136,35 @@ def decode_bench(dev, reps=200, warmup=20):
            "graph_equals_eager": same, "algorithmic_bytes": nbytes,
            "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                         "frac": gbs / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_DEFAULT_CASE}}
+    # cold: copies of the pool, tables and inputs at other addresses
+    copies = [c] + [dict(c, **{n: c[n].clone() for n in ("q", "k", "v", "w", "ctx", "bt", "slots", "cbt")})
+                    for _ in range(cold_copies - 1)]
+    graphs, outs = [graph], [out]
+    for cc in copies[1:]:
+        a = args_of(cc)
+        g, o = _capture(lambda a=a: nsa_decode(*a, **kw))
+        graphs.append(g)
+        outs.append(o)
+    cold_us = _time_replays(graphs, reps // len(graphs) * len(graphs), len(graphs) * 2)
+    cold_gbs = nbytes / (cold_us * 1e-6) / 1e9
+    res["us_per_step_cold"] = cold_us
+    res["cold_copies"] = len(graphs)
+    res["cold_equals_hot"] = all(bool(torch.equal(o, eager)) for o in outs)
+    res["roofline_cold"] = {"bound": "hbm", "achieved": cold_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                            "frac": cold_gbs / PEAK_HBM_GBS, "traffic": None}
+    del copies, graphs, outs
     # the same step with the cache write of the newest token's K/V inside the launch (KV-cache writer fused)
     page = c["page"]
-    B, KH, D = len(c["lens"]), c["k"].size(2), c["k"].size(3)
-    new_k = c["k"].view(-1, KH, D)[[int(c["bt"][b, (L - 1) // page]) * page + (L - 1) % page
-                                     for b, L in enumerate(c["lens"])]].clone()
-    new_v = c["v"].view(-1, KH, D)[[int(c["bt"][b, (L - 1) // page]) * page + (L - 1) % page
-                                     for b, L in enumerate(c["lens"])]].clone()
-    raw_slots = torch.tensor([int(c["bt"][b, (L - 1) // page]) * page + (L - 1) % page
-                              for b, L in enumerate(c["lens"])], dtype=torch.int32, device=dev)
+    KH, D = c["k"].size(2), c["k"].size(3)
+    newest = [int(c["bt"][b, (L - 1) // page]) * page + (L - 1) % page for b, L in enumerate(c["lens"])]
+    new_k = c["k"].view(-1, KH, D)[newest].clone()
+    new_v = c["v"].view(-1, KH, D)[newest].clone()
+    raw_slots = torch.tensor(newest, dtype=torch.int32, device=dev)
     kw2 = dict(kw, new_k=new_k, new_v=new_v, slot_mapping=raw_slots)
-    out2 = nsa_decode(*args, **kw2)
+    nsa_decode(*args, **kw2)
     torch.cuda.synchronize()
-    side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        nsa_decode(*args, **kw2)
-    torch.cuda.current_stream().wait_stream(side)
-    graph2 = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph2):
-        out2 = nsa_decode(*args, **kw2)
-    for _ in range(warmup):
-        graph2.replay()
-    torch.cuda.synchronize()
-    s.record()
-    for _ in range(reps):
-        graph2.replay()
-    e.record()
-    torch.cuda.synchronize()
-    res["us_per_step_with_cache_write"] = s.elapsed_time(e) * 1e3 / reps
+    graph2, out2 = _capture(lambda: nsa_decode(*args, **kw2))
+    res["us_per_step_with_cache_write"] = _time_replays([graph2], reps, warmup)
     res["cache_write_equals_plain"] = bool(torch.equal(out2, eager))
     return res
 
@@ -247,16 +216,6 @@ def cache_writer_bench(dev, reps=50):
 
 
 if __name__ == "__main__":
-    import json
-    import os
-    import sys
-    root = os.path.dirname(os.path.abspath(__file__))
-    sys.path.insert(0, os.path.join(root, "scalable-flash-native-sparse-attention_amd"))
-    print(json.dumps({"decode": decode_bench(torch.device("cuda:0")),
-                      "cache_writer": cache_writer_bench(torch.device("cuda:0"))}))
-
-
-if __name__ == "__main__":
     import argparse
     import json
     import os
@@ -270,4 +229,4 @@ if __name__ == "__main__":
     if a.sweep:
         decode_sweep(device)
     else:
-        print(json.dumps(decode_bench(device)))
+        print(json.dumps({"decode": decode_bench(device), "cache_writer": cache_writer_bench(device)}))

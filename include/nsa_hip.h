@@ -19,6 +19,12 @@ extern "C" {
 
 const char* nsa_last_error(void);
 int nsa_abi_version(void);
+/* Overrides one of the library's launch heuristics for this process (experiments and tests; nothing is read from
+ * the environment): name (host string) = "fwd_variant", "dq_min_blocks", "dkdv_key_blocks" or "topk_seg_blocks"
+ * (selection blocks per segment of the block selector: -1 = from the LDS budget, 0 = never segment).
+ * nsa_reset_tuning restores every default.  No upstream counterpart. */
+int nsa_set_tuning(const char* name, int value);
+int nsa_reset_tuning(void);
 
 /* flash_nsa/ops/compress_kv.py:335-366 mean_pooling_fwd */
 int nsa_mean_pool_fwd(const void* x, int64_t x_st, int64_t x_sh, void* y, int64_t y_st, int64_t y_sh,

@@ -4,6 +4,8 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <math.h>
+#include <string.h>
+#include <atomic>
 #include "nsa_common.h"
 #include "nsa_api_internal.h"
 
@@ -16,9 +18,29 @@ void nsa_set_error(const char* fmt, ...) {
   va_end(ap);
 }
 
-int nsa_tuning_knob(const char* env_name, int default_value) {
-  const char* v = getenv(env_name);
-  return (v && *v) ? atoi(v) : default_value;
+// Tuning values that a caller may override through nsa_set_tuning (never read from the environment).
+namespace {
+struct Knob {
+  const char* name;
+  std::atomic<int> value;
+  std::atomic<bool> is_set;
+};
+Knob g_knobs[] = {
+    {"fwd_variant", {0}, {false}},      // forward tile kernel: staging / rows per wave variant
+    {"dq_min_blocks", {0}, {false}},    // workgroups per CU of the dense dq kernel
+    {"dkdv_key_blocks", {0}, {false}},  // 32-key blocks per wave of the dense dk/dv kernel
+    {"topk_seg_blocks", {0}, {false}},  // selection blocks per segment of the block selector
+};
+Knob* find_knob(const char* name) {
+  for (Knob& k : g_knobs)
+    if (strcmp(k.name, name) == 0) return &k;
+  return nullptr;
+}
+}  // namespace
+
+int nsa_tuning_knob(const char* name, int default_value) {
+  Knob* k = find_knob(name);
+  return (k && k->is_set.load()) ? k->value.load() : default_value;
 }
 
 int nsa_check_launch(const char* what) {
@@ -53,6 +75,19 @@ extern "C" {
 
 const char* nsa_last_error(void) { return g_err; }
 int nsa_abi_version(void) { return 1; }
+
+int nsa_set_tuning(const char* name, int value) {
+  Knob* k = name ? find_knob(name) : nullptr;
+  NSA_REQUIRE(k != nullptr, NSA_ERR_BAD_ARG, "set_tuning: unknown name '%s' (fwd_variant, dq_min_blocks, "
+              "dkdv_key_blocks, topk_seg_blocks)", name ? name : "(null)");
+  k->value.store(value);
+  k->is_set.store(true);
+  return NSA_OK;
+}
+int nsa_reset_tuning(void) {
+  for (Knob& k : g_knobs) k.is_set.store(false);
+  return NSA_OK;
+}
 
 int nsa_cmp_attn_fwd(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr, int64_t ck_sh,
                      const void* cv, int64_t cv_sr, int64_t cv_sh, void* o, int64_t o_st, int64_t o_sh, float* lse,

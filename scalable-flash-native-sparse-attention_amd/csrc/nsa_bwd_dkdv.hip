@@ -486,7 +486,7 @@ template <int D, int VD>
 int launch(const NsaBwdTileParams& p0, int mode, int B, int max_q_len, int max_k_len, int n_items_bound,
            hipStream_t stream) {
   NsaBwdTileParams p = p0;
-  static const int kb_cmp = nsa_tuning_knob("NSA_DKDV_KB", 1);  // 32-key blocks per wave of the cmp / swa kernels
+  const int kb_cmp = nsa_tuning_knob("dkdv_key_blocks", 1);  // 32-key blocks per wave of the cmp / swa kernels
   if (mode == MODE_CMP) {
     if (B <= 0 || max_k_len <= 0) return NSA_OK;
     const int KW = 4 * 32 * (kb_cmp == 2 ? 2 : 1);

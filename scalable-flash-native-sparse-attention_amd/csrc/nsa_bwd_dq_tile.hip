@@ -229,7 +229,7 @@ template <int MODE>
 int dispatch(const NsaBwdTileParams& p, int B, int max_q_len, int D, int VD, hipStream_t stream) {
   if (B <= 0 || max_q_len <= 0) return NSA_OK;
   dim3 grid(cdiv_i(max_q_len * p.G, 128), B, p.KH);
-  static const int minb = nsa_tuning_knob("NSA_DQ_MINB", 2);
+  const int minb = nsa_tuning_knob("dq_min_blocks", 2);
   if (D == 128 && VD == 128) {
     if (minb == 2) bwd_dq_tile_kernel<128, 128, MODE, 2, true><<<grid, 256, 0, stream>>>(p);
     else bwd_dq_tile_kernel<128, 128, MODE, 1, false><<<grid, 256, 0, stream>>>(p);

@@ -159,7 +159,7 @@ enum {
 };
 
 void nsa_set_error(const char* fmt, ...);
-int nsa_tuning_knob(const char* env_name, int default_value);  // integer tuning override read from the environment
+int nsa_tuning_knob(const char* name, int default_value);  // value given to nsa_set_tuning for this name, else the default
 int nsa_check_launch(const char* what);
 
 #define NSA_REQUIRE(cond, code, ...)        \

@@ -393,7 +393,7 @@ int launch_fwd_tile(const NsaFwdTileParams& p, int B, int max_q_len, hipStream_t
   // 0 (default): direct-to-LDS staging for the compressed branch with power-of-two head dims (4.5 % faster there;
   // the window branch, with its short key loops, and d=192, whose swizzled addresses cost registers, are faster with
   // register staging); 1..4 force one variant for experiments
-  static const int variant = nsa_tuning_knob("NSA_FWD_VARIANT", 0);
+  const int variant = nsa_tuning_knob("fwd_variant", 0);
   constexpr bool pow2 = (D == 64 || D == 128) && (VD == 64 || VD == 128);
   const bool async = variant == 4 || (variant == 0 && MODE == MODE_CMP && pow2);
   if (variant == 2) {

@@ -481,8 +481,8 @@ int launch_topk(const NsaTopkParams& p_in, int B, int max_q_len, hipStream_t str
   NsaTopkParams p = p_in;
   const size_t stat = 128 * (D + NSA_LDS_PAD) * 2 + 2 * TWG * 132 * 4;
   // One pass while the score rows of all blocks leave room for two workgroups per CU; else segments of the largest
-  // whole number of key tiles that does.  NSA_TOPK_SEG_BLOCKS forces a segment length (0 = never segment).
-  const int forced_seg = nsa_tuning_knob("NSA_TOPK_SEG_BLOCKS", -1);
+  // whole number of key tiles that does.  The tuning value topk_seg_blocks forces a segment length (0 = never segment).
+  const int forced_seg = nsa_tuning_knob("topk_seg_blocks", -1);
   const size_t budget = 80 * 1024;
   size_t dyn = (size_t)TWG * p.nb_max * sizeof(float);
   p.seg_blocks = 0;

@@ -3,7 +3,6 @@ across the three branches and optional recomputation of saved activations
 (mirrors the interface of upstream flash_nsa/modules/megatron_level_nsa.py:46-159, 386-545; the
 context-parallel function of that file is outside this single-GPU build)."""
 import math
-import os
 
 import torch
 
@@ -21,8 +20,8 @@ from ..ops.sliding_window_attention import swa_fwd, swa_bwd
 # The backward runs on two streams: the memory-bound selected-block dq kernel leaves the matrix cores idle and the
 # dense dk/dv kernels leave the memory side idle, so the dq chain (window -> selected -> compressed) runs next to the
 # dk/dv kernels (measured: about 1 ms of a 75 ms step; the same split of the forward gained nothing).
-# NSA_OVERLAP_STREAMS=0 puts everything back on the caller's stream.
-OVERLAP_STREAMS = os.environ.get("NSA_OVERLAP_STREAMS", "1") != "0"
+# Setting this module attribute to False puts everything back on the caller's stream.
+OVERLAP_STREAMS = True
 _side_streams = {}
 
 

@@ -119,9 +119,9 @@ def test_topk_and_slc_fwd(device, lens, QH, KH, D):
                                           ([5000, 3000], 4, 2, 128), ([4500], 64, 1, 64)])
 def test_topk_segmented_selection_equals_one_pass(device, lens, QH, KH, D):
     """Long contexts keep the block scores of one segment of blocks in LDS and merge every finished segment into a
-    running list of winners.  The segment length (an integer tuning variable read at every launch) must not change
+    running list of winners.  The segment length (a tuning value set through nsa_set_tuning) must not change
     the result: indices and returned scores are bit-identical to the one-pass selector, and match the oracle."""
-    import os
+    from flash_nsa import _lib
     from flash_nsa.ops.compress_kv import mean_pooling_fwd
     from flash_nsa.ops.compress_attn import cmp_attn_fwd
     from flash_nsa.ops.topk import slc_topk_indices
@@ -138,10 +138,10 @@ def test_topk_segmented_selection_equals_one_pass(device, lens, QH, KH, D):
         for seg in (0, 32, 64, 96):
             if seg == 0 and G <= 2:
                 continue  # the score rows of 64 / 32 tokens per workgroup do not fit in one pass at this length
-            os.environ["NSA_TOPK_SEG_BLOCKS"] = str(seg)
+            _lib.call("nsa_set_tuning", b"topk_seg_blocks", seg)
             results[seg] = slc_topk_indices(qd, ck, lse, return_slc_prob=True)
     finally:
-        os.environ.pop("NSA_TOPK_SEG_BLOCKS", None)
+        _lib.call("nsa_reset_tuning")
     results["auto"] = slc_topk_indices(qd, ck, lse, return_slc_prob=True)
     keys = list(results)
     for key in keys[1:]:

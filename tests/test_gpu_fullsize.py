@@ -101,8 +101,7 @@ def test_long_context_262144_tokens(device):
     o and dq bit-equal to a 4096-token run (causality), the last 64 rows of kv group 0 against the oracle (their
     selection compared with the oracle's own, their output with the device's selection), and the block selector
     forced to work in short segments returns the same indices as the default at this length."""
-    import os
-    from flash_nsa import NSAConfig, NSACore, NSAHelper
+    from flash_nsa import NSAConfig, NSACore, NSAHelper, _lib
     from flash_nsa.ops.compress_kv import mean_pooling_fwd
     from flash_nsa.ops.compress_attn import cmp_attn_fwd
     from flash_nsa.ops.topk import slc_topk_indices
@@ -130,10 +129,10 @@ def test_long_context_262144_tokens(device):
         _, lse = cmp_attn_fwd(q, ck, cv)
         topk, _ = slc_topk_indices(q, ck, lse)
         try:
-            os.environ["NSA_TOPK_SEG_BLOCKS"] = "512"
+            _lib.call("nsa_set_tuning", b"topk_seg_blocks", 512)
             topk_seg, _ = slc_topk_indices(q, ck, lse)
         finally:
-            os.environ.pop("NSA_TOPK_SEG_BLOCKS", None)
+            _lib.call("nsa_reset_tuning")
     assert torch.equal(topk, topk_seg), "segment length changed the selection"
     # the last n rows of kv group 0 against the oracle: the sequence laid out as a paged pool with identity tables
     page = 256
@@ -281,12 +280,10 @@ def _decode_block_scores(c, kh, b, device, G=16, D=128, block=64, kernel=32, str
 def test_c5_decode_full_batch(device):
     """Batch 64, contexts uniform in [4096, 32768], page 256, random page permutation (benchmark configuration):
     fused decode == stage-by-stage decode; one request re-checked as a one-token paged prefill; graph replay."""
-    import sys, os
-    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
-    import bench_decode as bd
     from flash_nsa import nsa_decode, nsa_prefill
     from flash_nsa.inference import nsa_decode_staged, mean_pooling_prefill
-    c = bd.build_case(device)
+    from flash_nsa.inference.synthetic import build_decode_case
+    c = build_decode_case(device)
     page = c["page"]
     ycu = torch.zeros(65, dtype=torch.int32)
     ycu[1:] = torch.cumsum(torch.tensor(c["ys"]), 0)

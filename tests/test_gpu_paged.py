@@ -97,12 +97,12 @@ def test_chunked_prefill_equals_one_shot(device):
         assert torch.equal(one[b], four[b]), f"request {b}: chunked prefill differs from one-shot"
     assert torch.equal(d1["k"], d4["k"]) and torch.equal(d1["v"], d4["v"]), "pooled cache rows differ"
     # the paged block selector working segment by segment (as it does for contexts whose score rows do not fit LDS)
-    import os
-    os.environ["NSA_TOPK_SEG_BLOCKS"] = "32"
+    from flash_nsa import _lib
+    _lib.call("nsa_set_tuning", b"topk_seg_blocks", 32)
     try:
         seg, _ = run(4)
     finally:
-        os.environ.pop("NSA_TOPK_SEG_BLOCKS", None)
+        _lib.call("nsa_reset_tuning")
     for b in range(len(ctx)):
         assert torch.equal(one[b], seg[b]), f"request {b}: segmented block selection changed the prefill"
 

@@ -129,3 +129,11 @@ def test_inverse_index_refuses_more_blocks_than_its_histogram_holds():
     with pytest.raises(RuntimeError, match="exceed the LDS histogram"):
         _lib.call("nsa_build_inverse_index", None, 0, 0, 16, None, None, 1, 1 << 21, 4, 16385, 64, 1024, None, None,
                   None, None, 0, None)
+
+
+def test_tuning_values_are_set_by_name_not_by_environment():
+    from flash_nsa import _lib
+    _lib.call("nsa_set_tuning", b"topk_seg_blocks", 64)
+    _lib.call("nsa_reset_tuning")
+    with pytest.raises(RuntimeError, match="unknown name"):
+        _lib.call("nsa_set_tuning", b"no_such_value", 1)
