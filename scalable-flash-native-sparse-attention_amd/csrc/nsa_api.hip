@@ -166,8 +166,8 @@ int nsa_slc_attn_fwd(const void* q, int64_t q_st, int64_t q_sh, const void* k, i
                      int top_n, float sm_scale, void* stream) {
   int rc = check_heads("slc_attn_fwd", QH, KH, D, VD);
   if (rc) return rc;
-  NSA_REQUIRE(block_size % 64 == 0 && block_size > 0, NSA_ERR_UNSUPPORTED,
-              "slc_attn_fwd: block_size %d must be a multiple of 64", block_size);
+  NSA_REQUIRE(block_size % 32 == 0 && block_size > 0, NSA_ERR_UNSUPPORTED,
+              "slc_attn_fwd: block_size %d must be a multiple of 32", block_size);
   NSA_REQUIRE(top_n >= 1 && top_n <= 64, NSA_ERR_BAD_ARG, "slc_attn_fwd: top_n %d must be in [1,64]", top_n);
   NsaSlcParams p{};
   p.q = (const bf16_t*)q; p.q_st = q_st; p.q_sh = q_sh;
@@ -361,8 +361,8 @@ int nsa_slc_attn_bwd_dq(const void* q, int64_t q_st, int64_t q_sh, const void* k
                         int KH, int D, int VD, int block_size, int top_n, float sm_scale, void* stream) {
   int rc = check_heads("slc_attn_bwd_dq", QH, KH, D, VD);
   if (rc) return rc;
-  NSA_REQUIRE(block_size % 64 == 0 && block_size > 0, NSA_ERR_UNSUPPORTED,
-              "slc_attn_bwd_dq: block_size %d must be a multiple of 64", block_size);
+  NSA_REQUIRE(block_size % 32 == 0 && block_size > 0, NSA_ERR_UNSUPPORTED,
+              "slc_attn_bwd_dq: block_size %d must be a multiple of 32", block_size);
   NSA_REQUIRE(top_n >= 1 && top_n <= 64, NSA_ERR_BAD_ARG, "slc_attn_bwd_dq: top_n %d must be in [1,64]", top_n);
   NSA_REQUIRE(dq_mode >= 0 && dq_mode <= 2, NSA_ERR_BAD_ARG, "slc_attn_bwd_dq: dq_mode %d not in {0,1,2}", dq_mode);
   NsaSlcBwdDqParams p{};
@@ -390,8 +390,8 @@ int nsa_slc_attn_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void*
                           int QH, int KH, int D, int VD, int block_size, float sm_scale, void* stream) {
   int rc = check_heads("slc_attn_bwd_dkdv", QH, KH, D, VD);
   if (rc) return rc;
-  NSA_REQUIRE(block_size == 64 || block_size == 128, NSA_ERR_UNSUPPORTED,
-              "slc_attn_bwd_dkdv: block_size %d not built (64 or 128)", block_size);
+  NSA_REQUIRE(block_size % 32 == 0 && block_size > 0, NSA_ERR_UNSUPPORTED,
+              "slc_attn_bwd_dkdv: block_size %d must be a multiple of 32", block_size);
   BwdCommon c{q, q_st, q_sh, k, k_sr, k_sh, v, v_sr, v_sh, dO, do_st, do_sh, lse, lse_st, lse_sh, delta, delta_st,
               delta_sh};
   NsaBwdTileParams p = make_bwd(c, QH, KH, sm_scale);
@@ -508,8 +508,8 @@ int nsa_paged_slc_attn_fwd(const void* q, int64_t q_st, int64_t q_sh, const void
   if (rc) return rc;
   rc = check_page("paged_slc_attn_fwd", page_size);
   if (rc) return rc;
-  NSA_REQUIRE(block_size % 64 == 0 && block_size > 0, NSA_ERR_UNSUPPORTED,
-              "paged_slc_attn_fwd: block_size %d must be a multiple of 64", block_size);
+  NSA_REQUIRE(block_size % 32 == 0 && block_size > 0, NSA_ERR_UNSUPPORTED,
+              "paged_slc_attn_fwd: block_size %d must be a multiple of 32", block_size);
   NSA_REQUIRE(top_n >= 1 && top_n <= 64, NSA_ERR_BAD_ARG, "paged_slc_attn_fwd: top_n %d must be in [1,64]", top_n);
   NsaSlcParams p{};
   p.q = (const bf16_t*)q; p.q_st = q_st; p.q_sh = q_sh;

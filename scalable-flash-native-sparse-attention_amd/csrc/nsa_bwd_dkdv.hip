@@ -61,7 +61,8 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
     const int jb = lo;
     const int c = w - ioff[jb];
     b = p.blk_seq[jb];
-    key0 = (jb - p.kblk_cu[b]) * p.block_size;
+    // a selection block wider than the workgroup's NW*32 keys is cut into sub-blocks over grid.y (same token list)
+    key0 = (jb - p.kblk_cu[b]) * p.block_size + blockIdx.y * (NW * 32 * KB);
     const int s0 = p.csr_off[(int64_t)kh * (p.nblk_total + 1) + jb];
     const int s1 = p.csr_off[(int64_t)kh * (p.nblk_total + 1) + jb + 1];
     const int a = s0 + c * p.chunk_tokens;
@@ -98,6 +99,9 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
   } else {
     kbase = x0;
     nkeys = xl;
+    // MODE_SLC: the workgroup's keys end with its selection block (a block narrower than NW*32 keys, or the last
+    // sub-block of a wide one, leaves the upper waves without keys)
+    if (MODE == MODE_SLC) nkeys = min(xl, (key0 / p.block_size + 1) * p.block_size);
     if (MODE == MODE_SWA) {
       key0 = blockIdx.x * KW;
       if (key0 >= nkeys) return;
@@ -511,12 +515,18 @@ int launch(const NsaBwdTileParams& p0, int mode, int B, int max_q_len, int max_k
     }
   } else {
     if (n_items_bound <= 0) return NSA_OK;
-    dim3 grid(n_items_bound, 1, p.KH);
-    if (p.block_size == 64) bwd_dkdv_kernel<D, VD, MODE_SLC, 2, 1><<<grid, 128, 0, stream>>>(p);
-    else if (p.block_size == 128) bwd_dkdv_kernel<D, VD, MODE_SLC, 4, 1><<<grid, 256, 0, stream>>>(p);
-    else {
-      nsa_set_error("selected attention dk/dv: block_size %d not built (64 or 128)", p.block_size);
+    if (p.block_size <= 0 || p.block_size % 32 != 0) {
+      nsa_set_error("selected attention dk/dv: block_size %d must be a multiple of 32", p.block_size);
       return NSA_ERR_UNSUPPORTED;
+    }
+    // a workgroup owns 64 keys (blocks of 32 or 64) or 128 keys (wider blocks, cut into sub-blocks over grid.y);
+    // waves whose 32 keys lie past the end of the block only help staging the query rows
+    if (p.block_size <= 64) {
+      dim3 grid(n_items_bound, 1, p.KH);
+      bwd_dkdv_kernel<D, VD, MODE_SLC, 2, 1><<<grid, 128, 0, stream>>>(p);
+    } else {
+      dim3 grid(n_items_bound, cdiv_i(p.block_size, 128), p.KH);
+      bwd_dkdv_kernel<D, VD, MODE_SLC, 4, 1><<<grid, 256, 0, stream>>>(p);
     }
   }
   return nsa_check_launch("bwd_dkdv_kernel");

@@ -8,6 +8,24 @@ def _is_pow2(n: int) -> bool:
     return n > 0 and (n & (n - 1)) == 0
 
 
+# (qk head dim, v head dim) pairs the kernels are built for
+SUPPORTED_HEAD_DIMS = ((128, 128), (64, 64), (192, 128))
+
+
+def check_supported(qk_head_dim, v_head_dim, kernel_size, stride, block_size):
+    """The constraints of upstream (flash_nsa/config.py:48-52) plus the ones of this build's kernels, checked where a
+    model is configured so that an unsupported shape fails there and not at its first launch."""
+    assert _is_pow2(stride), "stride must be a power of 2"
+    assert kernel_size % stride == 0, "kernel_size must be a multiple of stride"
+    assert block_size >= kernel_size, "block_size must be >= kernel_size"
+    assert block_size % stride == 0, "block_size must be a multiple of stride"
+    assert block_size % 32 == 0, (
+        f"block_size {block_size}: the selected-attention kernels work in units of 32 keys; block sizes that are "
+        "multiples of 32 are supported (32, 64, 96, 128, 256, ...)")
+    assert (qk_head_dim, v_head_dim) in SUPPORTED_HEAD_DIMS, (
+        f"head dims qk={qk_head_dim} / v={v_head_dim} are not built; supported (qk, v) pairs: {SUPPORTED_HEAD_DIMS}")
+
+
 @dataclass
 class NSAConfig:
     hidden_size: int = 4096
@@ -49,6 +67,7 @@ class NSAConfig:
             assert self.head_dim is not None
             self.v_head_dim = self.head_dim
         assert self.num_heads % self.num_kv_heads == 0
+        check_supported(self.qk_head_dim, self.v_head_dim, self.kernel_size, self.stride, self.block_size)
 
     @classmethod
     def from_json(cls, json_file: str):

@@ -1,10 +1,9 @@
 """HuggingFace-level NSA core: one autograd node per stage, learned or mean KV compression
 (mirrors the interface of upstream flash_nsa/modules/hf_level_nsa.py:17-158)."""
-import math
 
 import torch
 
-from ..config import NSAConfig
+from ..config import NSAConfig, check_supported
 from ..utils import NSAHelper
 from ..ops.compress_kv import construct_block, mean_pooling
 from ..ops.compress_attn import compress_attn
@@ -58,9 +57,8 @@ class HFNSACore(torch.nn.Module):
         self.num_local_blocks = getattr(config, "num_local_blocks", 2)
         self.window_size = getattr(config, "window_size", 512)
         self.sm_scale = self.qk_head_dim ** -0.5
-        assert math.log2(self.stride).is_integer(), "stride must be a power of 2"
-        assert self.kernel_size % self.stride == 0
-        assert self.block_size % self.stride == 0
+        # the core also accepts config objects other than NSAConfig (any object with these attributes): validate here too
+        check_supported(self.qk_head_dim, self.v_head_dim, self.kernel_size, self.stride, self.block_size)
         self._set_helper()
         self.compress_k = CompressKV(config, head_dim=self.qk_head_dim, version=config.cmp_k_method)
         self.compress_v = CompressKV(config, head_dim=self.v_head_dim, version=config.cmp_v_method)

@@ -6,7 +6,7 @@ import math
 
 import torch
 
-from ..config import NSAConfig
+from ..config import NSAConfig, check_supported
 from ..utils import NSAHelper
 from ..ops.compress_kv import construct_block_fwd, construct_block_bwd, mean_pooling_fwd, mean_pooling_bwd
 from ..ops.compress_attn import cmp_attn_fwd, cmp_attn_bwd
@@ -202,9 +202,8 @@ class NSACore(torch.nn.Module):
                               recompute_slc_o=g("recompute_slc_o", False), recompute_swa_o=g("recompute_swa_o", False))
         self.pp_size = pp_size
         self.sm_scale = self.qk_head_dim ** -0.5
-        assert math.log2(self.stride).is_integer(), "stride must be a power of 2"
-        assert self.kernel_size % self.stride == 0
-        assert self.block_size % self.stride == 0
+        # the core also accepts config objects other than NSAConfig (any object with these attributes): validate here too
+        check_supported(self.qk_head_dim, self.v_head_dim, self.kernel_size, self.stride, self.block_size)
         self._set_helper()
 
         def make_weight(method, dim):

@@ -228,6 +228,13 @@ def test_nsa_core_fwd_bwd(device, core, lens, QH, KH, D, methods):
     dict(top_n=64, window_size=64),                                   # more slots than most tokens have blocks
     dict(top_n=1, num_init_blocks=0, num_local_blocks=1),             # the token's own block only
     dict(top_n=2, num_init_blocks=1, num_local_blocks=1, window_size=0),  # window = the token itself
+    # selection blocks other than 64 / 128 (upstream accepts every block >= kernel that is a multiple of the stride;
+    # this build: every multiple of 32)
+    dict(kernel_size=32, stride=16, block_size=32, top_n=12, window_size=64),
+    dict(kernel_size=32, stride=8, block_size=32, top_n=6, window_size=100),
+    dict(kernel_size=32, stride=16, block_size=96, top_n=5, window_size=64),
+    dict(kernel_size=64, stride=16, block_size=256, top_n=3, window_size=128),
+    dict(kernel_size=32, stride=32, block_size=160, top_n=4, num_local_blocks=1, window_size=32),
 ])
 def test_nsa_core_other_hyperparameters(device, hp):
     """Compression window / stride, selection block, top-n, forced blocks and window other than the defaults

@@ -112,6 +112,9 @@ def test_chunked_prefill_equals_one_shot(device):
     dict(kernel_size=64, stride=32, block_size=128, top_n=4, window_size=256),
     dict(kernel_size=32, stride=8, block_size=64, top_n=16, window_size=512),
     dict(kernel_size=16, stride=16, block_size=64, top_n=3, window_size=1, num_init_blocks=0, num_local_blocks=1),
+    dict(kernel_size=32, stride=16, block_size=32, top_n=12, window_size=64),
+    dict(kernel_size=64, stride=16, block_size=256, top_n=3, window_size=128),
+    dict(kernel_size=32, stride=16, block_size=96, top_n=5, window_size=64),
 ])
 def test_prefill_with_cached_prefix_equals_training_rows(device, hp):
     """Prefill of new tokens behind a cached prefix, default and other compression / block / top-n / window settings:
@@ -164,6 +167,9 @@ def _prefill_equals_training_rows(device, QH, KH, D, page, cached, new, hp):
     dict(kernel_size=64, stride=16, block_size=64, top_n=5, window_size=100),
     dict(kernel_size=32, stride=8, block_size=64, top_n=16, window_size=512),
     dict(kernel_size=16, stride=16, block_size=64, top_n=3, window_size=1, num_init_blocks=0, num_local_blocks=1),
+    dict(kernel_size=32, stride=16, block_size=32, top_n=12, window_size=64),
+    dict(kernel_size=64, stride=16, block_size=256, top_n=3, window_size=128),
+    dict(kernel_size=32, stride=16, block_size=96, top_n=5, window_size=64),
 ])
 def test_decode_other_hyperparameters_equals_training_row(device, hp):
     """Decode with compression, block, top-n, forced-block and window settings other than the defaults: every
@@ -181,11 +187,12 @@ def test_decode_other_hyperparameters_equals_training_row(device, hp):
     q, w = randn_bf16(B, QH, D, seed=8), randn_bf16(B, QH, 3, seed=9)
     d = to_dev(case, device)
     ctx_t = torch.tensor(ctx, dtype=torch.int32).to(device)
+    nb_cap = max(32, -(-max(ctx) // hp["block_size"]))  # capacity: at least the blocks of the longest context
     try:
         o = nsa_decode(q.to(device), d["k"], d["v"], w.to(device), ctx_t, d["bt"], slots.to(device), d["cbt"],
-                       fixed_y_maxlen=256, fixed_num_slc_blocks=32, **hp)
+                       fixed_y_maxlen=256, fixed_num_slc_blocks=nb_cap, **hp)
         o2 = nsa_decode_staged(q.to(device), d["k"], d["v"], w.to(device), ctx_t, d["bt"], d["cbt"],
-                               fixed_y_maxlen=256, fixed_num_slc_blocks=32, **hp)
+                               fixed_y_maxlen=256, fixed_num_slc_blocks=nb_cap, **hp)
         assert_close(o, o2, "one-launch vs stage-by-stage decode", atol=1e-2, rtol=1e-2)
         core = NSACore(NSAConfig(head_dim=D, num_heads=QH, num_kv_heads=KH, **hp))
         for b in range(B):

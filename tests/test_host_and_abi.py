@@ -137,3 +137,28 @@ def test_tuning_values_are_set_by_name_not_by_environment():
     _lib.call("nsa_reset_tuning")
     with pytest.raises(RuntimeError, match="unknown name"):
         _lib.call("nsa_set_tuning", b"no_such_value", 1)
+
+
+def test_unsupported_shapes_are_rejected_where_the_model_is_configured():
+    """Block sizes that are not multiples of 32 and head dims that are not built fail in NSAConfig and in both
+    cores' constructors (also for a plain attribute object), not at the first launch in the middle of a forward."""
+    from types import SimpleNamespace
+    from flash_nsa import NSAConfig, NSACore, HFNSACore
+    NSAConfig(block_size=32)
+    NSAConfig(block_size=256, kernel_size=64)
+    NSAConfig(qk_head_dim=192, v_head_dim=128)
+    with pytest.raises(AssertionError, match="multiples of 32"):
+        NSAConfig(block_size=48)
+    with pytest.raises(AssertionError, match="not built"):
+        NSAConfig(head_dim=256)
+    with pytest.raises(AssertionError, match="not built"):
+        NSAConfig(head_dim=32)
+    loose = SimpleNamespace(head_dim=128, qk_head_dim=None, v_head_dim=None, num_heads=16, num_kv_heads=1,
+                            kernel_size=32, stride=16, block_size=80, cmp_k_method="mean", cmp_v_method="mean")
+    for core in (NSACore, HFNSACore):
+        with pytest.raises(AssertionError, match="multiples of 32"):
+            core(loose)
+    loose.block_size, loose.head_dim = 64, 96
+    for core in (NSACore, HFNSACore):
+        with pytest.raises(AssertionError, match="not built"):
+            core(loose)
