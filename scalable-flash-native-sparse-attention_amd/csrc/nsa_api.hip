@@ -741,6 +741,8 @@ int nsa_decode_fused(const void* q, int64_t q_st, int64_t q_sh, const void* k_ca
   NSA_REQUIRE(QH / KH <= 16, NSA_ERR_UNSUPPORTED, "decode_fused: at most 16 q-heads per kv head (got %d)", QH / KH);
   NSA_REQUIRE(block_size % 32 == 0, NSA_ERR_UNSUPPORTED, "decode_fused: block_size %d must be a multiple of 32",
               block_size);
+  NSA_REQUIRE(o_st % 4 == 0 && o_sh % 4 == 0 && co_st % 4 == 0 && co_sh % 4 == 0, NSA_ERR_BAD_ARG,
+              "decode_fused: output strides must be multiples of 4 elements (8-byte stores)");
   NSA_REQUIRE(top_n >= 1 && top_n <= 64 && num_init >= 0 && num_local >= 0 && num_init + num_local <= top_n,
               NSA_ERR_BAD_ARG, "decode_fused: bad top_n/num_init/num_local %d/%d/%d", top_n, num_init, num_local);
   NSA_REQUIRE(fixed_y_maxlen >= 1 && fixed_num_slc_blocks >= 1 && table_stride >= 1 && cmp_table_stride >= 1,

@@ -182,13 +182,35 @@ struct UnitFlash {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
   }
+  // Loads of the first unit of the next run(), issued early (before a serial section of the kernel that does not
+  // touch the staging slot) so that their latency is hidden behind it; the next run() must be called with the same
+  // arguments.
+  bf16x8 pre_k[KJ], pre_v[VJ];
+  int pre_key;
+  bool pre_valid = false;
+  template <class KeyFn>
+  NSA_DEVICE void prefetch(int first, int nu, int klo, int khi, KeyFn key0_of, const int* tab_s, int page,
+                           const bf16_t* kbase, int64_t k_sr, const bf16_t* vbase, int64_t v_sr) {
+    pre_valid = true;
+    if (first < nu) { pre_key = key0_of(first); issue(pre_key, klo, khi, tab_s, page, kbase, k_sr, vbase, v_sr, pre_k, pre_v); }
+  }
   // pipelined loop over units u = first, first+step, ... < nu ; key0_of(u) gives the unit's first key
   template <class KeyFn>
   NSA_DEVICE void run(int first, int step, int nu, int klo, int khi, KeyFn key0_of, const int* tab_s, int page,
                       const bf16_t* kbase, int64_t k_sr, const bf16_t* vbase, int64_t v_sr) {
     bf16x8 kfA[KJ], kfB[KJ], vrA[VJ], vrB[VJ];
     int keyA = 0, keyB = 0;
-    if (first < nu) { keyA = key0_of(first); issue(keyA, klo, khi, tab_s, page, kbase, k_sr, vbase, v_sr, kfA, vrA); }
+    if (pre_valid) {
+      pre_valid = false;
+      keyA = pre_key;
+#pragma unroll
+      for (int j = 0; j < KJ; j++) kfA[j] = pre_k[j];
+#pragma unroll
+      for (int j = 0; j < VJ; j++) vrA[j] = pre_v[j];
+    } else if (first < nu) {
+      keyA = key0_of(first);
+      issue(keyA, klo, khi, tab_s, page, kbase, k_sr, vbase, v_sr, kfA, vrA);
+    }
     for (int u = first; u < nu; u += 2 * step) {
       const bool hasB = u + step < nu;
       if (hasB) { keyB = key0_of(u + step); issue(keyB, klo, khi, tab_s, page, kbase, k_sr, vbase, v_sr, kfB, vrB); }
@@ -241,6 +263,21 @@ NSA_DEVICE float merge_value(const float* wgt, const float* po, int nparts, int 
   float o = 0.f;
   for (int w = 0; w < nparts; w++) o += wgt[w * part_stride_ml + head] * po[w * part_stride_o + head * VD + d];
   return o;
+}
+
+// four consecutive channels at once (16-byte LDS reads; same summation order over the parts as merge_value)
+NSA_DEVICE f32x4 merge_value4(const float* wgt, const float* po, int nparts, int part_stride_ml, int part_stride_o,
+                              int head, int d, int VD) {
+  f32x4 o = {0.f, 0.f, 0.f, 0.f};
+  for (int w = 0; w < nparts; w++) {
+    const float a = wgt[w * part_stride_ml + head];
+    const f32x4 x = *reinterpret_cast<const f32x4*>(&po[w * part_stride_o + head * VD + d]);
+    o[0] += a * x[0]; o[1] += a * x[1]; o[2] += a * x[2]; o[3] += a * x[3];
+  }
+  return o;
+}
+NSA_DEVICE f32x4 round_bf16x4(f32x4 x) {
+  return f32x4{(float)(bf16_t)x[0], (float)(bf16_t)x[1], (float)(bf16_t)x[2], (float)(bf16_t)x[3]};
 }
 
 // head-summed probabilities of the compressed keys -> scores of the selection blocks (ascending key order per
@@ -920,9 +957,9 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_fused_kernel(NsaDecodeP
   constexpr int NW = DEC_WAVES;
   constexpr int SLOT = UF::SLOT;
   constexpr int NTHREADS = NW * 64;
-  constexpr int OPT = 16 * VD / NTHREADS;  // merged output values per thread
+  constexpr int NV4 = 16 * VD / 4;                             // groups of four merged output values
+  constexpr int OPT4 = (NV4 + NTHREADS - 1) / NTHREADS;        // groups per thread
   static_assert(SLOT * 2 >= 16 * VD * 4, "a wave's slot must hold its partial output");
-  static_assert((16 * VD) % NTHREADS == 0, "output values must divide over the threads");
   extern __shared__ __attribute__((aligned(16))) unsigned char dyn_raw[];
   bf16_t* slots = reinterpret_cast<bf16_t*>(dyn_raw);
   float* part_m = reinterpret_cast<float*>(dyn_raw + (size_t)NW * SLOT * 2);
@@ -1028,6 +1065,15 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_fused_kernel(NsaDecodeP
   // ---- compressed attention, units dealt round-robin to the waves ----
   uf.run(wave, NW, nu, 0, y - 1, [&](int u) { return u * UK; }, ctab_s, page, kbase, p.k_sr, vbase, p.v_sr);
   uf.publish(part_m + wave * 16, part_l + wave * 16, reinterpret_cast<float*>(slots + wave * SLOT));
+  // the window branch does not depend on anything computed here: the waves that will run it fetch their first
+  // unit now, behind the merge of the compressed branch, the block scores and the selection
+  const int swa_klo = max(0, t - p.window);
+  const int swa_k0 = (swa_klo / UK) * UK;
+  const int swa_nu = t >= 0 ? (t - swa_k0) / UK + 1 : 0;
+  auto swa_key = [&](int u) { return swa_k0 + u * UK; };
+  constexpr bool PREFETCH_SWA = false;  // costs 38 spilled registers in the unit loop: slower (83 against 75 us)
+  if (PREFETCH_SWA && wave != 0 && t >= 0)
+    uf.prefetch(wave - 1, swa_nu, swa_klo, t, swa_key, tab_s, page, kbase, p.k_sr, vbase, p.v_sr);
   __syncthreads();
   if (tid < 16) {
     const float lse2 = merge_weights(part_m, part_l, NW, 16, tid, p.scale_log2);
@@ -1035,14 +1081,17 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_fused_kernel(NsaDecodeP
     if (tid < G && p.lse_out) p.lse_out[(int64_t)b * p.lse_st + (kh * G + tid) * p.lse_sh] = lse2;
   }
   __syncthreads();
-  float o_cmp[OPT];
+  // every thread merges four consecutive channels of one head (16-byte LDS reads, 8-byte stores)
+  f32x4 o_cmp[OPT4];
 #pragma unroll
-  for (int r = 0; r < OPT; r++) {
+  for (int r = 0; r < OPT4; r++) {
     const int idx = tid + r * NTHREADS;
-    const int h = idx / VD, d = idx - h * VD;
-    const float o = merge_value(part_l, reinterpret_cast<const float*>(slots), NW, 16, SLOT / 2, h, d, VD);
-    o_cmp[r] = (float)(bf16_t)o;  // the staged path stores the branch output as bf16 before the gated sum
-    if (h < G && p.cmp_o) p.cmp_o[(int64_t)b * p.co_st + (int64_t)(kh * G + h) * p.co_sh + d] = (bf16_t)o;
+    const int h = min(idx / (VD / 4), 15), d = (idx % (VD / 4)) * 4;
+    // the staged path stores the branch output as bf16 before the gated sum
+    o_cmp[r] = round_bf16x4(merge_value4(part_l, reinterpret_cast<const float*>(slots), NW, 16, SLOT / 2, h, d, VD));
+    if (idx < NV4 && h < G && p.cmp_o)
+      *reinterpret_cast<bf16x4*>(p.cmp_o + (int64_t)b * p.co_st + (int64_t)(kh * G + h) * p.co_sh + d) =
+          pack4(o_cmp[r][0], o_cmp[r][1], o_cmp[r][2], o_cmp[r][3]);
   }
   __syncthreads();
   // ---- probabilities p = kept exp2((s - m_unit)*c) * exp2(m_unit*c - lse), summed over the heads ----
@@ -1070,13 +1119,8 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_fused_kernel(NsaDecodeP
     blk_s[lane] = lane < nvalid ? max(result, 0) : 0;
     if (p.topk && lane < p.top_n) p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + lane] = result;
   } else {
-    if (t >= 0) {
-      const int klo = max(0, t - p.window);
-      const int k0 = (klo / UK) * UK;
-      const int nuw = (t - k0) / UK + 1;
-      uf.run(wave - 1, NW - 1, nuw, klo, t, [&](int u) { return k0 + u * UK; }, tab_s, page, kbase, p.k_sr, vbase,
-             p.v_sr);
-    }
+    if (t >= 0)
+      uf.run(wave - 1, NW - 1, swa_nu, swa_klo, t, swa_key, tab_s, page, kbase, p.k_sr, vbase, p.v_sr);
     uf.publish(swa_m + wave * 16, swa_l + wave * 16, swa_o + (wave - 1) * 16 * VD);
   }
   __syncthreads();
@@ -1095,22 +1139,24 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_fused_kernel(NsaDecodeP
   else if (tid < 32) merge_weights(swa_m + 16, swa_l + 16, NW - 1, 16, tid - 16, p.scale_log2);
   __syncthreads();
 #pragma unroll
-  for (int r = 0; r < OPT; r++) {
+  for (int r = 0; r < OPT4; r++) {
     const int idx = tid + r * NTHREADS;
-    const int h = idx / VD, d = idx - h * VD;
-    if (h >= G) continue;
+    const int h = idx / (VD / 4), d = (idx % (VD / 4)) * 4;
+    if (idx >= NV4 || h >= G) continue;
     const int hq = kh * G + h;
-    float o_slc = merge_value(part_l, reinterpret_cast<const float*>(slots), NW, 16, SLOT / 2, h, d, VD);
-    float o_swa = merge_value(swa_l + 16, swa_o, NW - 1, 16, 16 * VD, h, d, VD);
-    o_slc = (float)(bf16_t)o_slc;
-    o_swa = (float)(bf16_t)o_swa;
-    if (p.slc_o) p.slc_o[(int64_t)b * p.co_st + (int64_t)hq * p.co_sh + d] = (bf16_t)o_slc;
-    if (p.swa_o) p.swa_o[(int64_t)b * p.co_st + (int64_t)hq * p.co_sh + d] = (bf16_t)o_swa;
+    const f32x4 o_slc =
+        round_bf16x4(merge_value4(part_l, reinterpret_cast<const float*>(slots), NW, 16, SLOT / 2, h, d, VD));
+    const f32x4 o_swa = round_bf16x4(merge_value4(swa_l + 16, swa_o, NW - 1, 16, 16 * VD, h, d, VD));
+    const int64_t co = (int64_t)b * p.co_st + (int64_t)hq * p.co_sh + d;
+    if (p.slc_o) *reinterpret_cast<bf16x4*>(p.slc_o + co) = pack4(o_slc[0], o_slc[1], o_slc[2], o_slc[3]);
+    if (p.swa_o) *reinterpret_cast<bf16x4*>(p.swa_o + co) = pack4(o_swa[0], o_swa[1], o_swa[2], o_swa[3]);
     const bf16_t* wp = p.w + (int64_t)b * p.w_st + (int64_t)hq * p.w_sh;
-    float s0 = 1.f / (1.f + __expf(-(float)wp[0]));
-    float s1 = 1.f / (1.f + __expf(-(float)wp[1]));
-    float s2 = 1.f / (1.f + __expf(-(float)wp[2]));
-    p.out[(int64_t)b * p.o_st + (int64_t)hq * p.o_sh + d] = (bf16_t)(o_cmp[r] * s0 + o_slc * s1 + o_swa * s2);
+    const float s0 = 1.f / (1.f + __expf(-(float)wp[0]));
+    const float s1 = 1.f / (1.f + __expf(-(float)wp[1]));
+    const float s2 = 1.f / (1.f + __expf(-(float)wp[2]));
+    *reinterpret_cast<bf16x4*>(p.out + (int64_t)b * p.o_st + (int64_t)hq * p.o_sh + d) =
+        pack4(o_cmp[r][0] * s0 + o_slc[0] * s1 + o_swa[0] * s2, o_cmp[r][1] * s0 + o_slc[1] * s1 + o_swa[1] * s2,
+              o_cmp[r][2] * s0 + o_slc[2] * s1 + o_swa[2] * s2, o_cmp[r][3] * s0 + o_slc[3] * s1 + o_swa[3] * s2);
   }
 }
 
