@@ -101,7 +101,7 @@ def _time_replays(graphs, reps, warmup):
     return s.elapsed_time(e) * 1e3 / reps
 
 
-def decode_bench(dev, reps=200, warmup=20, cold_copies=6):
+def decode_bench(dev, reps=500, warmup=100, cold_copies=6):
     """Hot: one graph replayed over one batch (its 342 MB of K/V can stay partly in the 256 MB memory-side cache between
     replays).  Cold: `cold_copies` copies of the batch in disjoint memory, one graph each, replayed round-robin, so
     that (cold_copies - 1) x 342 MB of other K/V pass through the caches before a copy is read again: every replay
@@ -132,7 +132,8 @@ def decode_bench(dev, reps=200, warmup=20, cold_copies=6):
     nbytes = algorithmic_bytes(c["lens"])
     gbs = nbytes / (us * 1e-6) / 1e9
     res = {"workload": "paged NSA decode, batch 64, ctx uniform [4096,32768] (seed 3), page 256, 64q/4kv heads, "
-                       "d=128, bf16, hipGraph replay", "us_per_step": us, "eager_us_per_step": eager_us,
+                       "d=128, bf16, hipGraph replay; K/V pools from allocate_kv_pools (V pool staggered by 256 B)",
+           "us_per_step": us, "eager_us_per_step": eager_us,
            "graph_equals_eager": same, "algorithmic_bytes": nbytes,
            "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                         "frac": gbs / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_DEFAULT_CASE}}
@@ -145,7 +146,7 @@ def decode_bench(dev, reps=200, warmup=20, cold_copies=6):
         g, o = _capture(lambda a=a: nsa_decode(*a, **kw))
         graphs.append(g)
         outs.append(o)
-    cold_us = _time_replays(graphs, reps // len(graphs) * len(graphs), len(graphs) * 2)
+    cold_us = _time_replays(graphs, reps // len(graphs) * len(graphs), len(graphs) * 8)
     cold_gbs = nbytes / (cold_us * 1e-6) / 1e9
     res["us_per_step_cold"] = cold_us
     res["cold_copies"] = len(graphs)
@@ -153,6 +154,16 @@ def decode_bench(dev, reps=200, warmup=20, cold_copies=6):
     res["roofline_cold"] = {"bound": "hbm", "achieved": cold_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                             "frac": cold_gbs / PEAK_HBM_GBS, "traffic": None}
     del copies, graphs, outs
+    # the same batch in pools whose K and V bases coincide modulo 1 KB (one pool allocated right behind the other, as
+    # upstream's engine does): both streams of a workgroup then share a quarter of the memory channels
+    ca = build_decode_case(dev, staggered_pools=False)
+    pool_all_rows(ca, dev)
+    aa = args_of(ca)
+    nsa_decode(*aa, **kw)
+    ga, oa = _capture(lambda: nsa_decode(*aa, **kw))
+    res["us_per_step_unstaggered_pools"] = _time_replays([ga], reps, warmup)
+    res["unstaggered_equals_staggered"] = bool(torch.equal(oa, eager))
+    del ca, aa, ga, oa
     # the same step with the cache write of the newest token's K/V inside the launch (KV-cache writer fused)
     page = c["page"]
     KH, D = c["k"].size(2), c["k"].size(3)

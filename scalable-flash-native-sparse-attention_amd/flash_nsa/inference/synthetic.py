@@ -4,7 +4,10 @@ compressed row that the newest token completes."""
 import torch
 
 
-def build_decode_case(dev, B=64, QH=64, KH=4, D=128, page=256, lo=4096, hi=32768, seed=3):
+def build_decode_case(dev, B=64, QH=64, KH=4, D=128, page=256, lo=4096, hi=32768, seed=3, staggered_pools=True):
+    """staggered_pools: the pools come from allocate_kv_pools (V pool staggered against the K pool, what a serving
+    engine built on this package allocates); False: two separate tensors whose bases coincide modulo 1 KB, which is
+    what an allocation of one pool right after the other gives."""
     g = torch.Generator().manual_seed(seed)
     lens = torch.randint(lo, hi + 1, (B,), generator=g).tolist()
     ys = [max((L - 32) // 16 + 1, 0) for L in lens]
@@ -23,6 +26,12 @@ def build_decode_case(dev, B=64, QH=64, KH=4, D=128, page=256, lo=4096, hi=32768
     gd = torch.Generator(device=dev).manual_seed(seed)
     k = torch.randn(P, page, KH, D, device=dev, generator=gd, dtype=torch.float32).to(torch.bfloat16)
     v = torch.randn(P, page, KH, D, device=dev, generator=gd, dtype=torch.float32).to(torch.bfloat16)
+    if staggered_pools:
+        from .paging import allocate_kv_pools
+        (ks, vs), = allocate_kv_pools(P, page, KH, D, device=dev)
+        ks.copy_(k)
+        vs.copy_(v)
+        k, v = ks, vs
     q = torch.randn(B, QH, D, device=dev, generator=gd, dtype=torch.float32).to(torch.bfloat16)
     w = torch.randn(B, QH, 3, device=dev, generator=gd, dtype=torch.float32).to(torch.bfloat16)
     slots = []

@@ -89,11 +89,21 @@ def test_decode_padding_for_a_captured_graph_and_exhaustion():
         b.prefill([2], [200], device="cpu")
 
 
-def test_pools_are_the_two_halves_of_one_allocation():
-    (k, v), = allocate_kv_pools(5, 64, 2, 32, 16, device="cpu", dtype=torch.float32)
-    assert k.shape == (5, 64, 2, 32) and v.shape == (5, 64, 2, 16)
-    assert v.data_ptr() == k.data_ptr() + k.numel() * k.element_size()
-    assert k.is_contiguous() and v.is_contiguous()
+def test_pools_of_a_layer_share_one_allocation_with_the_v_pool_staggered():
+    """K pool then V pool of every layer inside one allocation, none overlapping; every K pool starts on a 1 KB
+    boundary and its V pool 256 bytes past one, so that the K rows and the V rows of one kv head fall on different
+    quarters of a 1 KB window (the decode kernels stream both at once)."""
+    pools = allocate_kv_pools(5, 64, 2, 32, 16, num_layers=3, device="cpu", dtype=torch.float32)
+    spans = []
+    for k, v in pools:
+        assert k.shape == (5, 64, 2, 32) and v.shape == (5, 64, 2, 16)
+        assert k.is_contiguous() and v.is_contiguous()
+        assert k.data_ptr() % 1024 == 0 and v.data_ptr() % 1024 == 256
+        assert 0 <= v.data_ptr() - (k.data_ptr() + k.numel() * k.element_size()) < 2048
+        spans += [(t.data_ptr(), t.data_ptr() + t.numel() * t.element_size()) for t in (k, v)]
+    spans.sort()
+    assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:])), "pools overlap"
+    assert k.untyped_storage().data_ptr() == pools[0][0].untyped_storage().data_ptr()
 
 
 def test_oracle_store_kvcache_is_an_indexed_row_copy():
