@@ -1,6 +1,6 @@
 """Benchmark of the NSA hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--seq-len T] [--no-cpu] [--no-decode]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--seq-len T] [--no-cpu] [--no-decode] [--single-stream]
     python bench.py --sweep 4096,8192,16384,32768,65536,131072,262144,524288,1048576
 
 A step is one forward+backward of the NSA core (NSACore: mean K-compression, sigmoid-mul V-compression,
@@ -24,8 +24,8 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 # what the same counter reads for a 1 GiB copy: x2.000 and x1.000), measured on the T=65536 workload of this file;
 # reported as roofline.traffic for that workload only.
 MEASURED_TRAFFIC_T64K = {
-    "cmp_dkdv": 34.93e9, "slc_dq": 77.02e9, "slc_fwd": 73.09e9, "slc_dkdv": 36.58e9, "cmp_dq": 7.05e9,
-    "topk": 1.26e9, "cmp_fwd": 2.25e9, "swa_dkdv": 11.38e9, "swa_dq": 5.03e9, "swa_fwd": 3.24e9,
+    "cmp_dkdv": 34.79e9, "slc_dq": 75.52e9, "slc_fwd": 73.08e9, "slc_dkdv": 36.58e9, "cmp_dq": 7.04e9,
+    "topk": 1.26e9, "cmp_fwd": 2.25e9, "swa_dkdv": 11.38e9, "swa_dq": 6.32e9, "swa_fwd": 3.24e9,
 }
 PEAK_HBM_GBS = 8000.0
 
@@ -314,6 +314,9 @@ def main():
     ap.add_argument("--seq-len", type=int, default=65536)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-decode", action="store_true")
+    ap.add_argument("--single-stream", action="store_true",
+                    help="keep the backward on one stream (for kernel traces: with the default two streams the dq and "
+                         "dk/dv kernels overlap and each one's traced duration is stretched by the other)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain 1 GiB device-to-device copy kernel, so that a counter run of this "
                          "command holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE with")
@@ -329,6 +332,9 @@ def main():
     from flash_nsa import NSAConfig, NSACore
     from flash_nsa import _lib
     _lib.LIB.load()  # fail loudly if the HIP library is missing
+    if args.single_stream:
+        from flash_nsa.modules import megatron_level_nsa
+        megatron_level_nsa.OVERLAP_STREAMS = False
     if args.sweep:
         length_sweep([int(x) for x in args.sweep.split(",")])
         return
