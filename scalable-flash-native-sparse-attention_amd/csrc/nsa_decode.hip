@@ -37,6 +37,10 @@ struct UnitFlash {
   static constexpr int KLD = D + NSA_LDS_PAD;
   static constexpr int VLD = VD + NSA_LDS_PAD;
   static constexpr int SLOT = UK * (KLD > VLD ? KLD : VLD);  // bf16 elements of a wave's staging slot
+  // row stride (floats) of a published partial output [16 heads][OLD]: with VD floats the 16 rows that one
+  // 16-byte store instruction writes would all start in the same LDS bank (a 16-way conflict); 4 more floats
+  // spread them over all 64 banks
+  static constexpr int OLD = VD + 4;
   bf16x8 qf[KC];
   f32x4 oacc[VD / 16];
   float m_run, l_run;
@@ -78,6 +82,25 @@ struct UnitFlash {
     const int ks = __builtin_amdgcn_readfirstlane(max(klo, min(key0, khi)));
     const int pi = ks / page;
     const int rem0 = ks - pi * page;
+    if constexpr (64 % (D / 8) == 0 && 64 % (VD / 8) == 0) {
+      // A unit that lies inside [klo, khi] and inside one page (nearly all of them) is UK consecutive pool rows:
+      // one wave-uniform row address per group of 64 lanes' rows, and a per-lane byte offset that never changes.
+      const int k0 = __builtin_amdgcn_readfirstlane(key0);
+      if (k0 >= klo && k0 + UK - 1 <= khi && rem0 + UK <= page) {
+        const int64_t row0 = (int64_t)__builtin_amdgcn_readfirstlane(tab_s[pi]) * page + rem0;
+        const char* kp = reinterpret_cast<const char*>(kbase + row0 * k_sr);
+        const char* vp = reinterpret_cast<const char*>(vbase + row0 * v_sr);
+        const uint32_t koff = (uint32_t)(lane / (D / 8)) * (uint32_t)k_sr * 2u + (uint32_t)(lane % (D / 8)) * 16u;
+        const uint32_t voff = (uint32_t)(lane / (VD / 8)) * (uint32_t)v_sr * 2u + (uint32_t)(lane % (VD / 8)) * 16u;
+#pragma unroll
+        for (int j = 0; j < KJ; j++)
+          kf[j] = *reinterpret_cast<const bf16x8*>(kp + (int64_t)(j * (64 / (D / 8))) * k_sr * 2 + koff);
+#pragma unroll
+        for (int j = 0; j < VJ; j++)
+          vr[j] = *reinterpret_cast<const bf16x8*>(vp + (int64_t)(j * (64 / (VD / 8))) * v_sr * 2 + voff);
+        return;
+      }
+    }
     const int64_t base0 = (int64_t)tab_s[pi] * page;
     const int64_t base1 = (rem0 + UK > page && (int64_t)(pi + 1) * page <= khi) ? (int64_t)tab_s[pi + 1] * page - page : base0;
 #pragma unroll
@@ -231,7 +254,7 @@ struct UnitFlash {
     if (kq == 0) { pm[l16] = m_run; pl[l16] = l_tot; }
 #pragma unroll
     for (int dt = 0; dt < VD / 16; dt++)
-      *reinterpret_cast<f32x4*>(&po[l16 * VD + dt * 16 + kq * 4]) = oacc[dt];
+      *reinterpret_cast<f32x4*>(&po[l16 * OLD + dt * 16 + kq * 4]) = oacc[dt];
   }
 };
 
@@ -259,19 +282,57 @@ NSA_DEVICE float merge_weights(const float* pm, float* pl, int nparts, int part_
   return l > 0.f ? m * sc + fast_log2(l) : 0.f;
 }
 NSA_DEVICE float merge_value(const float* wgt, const float* po, int nparts, int part_stride_ml, int part_stride_o,
-                             int head, int d, int VD) {
+                             int head, int d, int row_ld) {
   float o = 0.f;
-  for (int w = 0; w < nparts; w++) o += wgt[w * part_stride_ml + head] * po[w * part_stride_o + head * VD + d];
+  for (int w = 0; w < nparts; w++) o += wgt[w * part_stride_ml + head] * po[w * part_stride_o + head * row_ld + d];
   return o;
 }
 
 // four consecutive channels at once (16-byte LDS reads; same summation order over the parts as merge_value)
 NSA_DEVICE f32x4 merge_value4(const float* wgt, const float* po, int nparts, int part_stride_ml, int part_stride_o,
-                              int head, int d, int VD) {
+                              int head, int d, int row_ld) {
   f32x4 o = {0.f, 0.f, 0.f, 0.f};
   for (int w = 0; w < nparts; w++) {
     const float a = wgt[w * part_stride_ml + head];
-    const f32x4 x = *reinterpret_cast<const f32x4*>(&po[w * part_stride_o + head * VD + d]);
+    const f32x4 x = *reinterpret_cast<const f32x4*>(&po[w * part_stride_o + head * row_ld + d]);
+    o[0] += a * x[0]; o[1] += a * x[1]; o[2] += a * x[2]; o[3] += a * x[3];
+  }
+  return o;
+}
+// The same merge without the shared weights: every thread evaluates the weights of its own head in registers
+// (the same operations in the same order as merge_weights, so the results are bit-identical) -- 2 * NP broadcast
+// LDS reads and NP exponentials per thread buy one barrier and a serial 16-thread step less.
+template <int NP>
+NSA_DEVICE float merge_weights_local(const float* pm, const float* pl, int part_stride_ml, int head, float sc,
+                                     float (&wgt)[NP]) {
+  float mw[NP];
+  float m = NSA_NEG_INF;
+#pragma unroll
+  for (int w = 0; w < NP; w++) { mw[w] = pm[w * part_stride_ml + head]; m = fmaxf(m, mw[w]); }
+  if (m == NSA_NEG_INF) {
+#pragma unroll
+    for (int w = 0; w < NP; w++) wgt[w] = 0.f;
+    return 0.f;
+  }
+  float l = 0.f;
+#pragma unroll
+  for (int w = 0; w < NP; w++) {
+    const float a = (mw[w] == NSA_NEG_INF) ? 0.f : fast_exp2((mw[w] - m) * sc);
+    l += a * pl[w * part_stride_ml + head];
+    wgt[w] = a;
+  }
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+  for (int w = 0; w < NP; w++) wgt[w] *= inv;
+  return l > 0.f ? m * sc + fast_log2(l) : 0.f;
+}
+template <int NP>
+NSA_DEVICE f32x4 merge_value4_local(const float (&wgt)[NP], const float* po, int part_stride_o, int head, int d, int row_ld) {
+  f32x4 o = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int w = 0; w < NP; w++) {
+    const float a = wgt[w];
+    const f32x4 x = *reinterpret_cast<const f32x4*>(&po[w * part_stride_o + head * row_ld + d]);
     o[0] += a * x[0]; o[1] += a * x[1]; o[2] += a * x[2]; o[3] += a * x[3];
   }
   return o;
@@ -435,7 +496,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_cmp_topk_kernel(NsaDeco
   //              else: [pg]
   extern __shared__ __attribute__((aligned(16))) unsigned char dyn_raw[];
   constexpr int SLOT = UF::SLOT;
-  static_assert(SLOT * 2 >= 16 * VD * 4, "a wave's slot must hold its partial output");
+  static_assert(SLOT * 2 >= 16 * UF::OLD * 4, "a wave's slot must hold its partial output");
   bf16_t* Vs_all = reinterpret_cast<bf16_t*>(dyn_raw);
   float* part_m = reinterpret_cast<float*>(dyn_raw + (size_t)NW * SLOT * 2);
   float* part_l = part_m + NW * 16;
@@ -492,7 +553,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_cmp_topk_kernel(NsaDeco
   __syncthreads();
   for (int idx = tid; idx < G * VD; idx += NW * 64) {
     int h = idx / VD, d = idx - h * VD;
-    float o = merge_value(part_l, reinterpret_cast<const float*>(Vs_all), NW, 16, SLOT / 2, h, d, VD);
+    float o = merge_value(part_l, reinterpret_cast<const float*>(Vs_all), NW, 16, SLOT / 2, h, d, UF::OLD);
     p.cmp_o[(int64_t)b * p.co_st + (int64_t)(kh * G + h) * p.co_sh + d] = (bf16_t)o;
   }
   __syncthreads();
@@ -639,7 +700,7 @@ __global__ __launch_bounds__(SPLIT_WAVES * 64) void decode_cmp_partial_kernel(Ns
         float mw = part_m[w * 16 + h];
         float a = (mw == NSA_NEG_INF) ? 0.f : fast_exp2((mw - m) * p.scale_log2);
         l += a * part_l[w * 16 + h];
-        o += a * po[w * (SLOT / 2) + h * VD + d];
+        o += a * po[w * (SLOT / 2) + h * UF::OLD + d];
       }
     }
     p.sp_o[(base + h) * VD + d] = o;
@@ -761,7 +822,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecod
   constexpr int NT = NW * 64;
   extern __shared__ __attribute__((aligned(16))) unsigned char dyn_raw[];
   constexpr int SLOT = UF::SLOT;
-  static_assert(SLOT * 2 >= 16 * VD * 4, "a wave's slot must hold its partial output");
+  static_assert(SLOT * 2 >= 16 * UF::OLD * 4, "a wave's slot must hold its partial output");
   bf16_t* Vs_all = reinterpret_cast<bf16_t*>(dyn_raw);
   float* part_m = reinterpret_cast<float*>(dyn_raw + (size_t)NW * SLOT * 2);
   float* part_l = part_m + NW * 16;
@@ -900,7 +961,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecod
   for (int r = 0; r < OPT; r++) {
     const int idx = tid + r * NT;
     const int h = idx / VD, d = idx - h * VD;
-    o_swa_pre[r] = merge_value(part_l + w_first * 16, part_o + w_first * (SLOT / 2), NW - w_first, 16, SLOT / 2, h, d, VD);
+    o_swa_pre[r] = merge_value(part_l + w_first * 16, part_o + w_first * (SLOT / 2), NW - w_first, 16, SLOT / 2, h, d, UF::OLD);
   }
   __syncthreads();  // the slots are staging space again
 
@@ -922,7 +983,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecod
     const int h = idx / VD, d = idx - h * VD;
     if (h >= G) continue;
     const int hq = kh * G + h;
-    float o_slc = merge_value(part_l, part_o, NW, 16, SLOT / 2, h, d, VD);
+    float o_slc = merge_value(part_l, part_o, NW, 16, SLOT / 2, h, d, UF::OLD);
     // branch outputs are rounded to bf16 before the gated sum, as the three-kernel path stores them
     o_slc = (float)(bf16_t)o_slc;
     const float o_swa = (float)(bf16_t)o_swa_pre[r];
@@ -959,7 +1020,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_fused_kernel(NsaDecodeP
   constexpr int NTHREADS = NW * 64;
   constexpr int NV4 = 16 * VD / 4;                             // groups of four merged output values
   constexpr int OPT4 = (NV4 + NTHREADS - 1) / NTHREADS;        // groups per thread
-  static_assert(SLOT * 2 >= 16 * VD * 4, "a wave's slot must hold its partial output");
+  static_assert(SLOT * 2 >= 16 * UF::OLD * 4, "a wave's slot must hold its partial output");
   extern __shared__ __attribute__((aligned(16))) unsigned char dyn_raw[];
   bf16_t* slots = reinterpret_cast<bf16_t*>(dyn_raw);
   float* part_m = reinterpret_cast<float*>(dyn_raw + (size_t)NW * SLOT * 2);
@@ -1075,37 +1136,40 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_fused_kernel(NsaDecodeP
   if (PREFETCH_SWA && wave != 0 && t >= 0)
     uf.prefetch(wave - 1, swa_nu, swa_klo, t, swa_key, tab_s, page, kbase, p.k_sr, vbase, p.v_sr);
   __syncthreads();
-  if (tid < 16) {
-    const float lse2 = merge_weights(part_m, part_l, NW, 16, tid, p.scale_log2);
-    lse_s[tid] = tid < G ? lse2 : 0.f;
-    if (tid < G && p.lse_out) p.lse_out[(int64_t)b * p.lse_st + (kh * G + tid) * p.lse_sh] = lse2;
-  }
-  __syncthreads();
-  // every thread merges four consecutive channels of one head (16-byte LDS reads, 8-byte stores)
+  // every thread merges four consecutive channels of one head (16-byte LDS reads, 8-byte stores) with weights it
+  // evaluates itself; the thread that holds channel 0 of a head also publishes the head's lse
   f32x4 o_cmp[OPT4];
 #pragma unroll
   for (int r = 0; r < OPT4; r++) {
     const int idx = tid + r * NTHREADS;
     const int h = min(idx / (VD / 4), 15), d = (idx % (VD / 4)) * 4;
+    float wgt[NW];
+    const float lse2 = merge_weights_local<NW>(part_m, part_l, 16, h, p.scale_log2, wgt);
+    if (idx < NV4 && d == 0) {
+      lse_s[h] = h < G ? lse2 : 0.f;
+      if (h < G && p.lse_out) p.lse_out[(int64_t)b * p.lse_st + (kh * G + h) * p.lse_sh] = lse2;
+    }
     // the staged path stores the branch output as bf16 before the gated sum
-    o_cmp[r] = round_bf16x4(merge_value4(part_l, reinterpret_cast<const float*>(slots), NW, 16, SLOT / 2, h, d, VD));
+    o_cmp[r] = round_bf16x4(merge_value4_local<NW>(wgt, reinterpret_cast<const float*>(slots), SLOT / 2, h, d, UF::OLD));
     if (idx < NV4 && h < G && p.cmp_o)
       *reinterpret_cast<bf16x4*>(p.cmp_o + (int64_t)b * p.co_st + (int64_t)(kh * G + h) * p.co_sh + d) =
           pack4(o_cmp[r][0], o_cmp[r][1], o_cmp[r][2], o_cmp[r][3]);
   }
   __syncthreads();
-  // ---- probabilities p = kept exp2((s - m_unit)*c) * exp2(m_unit*c - lse), summed over the heads ----
-  for (int i = tid; i < nu * 16; i += NTHREADS) {
-    int h = i & 15;
-    keep_m[i] = h < G ? fast_exp2(__builtin_fmaf(keep_m[i], p.scale_log2, -lse_s[h])) : 0.f;
-  }
-  __syncthreads();
-  for (int key = tid; key < y; key += NTHREADS) {
-    const float* fac = keep_m + (key / UK) * 16;
-    float acc = 0.f;
+  // ---- probabilities p = kept exp2((s - m_unit)*c) * exp2(m_unit*c - lse), summed over the heads; a thread takes
+  // four consecutive keys (one unit, so one set of 16 per-head factors) ----
+  for (int key = tid * 4; key < y; key += NTHREADS * 4) {
+    const float* um = keep_m + (key / UK) * 16;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int h = 0; h < 16; h++) acc += (float)keep_p[h * keep_ld + key] * fac[h];
-    pg[key] = acc;
+    for (int h = 0; h < 16; h++) {
+      const float fac = h < G ? fast_exp2(__builtin_fmaf(um[h], p.scale_log2, -lse_s[h])) : 0.f;
+      typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+      const h4 kp = *reinterpret_cast<const h4*>(&keep_p[h * keep_ld + key]);
+      acc[0] += (float)kp[0] * fac; acc[1] += (float)kp[1] * fac;
+      acc[2] += (float)kp[2] * fac; acc[3] += (float)kp[3] * fac;
+    }
+    *reinterpret_cast<f32x4*>(&pg[key]) = acc;
   }
   __syncthreads();
   fold_block_scores(pg, imp, y, nb, p.nb_cap, p, tid, NTHREADS);
@@ -1121,7 +1185,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_fused_kernel(NsaDecodeP
   } else {
     if (t >= 0)
       uf.run(wave - 1, NW - 1, swa_nu, swa_klo, t, swa_key, tab_s, page, kbase, p.k_sr, vbase, p.v_sr);
-    uf.publish(swa_m + wave * 16, swa_l + wave * 16, swa_o + (wave - 1) * 16 * VD);
+    uf.publish(swa_m + wave * 16, swa_l + wave * 16, swa_o + (wave - 1) * 16 * UF::OLD);
   }
   __syncthreads();
 
@@ -1135,18 +1199,18 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_fused_kernel(NsaDecodeP
   }
   uf.publish(part_m + wave * 16, part_l + wave * 16, reinterpret_cast<float*>(slots + wave * SLOT));
   __syncthreads();
-  if (tid < 16) merge_weights(part_m, part_l, NW, 16, tid, p.scale_log2);
-  else if (tid < 32) merge_weights(swa_m + 16, swa_l + 16, NW - 1, 16, tid - 16, p.scale_log2);
-  __syncthreads();
 #pragma unroll
   for (int r = 0; r < OPT4; r++) {
     const int idx = tid + r * NTHREADS;
     const int h = idx / (VD / 4), d = (idx % (VD / 4)) * 4;
     if (idx >= NV4 || h >= G) continue;
     const int hq = kh * G + h;
+    float w_slc[NW], w_swa[NW - 1];
+    merge_weights_local<NW>(part_m, part_l, 16, h, p.scale_log2, w_slc);
+    merge_weights_local<NW - 1>(swa_m + 16, swa_l + 16, 16, h, p.scale_log2, w_swa);
     const f32x4 o_slc =
-        round_bf16x4(merge_value4(part_l, reinterpret_cast<const float*>(slots), NW, 16, SLOT / 2, h, d, VD));
-    const f32x4 o_swa = round_bf16x4(merge_value4(swa_l + 16, swa_o, NW - 1, 16, 16 * VD, h, d, VD));
+        round_bf16x4(merge_value4_local<NW>(w_slc, reinterpret_cast<const float*>(slots), SLOT / 2, h, d, UF::OLD));
+    const f32x4 o_swa = round_bf16x4(merge_value4_local<NW - 1>(w_swa, swa_o, 16 * UF::OLD, h, d, UF::OLD));
     const int64_t co = (int64_t)b * p.co_st + (int64_t)hq * p.co_sh + d;
     if (p.slc_o) *reinterpret_cast<bf16x4*>(p.slc_o + co) = pack4(o_slc[0], o_slc[1], o_slc[2], o_slc[3]);
     if (p.swa_o) *reinterpret_cast<bf16x4*>(p.swa_o + co) = pack4(o_swa[0], o_swa[1], o_swa[2], o_swa[3]);
@@ -1302,7 +1366,7 @@ static size_t fused_lds(const NsaDecodeParams& p) {
   const size_t ntab_c = (size_t)(p.y_cap + p.page_size - 1) / p.page_size;
   const size_t units = (size_t)(p.y_cap + UK - 1) / UK;
   size_t region = 16 * (units * UK + 8) * sizeof(_Float16);
-  const size_t swa_part = (size_t)(DEC_WAVES - 1) * 16 * VD * sizeof(float);
+  const size_t swa_part = (size_t)(DEC_WAVES - 1) * 16 * UnitFlash<D, VD>::OLD * sizeof(float);
   if (region < swa_part) region = swa_part;
   region = (region + 15) & ~(size_t)15;
   size_t n = slot_bytes<D, VD>() +
