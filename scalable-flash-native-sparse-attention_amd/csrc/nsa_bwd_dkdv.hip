@@ -207,8 +207,31 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
   // MODE_SLC: tokens of the NEXT tile to load, fetched from the inverse-index list one tile ahead of their use so
   // that the dependent (list -> row) lookups never stall the pipeline
   int tq[QJ], to[OJ], tsn = 0;
+  // When a thread's rows of one load step (NT / QP consecutive rows) never straddle a token, the token of load step
+  // j is the same for every thread of the workgroup: the list entries become scalar loads, the row addresses one
+  // scalar base per step plus a per-thread byte offset that never changes, and the (list position -> token -> 64-bit
+  // address) arithmetic leaves the vector unit.
+  const bool tok_uniform = MODE == MODE_SLC && fastG && (NT / QP) <= G && (NT / OP) <= G;
+  uint32_t qoff_b[QJ], ooff_b[OJ];
+#pragma unroll
+  for (int j = 0; j < QJ; j++) qoff_b[j] = (uint32_t)(qoffs[j] * 2);
+#pragma unroll
+  for (int j = 0; j < OJ; j++) ooff_b[j] = (uint32_t)(ooffs[j] * 2);
   auto fetch_tokens = [&](int rt0) {
     if (MODE != MODE_SLC) return;
+    if (tok_uniform) {
+      const int n0 = rt0 >> gshift;
+#pragma unroll
+      for (int j = 0; j < QJ; j++)
+        tq[j] = __builtin_amdgcn_readfirstlane(list[min(n0 + ((j * (NT / QP)) >> gshift), n_lastrow)]);
+      if (QP != OP) {
+#pragma unroll
+        for (int j = 0; j < OJ; j++)
+          to[j] = __builtin_amdgcn_readfirstlane(list[min(n0 + ((j * (NT / OP)) >> gshift), n_lastrow)]);
+      }
+      if (tid < RT) tsn = list[min(n0 + (tid >> gshift), n_lastrow)];
+      return;
+    }
 #pragma unroll
     for (int j = 0; j < QJ; j++) {
       int pc = tid + j * NT, n;
@@ -260,6 +283,23 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
         lse_reg = *lptr;
         delta_reg = *dptr;
         t_reg = sn;
+      }
+    } else if (tok_uniform) {
+#pragma unroll
+      for (int j = 0; j < QJ; j++)
+        qreg[j] = *reinterpret_cast<const bf16x8*>(
+            reinterpret_cast<const char*>(p.q + (int64_t)(x0 + tq[j]) * p.q_st) + qoff_b[j]);
+#pragma unroll
+      for (int j = 0; j < OJ; j++)
+        oreg[j] = *reinterpret_cast<const bf16x8*>(
+            reinterpret_cast<const char*>(p.dO + (int64_t)(x0 + ((QP == OP) ? tq[j] : to[j])) * p.do_st) + ooff_b[j]);
+      if (tid < RT) {
+        const bool ok = rt0 + tid <= row_last;
+        const int64_t tok = x0 + tsn;
+        const int64_t hoff = kh * G + (tid & (G - 1));
+        lse_reg = p.lse[tok * p.lse_st + hoff * p.lse_sh];
+        delta_reg = p.delta[tok * p.delta_st + hoff * p.delta_sh];
+        t_reg = ok ? tsn : T_INVALID;
       }
     } else {
 #pragma unroll
