@@ -210,21 +210,20 @@ struct UnitFlash {
   // arguments.
   bf16x8 pre_k[KJ], pre_v[VJ];
   int pre_key;
-  bool pre_valid = false;
   template <class KeyFn>
   NSA_DEVICE void prefetch(int first, int nu, int klo, int khi, KeyFn key0_of, const int* tab_s, int page,
                            const bf16_t* kbase, int64_t k_sr, const bf16_t* vbase, int64_t v_sr) {
-    pre_valid = true;
     if (first < nu) { pre_key = key0_of(first); issue(pre_key, klo, khi, tab_s, page, kbase, k_sr, vbase, v_sr, pre_k, pre_v); }
   }
   // pipelined loop over units u = first, first+step, ... < nu ; key0_of(u) gives the unit's first key
-  template <class KeyFn>
+  // USE_PRE: the first unit was fetched by prefetch() with the same arguments.  Only the call that consumes the
+  // prefetched registers is instantiated with it, so that they are dead everywhere else.
+  template <bool USE_PRE = false, class KeyFn>
   NSA_DEVICE void run(int first, int step, int nu, int klo, int khi, KeyFn key0_of, const int* tab_s, int page,
                       const bf16_t* kbase, int64_t k_sr, const bf16_t* vbase, int64_t v_sr) {
     bf16x8 kfA[KJ], kfB[KJ], vrA[VJ], vrB[VJ];
     int keyA = 0, keyB = 0;
-    if (pre_valid) {
-      pre_valid = false;
+    if (USE_PRE) {
       keyA = pre_key;
 #pragma unroll
       for (int j = 0; j < KJ; j++) kfA[j] = pre_k[j];
@@ -1132,7 +1131,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_fused_kernel(NsaDecodeP
   const int swa_k0 = (swa_klo / UK) * UK;
   const int swa_nu = t >= 0 ? (t - swa_k0) / UK + 1 : 0;
   auto swa_key = [&](int u) { return swa_k0 + u * UK; };
-  constexpr bool PREFETCH_SWA = false;  // costs 38 spilled registers in the unit loop: slower (83 against 75 us)
+  constexpr bool PREFETCH_SWA = true;
   if (PREFETCH_SWA && wave != 0 && t >= 0)
     uf.prefetch(wave - 1, swa_nu, swa_klo, t, swa_key, tab_s, page, kbase, p.k_sr, vbase, p.v_sr);
   __syncthreads();
@@ -1184,7 +1183,8 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_fused_kernel(NsaDecodeP
     if (p.topk && lane < p.top_n) p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + lane] = result;
   } else {
     if (t >= 0)
-      uf.run(wave - 1, NW - 1, swa_nu, swa_klo, t, swa_key, tab_s, page, kbase, p.k_sr, vbase, p.v_sr);
+      uf.template run<PREFETCH_SWA>(wave - 1, NW - 1, swa_nu, swa_klo, t, swa_key, tab_s, page, kbase, p.k_sr, vbase,
+                                    p.v_sr);
     uf.publish(swa_m + wave * 16, swa_l + wave * 16, swa_o + (wave - 1) * 16 * UF::OLD);
   }
   __syncthreads();

@@ -10,7 +10,7 @@ from gpu_util import make_cu, make_qkvw, randn_bf16, assert_close
 pytestmark = pytest.mark.gpu
 
 LENS_CASES = [[1000], [5, 31, 32, 47, 48, 100, 333, 700], [64, 0, 129, 513]]
-HEAD_CASES = [(16, 1, 128), (8, 2, 128), (4, 4, 64)]
+HEAD_CASES = [(16, 1, 128), (8, 2, 128), (4, 4, 64), (16, 2, 128), (32, 1, 128)]
 
 
 def setup_helper(cu_dev, **kw):
