@@ -11,7 +11,7 @@ import torch
 PEAK_HBM_GBS = 8000.0
 # bytes per step crossing the L2 <-> memory-side boundary (rocprofv3 --pmc FETCH_SIZE x2.000 + WRITE_SIZE x1.000, the
 # factors being what the counters read for a 1 GiB copy), measured for the default case of build_decode_case()
-MEASURED_TRAFFIC_DEFAULT_CASE = 334.1e6
+MEASURED_TRAFFIC_DEFAULT_CASE = 331.9e6
 
 
 # Decode attention of one layer with a 4 GiB KV pool, batch = 4 GiB / (S * 4 kv heads * 2 (K,V) * 2 bytes * 128), every
