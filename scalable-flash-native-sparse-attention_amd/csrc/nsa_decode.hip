@@ -86,7 +86,7 @@ struct UnitFlash {
       // A unit that lies inside [klo, khi] and inside one page (nearly all of them) is UK consecutive pool rows:
       // one wave-uniform row address per group of 64 lanes' rows, and a per-lane byte offset that never changes.
       const int k0 = __builtin_amdgcn_readfirstlane(key0);
-      if (k0 >= klo && k0 + UK - 1 <= khi && rem0 + UK <= page) {
+      if (k0 >= klo && k0 + UK - 1 <= khi && rem0 + UK <= page && k_sr < (1 << 28) && v_sr < (1 << 28)) {
         const int64_t row0 = (int64_t)__builtin_amdgcn_readfirstlane(tab_s[pi]) * page + rem0;
         const char* kp = reinterpret_cast<const char*>(kbase + row0 * k_sr);
         const char* vp = reinterpret_cast<const char*>(vbase + row0 * v_sr);
