@@ -633,3 +633,22 @@ def test_decode_small_batch_long_context_takes_the_split_path(device):
     assert int((err > 1e-2).sum()) <= 1, err
     o1 = nsa_decode(q, d["k"], d["v"], w, ctx_t, d["bt"], none, d["cbt"], cmp_num_splits=1, **kw)
     assert_close(o1, ref, "no parts", atol=8e-3, rtol=1e-2)
+
+
+def test_decode_more_workgroups_than_compute_units(device):
+    """320 requests x 2 kv heads = 640 workgroups of the one-launch kernel on 256 CUs (several rounds per CU), contexts
+    of 40-1000 tokens (at most 16 selection blocks, so every block is selected and no tie can change the result):
+    equal to the stage-by-stage decode, and identical when the same batch is run again."""
+    from flash_nsa import nsa_decode
+    from flash_nsa.inference import nsa_decode_staged
+    from flash_nsa.inference.synthetic import build_decode_case, pool_all_rows
+    c = build_decode_case(device, B=320, QH=32, KH=2, D=128, page=64, lo=40, hi=1000, seed=11)
+    pool_all_rows(c, device)
+    kw = dict(fixed_y_maxlen=128, fixed_num_slc_blocks=32)
+    args = (c["q"], c["k"], c["v"], c["w"], c["ctx"], c["bt"])
+    fused = nsa_decode(*args, c["slots"], c["cbt"], **kw)
+    staged = nsa_decode_staged(*args, c["cbt"], **kw)
+    assert torch.isfinite(fused).all()
+    assert_close(fused, staged, "one-launch vs staged decode, 640 workgroups", atol=8e-3, rtol=1e-2)
+    again = nsa_decode(*args, torch.full_like(c["slots"], -1), c["cbt"], **kw)
+    assert torch.equal(fused, again)
