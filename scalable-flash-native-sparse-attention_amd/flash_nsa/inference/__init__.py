@@ -49,20 +49,30 @@ def nsa_prefill(q, k, v, w, x_cu_seqlens, y_cu_seqlens, x_maxlen, y_maxlen, cont
     return combine_prefill(cmp_o, slc_o, swa_o, w)
 
 
-def auto_cmp_splits(batch, num_kv_heads, fixed_y_maxlen, num_cus=256):
-    """Parts the compressed branch of a decode step is cut into per (request, kv head).  One workgroup per pair
-    fills the GPU from about one pair per CU on; a small batch of contexts of 16K tokens or more (>= 1024 compressed
-    rows of capacity) is cut so that there are again about num_cus workgroups (measured on MI355X, 4 kv heads: 32
-    requests of 64K tokens 153 -> 117 us with 2 parts, 16 requests of 128K tokens 222 -> 118 us with 4, one request of
-    32K tokens 56 -> 46 us with 8; when the actual contexts are much shorter than the capacity the second launch costs
-    1-2 us)."""
+def auto_cmp_splits(batch, num_kv_heads, fixed_y_maxlen, num_cus=256, one_launch_fits=None):
+    """Parts the compressed branch of a decode step is cut into per (request, kv head); 1 = not cut.
+    one_launch_fits: whether the one-launch kernel holds this capacity (None: assumed up to 2048 compressed rows).
+    Measured on MI355X (4 kv heads, d = 128, graph replay, microseconds for 1 / 2 / 4 / 8 parts):
+      capacity 2048 rows (one launch possible): 1 x 32K 50 / 49 / 46 / 42, 4 x 32K 52 / 54 / 51 / 47, 4 x 4K
+      38 / 39 / 40 / 39, 8 x 32K 54 / 59 / 58 / 55, 16 x 32K 61 / 62 / 62 / 65 -- parts pay for up to 16 (request,
+      kv head) pairs and then only with 8 of them; short contexts in a large capacity lose 1-2 us to them;
+      capacity 8192 rows (two launches without parts): 8 x 64K 105 / 72 / 68 / 64, 16 x 64K 114 / 80 / 77 / 80,
+      16 x 128K 192 / 127 / 114 / 114, 32 x 64K 140 / 111 / 119 / 126, 32 x 128K 240 / 185 / 188 / 191."""
     pairs = batch * num_kv_heads
-    if fixed_y_maxlen < 1024 or pairs * 2 > num_cus:
+    if fixed_y_maxlen < 1024:
         return 1
-    n = 2
-    while n < 8 and pairs * n * 2 <= num_cus:
-        n *= 2
-    return n
+    if one_launch_fits is None:
+        one_launch_fits = fixed_y_maxlen <= 2048
+    scale = num_cus / 256.0
+    if one_launch_fits:
+        return 8 if pairs <= 16 * scale else 1
+    if pairs <= 32 * scale:
+        return 8
+    if pairs <= 64 * scale:
+        return 4
+    if pairs <= 128 * scale:
+        return 2
+    return 1
 
 
 def nsa_decode(q, k, v, w, context_lens, block_tables, cmp_slot_mapping, cmp_block_tables, cmp_num_splits=0,
@@ -81,7 +91,11 @@ def nsa_decode(q, k, v, w, context_lens, block_tables, cmp_slot_mapping, cmp_blo
     if cmp_num_splits == 0:
         # the split kernels exist for the shapes of the fused decode kernels (head dims 128/128 or 64/64, at most 16
         # q-heads per kv head)
-        cmp_num_splits = auto_cmp_splits(q.size(0), k.size(2), fixed_y_maxlen) if fused_decode_supported(q, k, v) else 1
+        if fused_decode_supported(q, k, v):
+            fits = decode_one_launch_fits(q, k, v, block_tables, fixed_y_maxlen, fixed_num_slc_blocks)
+            cmp_num_splits = auto_cmp_splits(q.size(0), k.size(2), fixed_y_maxlen, one_launch_fits=fits)
+        else:
+            cmp_num_splits = 1
     one_launch = (fused_decode_supported(q, k, v) and cmp_num_splits <= 1 and
                   decode_one_launch_fits(q, k, v, block_tables, fixed_y_maxlen, fixed_num_slc_blocks))
     if one_launch:

@@ -119,8 +119,8 @@ def test_oracle_store_kvcache_is_an_indexed_row_copy():
 
 def test_decode_picks_parts_only_for_small_batches_of_long_contexts():
     """auto_cmp_splits: one workgroup per (request, kv head) while those pairs fill the GPU or the capacity is below
-    16K tokens; otherwise a power of two of parts, at most 8, that brings the workgroup count back to about the CU
-    count."""
+    16K tokens; a capacity the one-launch kernel holds is cut (into 8) only for up to 16 pairs; larger capacities into
+    the power of two of parts, at most 8, that brings the workgroup count back to about the CU count."""
     from flash_nsa.inference import auto_cmp_splits
     assert auto_cmp_splits(64, 4, 4096) == 1          # 256 pairs: the GPU is full
     assert auto_cmp_splits(33, 4, 4096) == 1          # more than half full
@@ -129,6 +129,8 @@ def test_decode_picks_parts_only_for_small_batches_of_long_contexts():
     assert auto_cmp_splits(8, 4, 8192) == 8
     assert auto_cmp_splits(1, 1, 8192) == 8           # never more than 8
     assert auto_cmp_splits(1, 1, 2048) == 8           # 32K tokens of capacity: worth the second launch
+    assert auto_cmp_splits(4, 4, 2048) == 8 and auto_cmp_splits(5, 4, 2048) == 1   # ... for up to 16 pairs
+    assert auto_cmp_splits(8, 4, 2048) == 1 and auto_cmp_splits(8, 4, 2048, one_launch_fits=False) == 8
     assert auto_cmp_splits(1, 1, 1000) == 1           # below 16K tokens of capacity: one launch
     for b in range(1, 80):
         n = auto_cmp_splits(b, 4, 4096)
