@@ -1053,7 +1053,9 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_fused_kernel(NsaDecodeP
   {
     const int32_t* ctab = p.cmp_table + (int64_t)b * p.cmp_table_stride;
     const int32_t* tab = p.table + (int64_t)b * p.table_stride;
-    const int nc = (y + page - 1) / page, nr = min((L + page - 1) / page, p.table_stride);
+    // whole table rows (their widths are the capacity, the entries past a request's pages are never used), so that
+    // these loads do not wait for the context length and both round trips overlap
+    const int nc = min(ntab_c, p.cmp_table_stride), nr = p.table_stride;
     for (int i = tid; i < nc + nr; i += NTHREADS) {
       if (i < nc) ctab_s[i] = ctab[i];
       else tab_s[i - nc] = tab[i - nc];
