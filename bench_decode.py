@@ -6,7 +6,13 @@ block tables = slices of a random permutation of the pool, 64 q / 4 kv heads, d=
 compressed K for the importance pass is an implementation choice and is not counted), 16 selected blocks, the
 513 window rows, q + w + o.
 """
+import os
+import sys
+
 import torch
+
+# the synthetic batches are test / benchmark scaffolding and live beside the tests
+sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests"))
 
 PEAK_HBM_GBS = 8000.0
 # bytes per step crossing the L2 <-> memory-side boundary (rocprofv3 --pmc FETCH_SIZE x2.000 + WRITE_SIZE x1.000, the
@@ -27,7 +33,7 @@ def decode_sweep(dev, lengths=(4096, 8192, 16384, 32768, 65536, 131072), reps=10
     import json
     from flash_nsa import nsa_decode
     from flash_nsa.inference import auto_cmp_splits
-    from flash_nsa.inference.synthetic import build_decode_case, pool_all_rows
+    from synthetic_decode import build_decode_case, pool_all_rows
     for S in lengths:
         B = (4 << 30) // (S * 4 * 2 * 2 * 128)
         c = build_decode_case(dev, B=B, lo=S, hi=S, seed=5)
@@ -107,7 +113,7 @@ def decode_bench(dev, reps=500, warmup=100, cold_copies=6):
     that (cold_copies - 1) x 342 MB of other K/V pass through the caches before a copy is read again: every replay
     streams its K/V from HBM."""
     from flash_nsa import nsa_decode
-    from flash_nsa.inference.synthetic import build_decode_case, pool_all_rows
+    from synthetic_decode import build_decode_case, pool_all_rows
     c = build_decode_case(dev)
     pool_all_rows(c, dev)  # the compressed rows of the cached context, as earlier steps left them
     kw = dict(fixed_y_maxlen=2048, fixed_num_slc_blocks=512)

@@ -283,7 +283,7 @@ int nsa_decode_split(const void* q, int64_t q_st, int64_t q_sh, const void* k_ca
  * memory around the call (code under graph capture, tight serving loops, harnesses that forbid hipMalloc).  The
  * arguments are those of nsa_decode_split minus the five scratch buffers, which are carved out of one file-scope
  * device array of nsa_decode_split_static_capacity() bytes (32 MiB, held by every GPU the library runs on until the
- * process ends).  nsa_decode_split_static_bytes gives the bytes a call needs (e.g. 21.6 MB for 16 requests x 4 kv
+ * process ends).  nsa_decode_split_static_bytes gives the bytes a call needs (e.g. 22.1 MB for 16 requests x 4 kv
  * heads x 8 parts at fixed_y_maxlen 8192); a call that needs more is refused with NSA_ERR_UNSUPPORTED.  All calls on
  * one GPU share the array: calls that overlap there (other streams or threads) race.  Neither this entry point nor
  * anything below it calls hipMalloc / hipFree. */

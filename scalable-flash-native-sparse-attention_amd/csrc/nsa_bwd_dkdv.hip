@@ -214,7 +214,10 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
   // (the per-thread offsets are kept as 32-bit byte offsets: head strides beyond that take the general path)
   const bool off32 = ((int64_t)(kh * G + G) * p.q_sh + D) * 2 < ((int64_t)1 << 32) &&
                      ((int64_t)(kh * G + G) * p.do_sh + VD) * 2 < ((int64_t)1 << 32) && p.q_sh >= 0 && p.do_sh >= 0;
-  const bool tok_uniform = MODE == MODE_SLC && fastG && (NT / QP) <= G && (NT / OP) <= G && off32;
+  // (a head dim of 192 has 24 chunks per row, which do not divide the thread count: its load steps straddle tokens)
+  constexpr bool steps_whole_rows = (NT % QP == 0) && (NT % OP == 0);
+  const bool tok_uniform = MODE == MODE_SLC && steps_whole_rows && fastG && (NT / QP) <= G && G % (NT / QP) == 0 &&
+                           (NT / OP) <= G && G % (NT / OP) == 0 && off32;
   uint32_t qoff_b[QJ], ooff_b[OJ];
 #pragma unroll
   for (int j = 0; j < QJ; j++) qoff_b[j] = (uint32_t)(qoffs[j] * 2);

@@ -86,7 +86,8 @@ struct UnitFlash {
       // A unit that lies inside [klo, khi] and inside one page (nearly all of them) is UK consecutive pool rows:
       // one wave-uniform row address per group of 64 lanes' rows, and a per-lane byte offset that never changes.
       const int k0 = __builtin_amdgcn_readfirstlane(key0);
-      if (k0 >= klo && k0 + UK - 1 <= khi && rem0 + UK <= page && k_sr < (1 << 28) && v_sr < (1 << 28)) {
+      if (k0 >= klo && k0 + UK - 1 <= khi && rem0 + UK <= page && k_sr > 0 && v_sr > 0 && k_sr < (1 << 28) &&
+          v_sr < (1 << 28)) {
         const int64_t row0 = (int64_t)__builtin_amdgcn_readfirstlane(tab_s[pi]) * page + rem0;
         const char* kp = reinterpret_cast<const char*>(kbase + row0 * k_sr);
         const char* vp = reinterpret_cast<const char*>(vbase + row0 * v_sr);
@@ -1134,9 +1135,15 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_fused_kernel(NsaDecodeP
   const int swa_nu = t >= 0 ? (t - swa_k0) / UK + 1 : 0;
   auto swa_key = [&](int u) { return swa_k0 + u * UK; };
   constexpr bool PREFETCH_SWA = true;
-  if (PREFETCH_SWA && wave != 0 && t >= 0)
+  // When the newest token's row was stored by waves 0 / 1 after the first barrier (nothing pooled at this step),
+  // only the next barrier orders that store before other waves' reads of the row, and the window's last unit holds
+  // it: the prefetch then waits for the barrier (workgroup-uniform condition).
+  const bool stored_late = !pool_now && raw_slot >= 0;
+  if (PREFETCH_SWA && !stored_late && wave != 0 && t >= 0)
     uf.prefetch(wave - 1, swa_nu, swa_klo, t, swa_key, tab_s, page, kbase, p.k_sr, vbase, p.v_sr);
   __syncthreads();
+  if (PREFETCH_SWA && stored_late && wave != 0 && t >= 0)
+    uf.prefetch(wave - 1, swa_nu, swa_klo, t, swa_key, tab_s, page, kbase, p.k_sr, vbase, p.v_sr);
   // every thread merges four consecutive channels of one head (16-byte LDS reads, 8-byte stores) with weights it
   // evaluates itself; the thread that holds channel 0 of a head also publishes the head's lse
   f32x4 o_cmp[OPT4];

@@ -19,18 +19,36 @@ constexpr int MAX_DEVICES = 64;
 std::mutex g_lock;
 unsigned char* g_scratch_ptr[MAX_DEVICES] = {};  // device address of `scratch` on each GPU, resolved on first use
 
-// Device address of this GPU's copy of the array (the array's name is only a host-side handle).
-int scratch_base(unsigned char** base) {
+// Device address of the array's copy on the GPU that owns `dev_ptr` (the array's name is only a host-side handle, and
+// every GPU has its own copy at its own address).  The GPU is taken from the output pointer, not from the calling
+// thread's current device, so a caller whose current device differs from the one its tensors and stream live on
+// still gets the right copy; the first call for a GPU makes it current for the duration of the lookup.
+int scratch_base(const void* dev_ptr, unsigned char** base) {
   int dev = -1;
-  hipError_t e = hipGetDevice(&dev);
+  hipPointerAttribute_t attr;
+  hipError_t e = hipPointerGetAttributes(&attr, dev_ptr);
+  if (e == hipSuccess) {
+    dev = attr.device;
+  } else {
+    (void)hipGetLastError();
+    e = hipGetDevice(&dev);
+  }
   if (e != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
-    nsa_set_error("decode_split_static: hipGetDevice failed or device %d out of range: %s", dev, hipGetErrorString(e));
+    nsa_set_error("decode_split_static: cannot tell the GPU of the output buffer (device %d): %s", dev,
+                  hipGetErrorString(e));
     return NSA_ERR_LAUNCH;
   }
   std::lock_guard<std::mutex> guard(g_lock);
   if (g_scratch_ptr[dev] == nullptr) {
+    int cur = -1;
+    (void)hipGetDevice(&cur);
+    if (cur != dev && hipSetDevice(dev) != hipSuccess) {
+      nsa_set_error("decode_split_static: hipSetDevice(%d) failed", dev);
+      return NSA_ERR_LAUNCH;
+    }
     void* ptr = nullptr;
     e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (cur != dev && cur >= 0) (void)hipSetDevice(cur);
     if (e != hipSuccess || ptr == nullptr) {
       nsa_set_error("decode_split_static: hipGetSymbolAddress(scratch) failed on device %d: %s", dev,
                     hipGetErrorString(e));
@@ -105,7 +123,7 @@ int nsa_decode_split_static(const void* q, int64_t q_st, int64_t q_sh, const voi
               B, KH, nsplit, fixed_y_maxlen, s.total, STATIC_SCRATCH_BYTES);
   if (B == 0) return NSA_OK;
   unsigned char* base = nullptr;
-  int rc = scratch_base(&base);
+  int rc = scratch_base(out, &base);
   if (rc) return rc;
   return nsa_decode_split(q, q_st, q_sh, k_cache, k_sr, k_sh, v_cache, v_sr, v_sh, w, w_st, w_sh, out, o_st, o_sh,
                           cmp_o, slc_o, swa_o, co_st, co_sh, lse, lse_st, lse_sh, topk, tk_sh, tk_st,

@@ -20,3 +20,16 @@ def device():
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     return torch.device("cuda:0")
+
+
+@pytest.fixture(autouse=True)
+def _tuning_values_do_not_leak():
+    """nsa_set_tuning keeps process-wide overrides: whatever a test sets (or leaves set when it fails half way) is
+    dropped before the next test runs."""
+    yield
+    try:
+        from flash_nsa import _lib
+        if _lib.LIB._dll is not None:
+            _lib.call("nsa_reset_tuning")
+    except ImportError:
+        pass

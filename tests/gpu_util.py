@@ -44,3 +44,17 @@ def assert_close(dev, ref, name, atol=ATOL, rtol=RTOL, row_scale=False):
     assert not bad.any(), (f"{name}: {int(bad.sum())}/{bad.numel()} outside atol={atol} rtol={rtol}; "
                            f"max abs err {float(err.max()):.4g} at {np.unravel_index(int(err.argmax()), err.shape)}")
     return float(err.max())
+
+
+def bar_violations(dev, ref, atol=ATOL, rtol=RTOL, row_scale=False):
+    """(number of elements outside atol + rtol * base, number of elements, largest |dev - ref|), base as in
+    assert_close.  For assertions that state how many elements miss the plain bar instead of hiding them behind the
+    row-scaled one."""
+    dev = dev.detach().float().cpu()
+    ref = ref.detach().float().cpu()
+    assert dev.shape == ref.shape and torch.isfinite(dev).all()
+    err = (dev - ref).abs()
+    mag = ref.abs()
+    if row_scale and ref.numel():
+        mag = torch.maximum(mag, ref.pow(2).mean(-1, keepdim=True).sqrt())
+    return int((err > atol + rtol * mag).sum()), ref.numel(), float(err.max()) if ref.numel() else 0.0

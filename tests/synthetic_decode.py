@@ -1,4 +1,5 @@
-"""Synthetic paged-KV batches for benchmarks and full-size tests: a pool whose pages are handed out from a seeded
+"""Synthetic paged-KV batches for the decode benchmark and the full-size tests (test and benchmark scaffolding, not
+part of the flash_nsa package): a pool whose pages are handed out from a seeded
 random permutation (raw pages, then compressed-row pages, per request), random K/V/q/gates, and the slot of the
 compressed row that the newest token completes."""
 import torch
@@ -27,7 +28,7 @@ def build_decode_case(dev, B=64, QH=64, KH=4, D=128, page=256, lo=4096, hi=32768
     k = torch.randn(P, page, KH, D, device=dev, generator=gd, dtype=torch.float32).to(torch.bfloat16)
     v = torch.randn(P, page, KH, D, device=dev, generator=gd, dtype=torch.float32).to(torch.bfloat16)
     if staggered_pools:
-        from .paging import allocate_kv_pools
+        from flash_nsa.inference import allocate_kv_pools
         (ks, vs), = allocate_kv_pools(P, page, KH, D, device=dev)
         ks.copy_(k)
         vs.copy_(v)
@@ -48,7 +49,7 @@ def build_decode_case(dev, B=64, QH=64, KH=4, D=128, page=256, lo=4096, hi=32768
 
 def pool_all_rows(c, dev):
     """Pools every compressed row of the cached contexts of a build_case() dict (what earlier steps left behind)."""
-    from .stages import mean_pooling_prefill
+    from flash_nsa.inference import mean_pooling_prefill
     B, page = len(c["lens"]), c["page"]
     ycu = torch.zeros(B + 1, dtype=torch.int32)
     ycu[1:] = torch.cumsum(torch.tensor(c["ys"]), 0)

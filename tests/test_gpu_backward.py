@@ -274,18 +274,22 @@ def test_nsa_core_other_hyperparameters(device, hp):
     assert_close(wd.grad, ref["dw"], "dw")
 
 
-def test_nsa_core_qk192_v128(device):
-    """Dqk = 192, Dv = 128 (the head shape upstream's inference notebook exercises), forward + backward."""
+@pytest.mark.parametrize("QH,KH,block_size", [(8, 2, 64), (16, 2, 64), (32, 2, 64), (16, 2, 128), (16, 1, 96)])
+def test_nsa_core_qk192_v128(device, QH, KH, block_size):
+    """Dqk = 192, Dv = 128 (the head shape upstream's inference notebook exercises), forward + backward, with 4, 8
+    and 16 q-heads per kv head: a row of 192 channels is 24 sixteen-byte pieces, which do not divide the thread count
+    of the selected dK/dV kernel, so its load steps straddle tokens and take the general addressing path."""
     from flash_nsa import NSAConfig, NSACore
     from flash_nsa.ops.compress_kv import mean_pooling_fwd
     from flash_nsa.ops.compress_attn import cmp_attn_fwd
     from flash_nsa.ops.topk import slc_topk_indices
-    lens, QH, KH, D, VD = [700, 333], 8, 2, 192, 128
+    lens, D, VD = [700, 333], 192, 128
     cu = make_cu(lens)
     T = int(cu[-1])
     q, k, v, w = make_qkvw(T, QH, KH, D, VD, seed=80)
     do = randn_bf16(T, QH, VD, seed=85)
-    cfg = NSAConfig(qk_head_dim=D, v_head_dim=VD, num_heads=QH, num_kv_heads=KH, top_n=6, window_size=100)
+    cfg = NSAConfig(qk_head_dim=D, v_head_dim=VD, num_heads=QH, num_kv_heads=KH, top_n=6, window_size=100,
+                    block_size=block_size)
     mod = NSACore(cfg)
     qd, kd, vd, wd = [t.to(device).requires_grad_() for t in (q, k, v, w)]
     out = mod(qd, kd, vd, wd, cu.to(device))
@@ -295,7 +299,7 @@ def test_nsa_core_qk192_v128(device):
         _, lse = cmp_attn_fwd(qd.detach(), ck, cv)
         topk, _ = slc_topk_indices(qd.detach(), ck, lse)
     ref = O.nsa_forward_backward(q.float(), k.float(), v.float(), w.float(), do.float(), cu,
-                                 O.OracleConfig(top_n=6, window_size=100), topk=topk.cpu(),
+                                 O.OracleConfig(top_n=6, window_size=100, block_size=block_size), topk=topk.cpu(),
                                  round_dtype=torch.bfloat16, round_mma=True)
     assert_close(out, ref["o"], "o")
     assert_close(qd.grad, ref["dq"], "dq")

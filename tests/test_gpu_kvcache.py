@@ -106,3 +106,44 @@ def test_generation_loop_equals_training_forward(device, QH, KH, D, caps):
         # the pool holds the sequence's rows and compressed rows
         rows = torch.tensor([b.slot(ids[i], p) for p in range(L)], device=device)
         assert torch.equal(kc.view(-1, KH, D)[rows], k[i]) and torch.equal(vc.view(-1, KH, D)[rows], v[i])
+
+
+@pytest.mark.parametrize("window", [64, 128, 512])
+def test_fused_cache_write_is_ordered_before_the_window_reads(device, window):
+    """The one-launch decode kernel writes the newest token's K/V row itself when the caller passes it.  On steps that
+    pool nothing the row is stored after the kernel's first barrier, and with a short context or a narrow window the
+    wave that attends the window's last unit (which holds that row) is ready for it early: its fetch must come after
+    the store.  The pool rows of the newest tokens hold large finite garbage before the step, so a read that overtakes
+    the store changes the output; the reference is the separate writer followed by the same kernel without new rows."""
+    from flash_nsa.inference import decode_one_launch, store_kvcache, decode_one_launch_fits
+    from paged_util import build_pool, prepool, decode_slot_mapping
+    QH, KH, D, page = 64, 4, 128, 128
+    ctx = [1, 2, 17, 31, 33, 47, 63, 65, 97, 130, 200, 223, 225, 300, 513, 1000]   # none completes a compressed row
+    B = len(ctx)
+    case = build_pool(ctx, KH, D, D, page=page, seed=41)
+    prepool(case, ctx)
+    slots = decode_slot_mapping(case)
+    assert int((slots >= 0).sum()) == 0, "this test is about steps that pool nothing"
+    raw_slot = torch.tensor([int(case["bt"][b, (L - 1) // page]) * page + (L - 1) % page for b, L in enumerate(ctx)],
+                            dtype=torch.int32)
+    new_k, new_v = randn_bf16(B, KH, D, seed=42), randn_bf16(B, KH, D, seed=43)
+    q, w = randn_bf16(B, QH, D, seed=44).to(device), randn_bf16(B, QH, 3, seed=45).to(device)
+    ctx_t = torch.tensor(ctx, dtype=torch.int32, device=device)
+    # garbage where the newest rows go
+    for name in ("k", "v"):
+        case[name].view(-1, KH, D)[raw_slot.long()] = 3.0e4
+    kw = dict(fixed_y_maxlen=256, fixed_num_slc_blocks=32, window_size=window, return_parts=True)
+    d1 = {k: (v.to(device) if torch.is_tensor(v) else v) for k, v in case.items()}
+    d2 = {k: (v.to(device) if torch.is_tensor(v) else v) for k, v in case.items()}
+    assert decode_one_launch_fits(q, d1["k"], d1["v"], d1["bt"], 256, 32)
+    store_kvcache(new_k.to(device), new_v.to(device), d1["k"], d1["v"], raw_slot.to(device))
+    ref = decode_one_launch(q, d1["k"], d1["v"], w, d1["bt"], d1["cbt"], ctx_t, cmp_slot_mapping=slots.to(device), **kw)
+    for rep in range(3):
+        d2["k"].copy_(case["k"].to(device)); d2["v"].copy_(case["v"].to(device))
+        got = decode_one_launch(q, d2["k"], d2["v"], w, d2["bt"], d2["cbt"], ctx_t, cmp_slot_mapping=slots.to(device),
+                                new_k=new_k.to(device), new_v=new_v.to(device), slot_mapping=raw_slot.to(device), **kw)
+        torch.cuda.synchronize()
+        for name, a, r in zip(("out", "cmp_o", "slc_o", "swa_o", "topk", "lse"), got, ref):
+            assert torch.equal(a, r), f"{name}: fused cache write differs from store + decode (repeat {rep})"
+        assert torch.equal(d1["k"], d2["k"]) and torch.equal(d1["v"], d2["v"])
+    assert torch.isfinite(ref[0].float()).all()

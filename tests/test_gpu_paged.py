@@ -312,6 +312,60 @@ def test_decode_vs_oracle_and_training_forward(device, QH, KH, D):
         assert_close(o[b], full[-1], f"decode vs training row (request {b})", atol=1e-2, rtol=1e-2)
 
 
+@pytest.mark.parametrize("page,hp", [
+    (128, dict(block_size=64, top_n=16)),
+    (256, dict(block_size=64, top_n=16)),
+    (128, dict(block_size=32, top_n=12)),
+    (256, dict(block_size=96, top_n=5)),
+])
+def test_decode_selectors_return_the_oracle_selection(device, page, hp):
+    """Every decode selector (the staged topk_decode, the one-launch kernel, the split path) against the oracle's own
+    selection from the oracle's own scores on the same pool: index sets identical, differences excused only between
+    blocks whose scores lie within 1e-3 of each other (none of the outputs feeds the oracle here)."""
+    from flash_nsa.inference import (cmp_attn_decode, topk_decode, decode_one_launch, decode_split,
+                                     decode_one_launch_fits, decode_split_fits)
+    QH, KH, D = 64, 4, 128
+    ctx = [1, 31, 32, 64, 65, 4097, 333, 2999, 640, 1024, 127, 129, 4096, 1777]
+    case = build_pool(ctx, KH, D, D, page=page, seed=91)
+    prepool(case, ctx)                               # every compressed row pooled on the CPU: one pool for both sides
+    B = len(ctx)
+    d = to_dev(case, device)
+    q, w = randn_bf16(B, QH, D, seed=92), randn_bf16(B, QH, 3, seed=93)
+    ctx_t = torch.tensor(ctx, dtype=torch.int32)
+    Bs, top_n = hp["block_size"], hp["top_n"]
+    y_cap, nb_cap = 512, (4608 // Bs)
+    kw = dict(fixed_y_maxlen=y_cap, fixed_num_slc_blocks=nb_cap, block_size=Bs, top_n=top_n)
+    cfg = O.OracleConfig(block_size=Bs, top_n=top_n)
+    xcu = torch.arange(B + 1, dtype=torch.int32)
+    _, parts = O.nsa_paged_forward(q.float(), case["k"].float(), case["v"].float(), w.float(), xcu, ctx_t, case["bt"],
+                                   case["cbt"], cfg, return_parts=True)
+    own = torch.cat([p["topk"] for p in parts], 1)
+    imps = [p["imp"] for p in parts]
+    qd, wd, cd = q.to(device), w.to(device), ctx_t.to(device)
+    got = {}
+    _, lse = cmp_attn_decode(qd, d["k"], d["v"], d["cbt"], cd)
+    got["topk_decode"] = topk_decode(qd, d["k"], lse, d["cbt"], cd, **kw)
+    assert decode_one_launch_fits(qd, d["k"], d["v"], d["bt"], y_cap, nb_cap)
+    got["decode_one_launch"] = decode_one_launch(qd, d["k"], d["v"], wd, d["bt"], d["cbt"], cd, return_parts=True,
+                                                 **kw)[4]
+    assert decode_split_fits(qd, d["k"], d["v"], d["bt"], y_cap, nb_cap)
+    for nsplit in (2, 8):
+        got[f"decode_split[{nsplit}]"] = decode_split(qd, d["k"], d["v"], wd, d["bt"], d["cbt"], cd, nsplit=nsplit,
+                                                      return_parts=True, **kw)[4]
+    for name, tk in got.items():
+        tk = tk.cpu()
+        assert tk.shape == own.shape and tk.dtype == torch.int32, name
+        n_rows, n_diff, n_bad = O.topk_mismatch_report(tk, own, imps, xcu, Bs, top_n, tie_tol=1e-3,
+                                                       t_offsets=[L - 1 for L in ctx])
+        assert n_rows == B * KH and n_bad == 0 and n_diff <= 1, (name, n_rows, n_diff, n_bad)
+        # unused slots carry the inference ignore value, used ones are distinct
+        for b, L in enumerate(ctx):
+            nv = min(top_n, (L - 1) // Bs + 1)
+            for kh in range(KH):
+                row = tk[kh, b].tolist()
+                assert len(set(row[:nv])) == nv and all(x == -1 for x in row[nv:]), (name, b, kh, row)
+
+
 def test_decode_graph_replay_equals_eager(device):
     from flash_nsa import nsa_decode
     QH, KH, D = 64, 4, 128
@@ -641,7 +695,7 @@ def test_decode_more_workgroups_than_compute_units(device):
     equal to the stage-by-stage decode, and identical when the same batch is run again."""
     from flash_nsa import nsa_decode
     from flash_nsa.inference import nsa_decode_staged
-    from flash_nsa.inference.synthetic import build_decode_case, pool_all_rows
+    from synthetic_decode import build_decode_case, pool_all_rows
     c = build_decode_case(device, B=320, QH=32, KH=2, D=128, page=64, lo=40, hi=1000, seed=11)
     pool_all_rows(c, device)
     kw = dict(fixed_y_maxlen=128, fixed_num_slc_blocks=32)

@@ -452,3 +452,19 @@ def test_topk_mismatch_report_hand_cases():
     off_a, off_b = base[:, 130:].clone(), base[:, 130:].clone()
     off_b[0, 0] = torch.tensor([0, 2, 3], dtype=torch.int32)        # block 3 is beyond position 130
     assert O.topk_mismatch_report(off_a, off_b, [imp[:, 130:]], [0, T - 130], 64, N, t_offsets=[130])[1:] == (1, 1)
+
+
+def test_store_kvcache_hand_case():
+    """The cache writer of the oracle on a case small enough to write down: 2 pages of 2 rows, three tokens, the
+    middle one skipped (slot -1); rows land where a plain dictionary says and nothing else changes."""
+    kc = torch.full((2, 2, 1, 2), -7.0)
+    vc = torch.full((2, 2, 1, 3), -9.0)
+    key = torch.tensor([[[1.0, 2.0]], [[3.0, 4.0]], [[5.0, 6.0]]])
+    val = torch.tensor([[[10.0, 11.0, 12.0]], [[13.0, 14.0, 15.0]], [[16.0, 17.0, 18.0]]])
+    O.store_kvcache(key, val, kc, vc, torch.tensor([3, -1, 0], dtype=torch.int32))
+    want_k = {0: [5.0, 6.0], 1: [-7.0, -7.0], 2: [-7.0, -7.0], 3: [1.0, 2.0]}     # flat row -> contents
+    want_v = {0: [16.0, 17.0, 18.0], 1: [-9.0] * 3, 2: [-9.0] * 3, 3: [10.0, 11.0, 12.0]}
+    for row in range(4):
+        page, off = divmod(row, 2)
+        assert kc[page, off, 0].tolist() == want_k[row], row
+        assert vc[page, off, 0].tolist() == want_v[row], row

@@ -71,3 +71,36 @@ def test_static_scratch_decode_refuses_sizes_beyond_its_buffer(device):
     with pytest.raises(RuntimeError, match="static buffer holds"):
         decode_split(q, d["k"], d["v"], w, d["bt"], d["cbt"], ctx_t, nsplit=8, fixed_y_maxlen=8192,
                      fixed_num_slc_blocks=2048, static_scratch=True)
+
+
+def test_static_scratch_decode_under_graph_capture(device):
+    """What the entry point is for: the step recorded into a HIP graph (its outputs come from the graph's own pool, the
+    scratch from the static array) replays bit-equal to the eager call, several times, with the program's own eager
+    work and synchronisations between the replays and with new inputs through the same buffers."""
+    from flash_nsa.inference import decode_split
+    ctx = [8192, 4099, 333, 2064, 777, 6000]
+    case = build_pool(ctx, KH, D, D, page=128, seed=85)
+    prepool(case, ctx)
+    d = _to_dev(case, device)
+    B = len(ctx)
+    q, w = randn_bf16(B, QH, D, seed=86).to(device), randn_bf16(B, QH, 3, seed=87).to(device)
+    ctx_t = torch.tensor(ctx, dtype=torch.int32, device=device)
+    kw = dict(nsplit=4, fixed_y_maxlen=512, fixed_num_slc_blocks=128, static_scratch=True)
+    args = (q, d["k"], d["v"], w, d["bt"], d["cbt"], ctx_t)
+    eager = decode_split(*args, **kw).clone()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = decode_split(*args, **kw)
+    for it in range(3):
+        out.zero_()
+        junk = torch.randn(1 << 20, device=device).sum()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {it} differs from the eager call"
+    q.copy_(randn_bf16(B, QH, D, seed=88).to(device))
+    eager2 = decode_split(*args, **kw).clone()
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out, eager2) and not torch.equal(eager, eager2)
