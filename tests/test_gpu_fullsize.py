@@ -212,7 +212,10 @@ def test_c2_prefix_consistency_and_oracle_slice(device):
         cv = compress_kv_fwd(vs, core16.cmp_v_weight, "sigmoid-mul", NSAHelper)[2]
         _, lse = cmp_attn_fwd(qs, ck, cv)
         topk, _ = slc_topk_indices(qs, ck, lse)
-    assert torch.equal(o16, out[:n, :16]), "a kv group computed alone differs from the same group inside 4 groups"
+    # not bit-equal: the compression GEMM of 63 windows and the one of 4 x 4095 windows take different library
+    # kernels, whose V rows differ in the last bf16 bit
+    assert_close(o16, out[:n, :16], "a kv group computed alone against the same group inside 4 groups", atol=4e-3,
+                 rtol=8e-3)
     qr = qs.float().cpu().requires_grad_()
     ocfg = O.OracleConfig(cmp_v_method="sigmoid-mul")
     ref = O.nsa_forward(qr, ks.float().cpu(), vs.float().cpu(), ws.float().cpu(), [0, n], ocfg,
