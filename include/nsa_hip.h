@@ -78,6 +78,21 @@ int nsa_topk_select(const void* q, int64_t q_st, int64_t q_sh, const void* ck, i
                     const int32_t* y_cu, int B, int x_maxlen, int QH, int KH, int D, int kernel_size, int stride,
                     int block_size, int top_n, int num_init, int num_local, int ignore_index, float sm_scale,
                     void* stream);
+/* The same selection in two launches, the fp32 block scores between them in `workspace` (upstream keeps them in its
+ * slc_probs tensor between its two kernels, flash_nsa/ops/topk.py:226-425, 498-560): scoring then runs at twice the
+ * occupancy of the one-launch kernel, which keeps the scores of its tokens in LDS.  total_tokens = tokens of the packed
+ * batch (x_cu[B]).  nsa_topk_workspace_bytes(total_tokens, max_blocks, KH), max_blocks = selection blocks of the
+ * longest sequence, is what one pass over all tokens needs; a smaller workspace makes the call work in chunks of as
+ * many tokens as it holds (identical results).  workspace NULL, or a shape the two launches do not take (more than 16
+ * q-heads per kv head, more than 2048 selection blocks, block sizes that are not 1..64 strides in powers of two):
+ * the one-launch kernel runs, as in nsa_topk_select.  The workspace is scratch: nothing is kept between calls. */
+int64_t nsa_topk_workspace_bytes(int total_tokens, int max_blocks, int KH);
+int nsa_topk_select_ws(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr, int64_t ck_sh,
+                       const float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk, int64_t tk_sh, int64_t tk_st,
+                       float* imp_out, int64_t imp_sh, int64_t imp_st, int imp_cols, const int32_t* x_cu,
+                       const int32_t* y_cu, int B, int x_maxlen, int QH, int KH, int D, int kernel_size, int stride,
+                       int block_size, int top_n, int num_init, int num_local, int ignore_index, float sm_scale,
+                       int total_tokens, void* workspace, int64_t workspace_bytes, void* stream);
 /* flash_nsa/ops/select_attn.py:439-507 slc_attn_fwd */
 int nsa_slc_attn_fwd(const void* q, int64_t q_st, int64_t q_sh, const void* k, int64_t k_sr, int64_t k_sh,
                      const void* v, int64_t v_sr, int64_t v_sh, const int32_t* topk, int64_t tk_sh, int64_t tk_st,
@@ -189,6 +204,15 @@ int nsa_paged_topk_select(const void* q, int64_t q_st, int64_t q_sh, const void*
                           int fixed_num_slc_blocks, int QH, int KH, int D, int kernel_size, int stride,
                           int block_size, int top_n, int num_init, int num_local, int ignore_index, float sm_scale,
                           void* stream);
+/* nsa_paged_topk_select in two launches with a workspace, as nsa_topk_select_ws (max_blocks = fixed_num_slc_blocks) */
+int nsa_paged_topk_select_ws(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr,
+                             int64_t k_sh, const float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk,
+                             int64_t tk_sh, int64_t tk_st, const int32_t* x_cu, const int32_t* context_lens,
+                             const int32_t* cmp_block_tables, int table_stride, int page_size, int B, int x_maxlen,
+                             int fixed_num_slc_blocks, int QH, int KH, int D, int kernel_size, int stride,
+                             int block_size, int top_n, int num_init, int num_local, int ignore_index,
+                             float sm_scale, int total_tokens, void* workspace, int64_t workspace_bytes,
+                             void* stream);
 /* flash_nsa/inference/select_attn.py:103-166 slc_attn_prefill */
 int nsa_paged_slc_attn_fwd(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr,
                            int64_t k_sh, const void* v_cache, int64_t v_sr, int64_t v_sh, const int32_t* topk,

@@ -30,6 +30,7 @@ Knob g_knobs[] = {
     {"dq_min_blocks", {0}, {false}},    // workgroups per CU of the dense dq kernel
     {"dkdv_key_blocks", {0}, {false}},  // 32-key blocks per wave of the dense dk/dv kernel
     {"topk_seg_blocks", {0}, {false}},  // selection blocks per segment of the block selector
+    {"topk_two_pass", {0}, {false}},    // 0: the one-launch selector even when a workspace is given
 };
 Knob* find_knob(const char* name) {
   for (Knob& k : g_knobs)
@@ -79,7 +80,7 @@ int nsa_abi_version(void) { return 1; }
 int nsa_set_tuning(const char* name, int value) {
   Knob* k = name ? find_knob(name) : nullptr;
   NSA_REQUIRE(k != nullptr, NSA_ERR_BAD_ARG, "set_tuning: unknown name '%s' (fwd_variant, dq_min_blocks, "
-              "dkdv_key_blocks, topk_seg_blocks)", name ? name : "(null)");
+              "dkdv_key_blocks, topk_seg_blocks, topk_two_pass)", name ? name : "(null)");
   k->value.store(value);
   k->is_set.store(true);
   return NSA_OK;
@@ -130,12 +131,13 @@ int nsa_swa_fwd(const void* q, int64_t q_st, int64_t q_sh, const void* k, int64_
   return nsa_fwd_tile_launch(p, 1, false, B, x_maxlen, D, VD, (hipStream_t)stream);
 }
 
-int nsa_topk_select(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr, int64_t ck_sh,
-                    const float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk, int64_t tk_sh, int64_t tk_st,
-                    float* imp_out, int64_t imp_sh, int64_t imp_st, int imp_cols, const int32_t* x_cu,
-                    const int32_t* y_cu, int B, int x_maxlen, int QH, int KH, int D, int kernel_size, int stride,
-                    int block_size, int top_n, int num_init, int num_local, int ignore_index, float sm_scale,
-                    void* stream) {
+static int topk_select_impl(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr, int64_t ck_sh,
+                            const float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk, int64_t tk_sh,
+                            int64_t tk_st, float* imp_out, int64_t imp_sh, int64_t imp_st, int imp_cols,
+                            const int32_t* x_cu, const int32_t* y_cu, int B, int x_maxlen, int QH, int KH, int D,
+                            int kernel_size, int stride, int block_size, int top_n, int num_init, int num_local,
+                            int ignore_index, float sm_scale, int total_tokens, void* workspace,
+                            int64_t workspace_bytes, void* stream) {
   int rc = check_heads("topk_select", QH, KH, D, 32);
   if (rc) return rc;
   rc = check_nsa_sizes("topk_select", kernel_size, stride, block_size);
@@ -156,7 +158,40 @@ int nsa_topk_select(const void* q, int64_t q_st, int64_t q_sh, const void* ck, i
   p.top_n = top_n; p.num_init = num_init; p.num_local = num_local; p.ignore_index = ignore_index;
   p.nb_max = (x_maxlen + block_size - 1) / block_size;
   if (p.nb_max < 1) p.nb_max = 1;
+  if (workspace != nullptr && nsa_tuning_knob("topk_two_pass", 1) != 0 && nsa_topk_two_pass_supported(p, D))
+    return nsa_topk_two_pass_launch(p, false, B, x_maxlen, total_tokens, D, workspace, workspace_bytes,
+                                    (hipStream_t)stream);
   return nsa_topk_launch(p, false, B, x_maxlen, D, (hipStream_t)stream);
+}
+
+int nsa_topk_select(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr, int64_t ck_sh,
+                    const float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk, int64_t tk_sh, int64_t tk_st,
+                    float* imp_out, int64_t imp_sh, int64_t imp_st, int imp_cols, const int32_t* x_cu,
+                    const int32_t* y_cu, int B, int x_maxlen, int QH, int KH, int D, int kernel_size, int stride,
+                    int block_size, int top_n, int num_init, int num_local, int ignore_index, float sm_scale,
+                    void* stream) {
+  return topk_select_impl(q, q_st, q_sh, ck, ck_sr, ck_sh, lse, lse_st, lse_sh, topk, tk_sh, tk_st, imp_out, imp_sh,
+                          imp_st, imp_cols, x_cu, y_cu, B, x_maxlen, QH, KH, D, kernel_size, stride, block_size,
+                          top_n, num_init, num_local, ignore_index, sm_scale, 0, nullptr, 0, stream);
+}
+
+int64_t nsa_topk_workspace_bytes(int total_tokens, int max_blocks, int KH) {
+  if (total_tokens <= 0 || max_blocks <= 0 || KH <= 0) return 0;
+  return (int64_t)total_tokens * nsa_topk_two_pass_bytes_per_token(KH, max_blocks) + 512;
+}
+
+int nsa_topk_select_ws(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr, int64_t ck_sh,
+                       const float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk, int64_t tk_sh, int64_t tk_st,
+                       float* imp_out, int64_t imp_sh, int64_t imp_st, int imp_cols, const int32_t* x_cu,
+                       const int32_t* y_cu, int B, int x_maxlen, int QH, int KH, int D, int kernel_size, int stride,
+                       int block_size, int top_n, int num_init, int num_local, int ignore_index, float sm_scale,
+                       int total_tokens, void* workspace, int64_t workspace_bytes, void* stream) {
+  NSA_REQUIRE(total_tokens >= 0 && (workspace == nullptr || workspace_bytes > 0), NSA_ERR_BAD_ARG,
+              "topk_select_ws: bad token count %d or workspace size %lld", total_tokens, (long long)workspace_bytes);
+  return topk_select_impl(q, q_st, q_sh, ck, ck_sr, ck_sh, lse, lse_st, lse_sh, topk, tk_sh, tk_st, imp_out, imp_sh,
+                          imp_st, imp_cols, x_cu, y_cu, B, x_maxlen, QH, KH, D, kernel_size, stride, block_size,
+                          top_n, num_init, num_local, ignore_index, sm_scale, total_tokens, workspace,
+                          workspace_bytes, stream);
 }
 
 int nsa_slc_attn_fwd(const void* q, int64_t q_st, int64_t q_sh, const void* k, int64_t k_sr, int64_t k_sh,
@@ -466,13 +501,13 @@ int nsa_paged_swa_fwd(const void* q, int64_t q_st, int64_t q_sh, const void* k_c
   return nsa_fwd_tile_launch(p, 1, true, B, x_maxlen, D, VD, (hipStream_t)stream);
 }
 
-int nsa_paged_topk_select(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr,
+static int paged_topk_select_impl(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr,
                           int64_t k_sh, const float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk,
                           int64_t tk_sh, int64_t tk_st, const int32_t* x_cu, const int32_t* context_lens,
                           const int32_t* cmp_block_tables, int table_stride, int page_size, int B, int x_maxlen,
                           int fixed_num_slc_blocks, int QH, int KH, int D, int kernel_size, int stride,
                           int block_size, int top_n, int num_init, int num_local, int ignore_index, float sm_scale,
-                          void* stream) {
+                          int total_tokens, void* workspace, int64_t workspace_bytes, void* stream) {
   int rc = check_heads("paged_topk_select", QH, KH, D, 32);
   if (rc) return rc;
   rc = check_nsa_sizes("paged_topk_select", kernel_size, stride, block_size);
@@ -495,7 +530,40 @@ int nsa_paged_topk_select(const void* q, int64_t q_st, int64_t q_sh, const void*
   p.kernel_size = kernel_size; p.stride = stride; p.block_size = block_size;
   p.top_n = top_n; p.num_init = num_init; p.num_local = num_local; p.ignore_index = ignore_index;
   p.nb_max = fixed_num_slc_blocks;
+  if (workspace != nullptr && nsa_tuning_knob("topk_two_pass", 1) != 0 && nsa_topk_two_pass_supported(p, D))
+    return nsa_topk_two_pass_launch(p, true, B, x_maxlen, total_tokens, D, workspace, workspace_bytes,
+                                    (hipStream_t)stream);
   return nsa_topk_launch(p, true, B, x_maxlen, D, (hipStream_t)stream);
+}
+
+int nsa_paged_topk_select(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr,
+                          int64_t k_sh, const float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk,
+                          int64_t tk_sh, int64_t tk_st, const int32_t* x_cu, const int32_t* context_lens,
+                          const int32_t* cmp_block_tables, int table_stride, int page_size, int B, int x_maxlen,
+                          int fixed_num_slc_blocks, int QH, int KH, int D, int kernel_size, int stride,
+                          int block_size, int top_n, int num_init, int num_local, int ignore_index, float sm_scale,
+                          void* stream) {
+  return paged_topk_select_impl(q, q_st, q_sh, k_cache, k_sr, k_sh, lse, lse_st, lse_sh, topk, tk_sh, tk_st, x_cu,
+                                context_lens, cmp_block_tables, table_stride, page_size, B, x_maxlen,
+                                fixed_num_slc_blocks, QH, KH, D, kernel_size, stride, block_size, top_n, num_init,
+                                num_local, ignore_index, sm_scale, 0, nullptr, 0, stream);
+}
+
+int nsa_paged_topk_select_ws(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr,
+                             int64_t k_sh, const float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk,
+                             int64_t tk_sh, int64_t tk_st, const int32_t* x_cu, const int32_t* context_lens,
+                             const int32_t* cmp_block_tables, int table_stride, int page_size, int B, int x_maxlen,
+                             int fixed_num_slc_blocks, int QH, int KH, int D, int kernel_size, int stride,
+                             int block_size, int top_n, int num_init, int num_local, int ignore_index,
+                             float sm_scale, int total_tokens, void* workspace, int64_t workspace_bytes,
+                             void* stream) {
+  NSA_REQUIRE(total_tokens >= 0 && (workspace == nullptr || workspace_bytes > 0), NSA_ERR_BAD_ARG,
+              "paged_topk_select_ws: bad token count %d or workspace size %lld", total_tokens,
+              (long long)workspace_bytes);
+  return paged_topk_select_impl(q, q_st, q_sh, k_cache, k_sr, k_sh, lse, lse_st, lse_sh, topk, tk_sh, tk_st, x_cu,
+                                context_lens, cmp_block_tables, table_stride, page_size, B, x_maxlen,
+                                fixed_num_slc_blocks, QH, KH, D, kernel_size, stride, block_size, top_n, num_init,
+                                num_local, ignore_index, sm_scale, total_tokens, workspace, workspace_bytes, stream);
 }
 
 int nsa_paged_slc_attn_fwd(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr,

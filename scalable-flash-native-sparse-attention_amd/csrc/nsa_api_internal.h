@@ -55,6 +55,11 @@ int nsa_fwd_tile_launch(const NsaFwdTileParams& p, int mode, bool paged, int B, 
                         hipStream_t stream);
 int nsa_slc_fwd_launch(const NsaSlcParams& p, bool paged, int B, int max_q_len, int D, int VD, hipStream_t stream);
 int nsa_topk_launch(const NsaTopkParams& p, bool paged, int B, int max_q_len, int D, hipStream_t stream);
+// two launches with the block scores in a workspace (nsa_topk_two_pass.hip)
+bool nsa_topk_two_pass_supported(const NsaTopkParams& p, int D);
+int64_t nsa_topk_two_pass_bytes_per_token(int KH, int nb_max);
+int nsa_topk_two_pass_launch(const NsaTopkParams& p, bool paged, int B, int max_q_len, int total_tokens, int D,
+                             void* workspace, int64_t workspace_bytes, hipStream_t stream);
 
 // backward of the range-keyed branches and of the gathered (selected) branch
 struct NsaBwdTileParams {

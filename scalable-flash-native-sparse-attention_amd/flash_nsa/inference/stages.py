@@ -6,6 +6,7 @@ import torch
 from .. import _lib
 from ..ops._common import check_bf16
 from ..ops.combine import combine_fwd
+from ..ops.topk import topk_workspace
 
 _ARANGE = {}
 
@@ -137,11 +138,13 @@ def topk_prefill(q, k, lse, x_cu_seqlens, x_maxlen, y_maxlen, block_tables, cont
     sm_scale = q.size(-1) ** -0.5 if sm_scale is None else sm_scale
     assert lse.dtype == torch.float32 and lse.shape == (QH, t)
     topk = torch.empty(KH, t, top_n, device=q.device, dtype=torch.int32)
-    _lib.call("nsa_paged_topk_select", q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), ksr, ksh, lse.data_ptr(),
-              lse.stride(1), lse.stride(0), topk.data_ptr(), topk.stride(0), topk.stride(1),
+    ws = topk_workspace(t, int(fixed_num_slc_blocks), KH, q.device)
+    _lib.call("nsa_paged_topk_select_ws", q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), ksr, ksh,
+              lse.data_ptr(), lse.stride(1), lse.stride(0), topk.data_ptr(), topk.stride(0), topk.stride(1),
               _i32(x_cu_seqlens).data_ptr(), _i32(context_lens).data_ptr(), _i32(block_tables).data_ptr(),
               block_tables.stride(0), page, B, int(x_maxlen), int(fixed_num_slc_blocks), QH, KH, D, kernel_size,
-              stride, block_size, top_n, num_inital, num_local, -1, sm_scale, _lib.stream_ptr())
+              stride, block_size, top_n, num_inital, num_local, -1, sm_scale, t, _lib.ptr(ws),
+              ws.numel() if ws is not None else 0, _lib.stream_ptr())
     return topk
 
 

@@ -34,14 +34,30 @@ def slc_topk_indices(q, k, lse, sm_scale=None, return_slc_prob=False, align=True
         if align:
             cols = max(1 << (nblk - 1).bit_length(), 8)
         probs = torch.empty(KH, T, cols, device=q.device, dtype=torch.float32)
-    _lib.call("nsa_topk_select", q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), k.stride(0), k.stride(1),
+    ws = topk_workspace(T, nblk, KH, q.device)
+    _lib.call("nsa_topk_select_ws", q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), k.stride(0), k.stride(1),
               lse.data_ptr(), lse.stride(1), lse.stride(0), topk.data_ptr(), topk.stride(0), topk.stride(1),
               _lib.ptr(probs), probs.stride(0) if probs is not None else 0,
               probs.stride(1) if probs is not None else 0, cols, helper.x_cu_seqlens.data_ptr(),
               helper.y_cu_seqlens.data_ptr(), helper.batch, helper.x_maxlen, QH, KH, D, helper.kernel_size,
               helper.stride, helper.block_size, helper.top_n, helper.num_init_blocks, helper.num_local_blocks,
-              ignore_index, sm_scale, _lib.stream_ptr())
+              ignore_index, sm_scale, T, _lib.ptr(ws), ws.numel() if ws is not None else 0, _lib.stream_ptr())
     return topk, probs
+
+
+# most bytes of block scores held between the two launches of the selector; batches that need more run in chunks
+TOPK_WORKSPACE_LIMIT = 2 << 30
+# below this many tokens the one-launch selector (scores in LDS, no workspace) is at least as fast
+TOPK_TWO_PASS_MIN_TOKENS = 256
+
+
+def topk_workspace(total_tokens, max_blocks, KH, device):
+    """Scratch for the two-launch block selector (fp32 block scores of a chunk of tokens), from torch's caching
+    allocator; None for batches too small to gain from it."""
+    if total_tokens < TOPK_TWO_PASS_MIN_TOKENS:
+        return None
+    need = _lib.value("nsa_topk_workspace_bytes", int(total_tokens), int(max_blocks), int(KH))
+    return torch.empty(min(need, TOPK_WORKSPACE_LIMIT), dtype=torch.uint8, device=device)
 
 
 @torch.no_grad()
