@@ -78,3 +78,82 @@ NSA_DEVICE int select_blocks_regs(const float* imp, int t, int nb_cap, const P& 
   return result;
 }
 
+
+// wave-wide maximum of a float on the DPP crossbar, the same value in every lane
+NSA_DEVICE float wave_fmax_uniform(float x) {
+  float m = x;
+  m = dpp_fmax_step<0x111, 0xf>(m);  // row_shr:1
+  m = dpp_fmax_step<0x112, 0xf>(m);  // row_shr:2
+  m = dpp_fmax_step<0x114, 0xf>(m);  // row_shr:4
+  m = dpp_fmax_step<0x118, 0xf>(m);  // row_shr:8
+  m = dpp_fmax_step<0x142, 0xa>(m);  // row_bcast:15
+  m = dpp_fmax_step<0x143, 0xc>(m);  // row_bcast:31 -> lane 63 holds the wave maximum
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, m), 63));
+}
+
+// The same selection as select_blocks_regs, with the repeated arg-max run over a short list instead of the NV
+// registers of every lane: the R-th largest of the 64 lane maxima is a lower bound of the R-th largest score (R =
+// number of arg-max rounds), so only the scores at or above it can be selected; they are compacted (ballot + prefix
+// count) into a wave-private list of at most 64 entries in LDS (cand_v / cand_i), one per lane, and a round is one
+// wave reduction plus one compare.  The picks and their order are those of select_blocks_regs (descending score,
+// lowest index on ties); rows with more than 64 scores at the bound (many equal values) take that function.
+template <int NV, class P>
+NSA_DEVICE int select_blocks_short_list(const float* imp, int t, int nb_cap, const P& p, int lane, float* cand_v,
+                                        int* cand_i) {
+  const int nk = t >= 0 ? t / p.block_size : -1;
+  const int forced = p.num_init + p.num_local;
+  const int nsel = min(p.top_n, nk + 1);
+  const int rounds = nsel - forced;
+  int result = p.ignore_index;
+  if (lane < p.num_init) {
+    if (lane <= nk) result = lane;
+  } else if (lane < forced) {
+    if (lane <= nk) result = nk - (lane - p.num_init);
+  }
+  if (rounds <= 0) return result;
+  const int jmax = min(nk, nb_cap - 1);
+  float v[NV];
+  float m = -3.f;
+#pragma unroll
+  for (int k = 0; k < NV; k++) {
+    const int j = lane + 64 * k;
+    float x = j <= jmax ? imp[min(j, nb_cap - 1)] : -3.f;
+    if (j <= jmax && (j < p.num_init || j > nk - p.num_local)) x = -1.f;  // forced blocks: behind every real score
+    v[k] = x;
+    m = fmaxf(m, x);
+  }
+  // bound: the lane maxima in descending order until `rounds` lanes are counted
+  float theta = -1.f;
+  int counted = 0;
+  for (int r = 0; r < rounds; r++) {
+    const float mx = wave_fmax_uniform(m);
+    if (mx < -1.f) { theta = -1.f; break; }  // fewer lanes than rounds hold a candidate: everything is listed
+    theta = mx;
+    const bool hit = m == mx;
+    counted += __builtin_popcountll(__builtin_amdgcn_ballot_w64(hit));
+    if (hit) m = -4.f;
+    if (counted >= rounds) break;
+  }
+  // compaction of the scores >= theta, register by register (ascending block number within a register)
+  int base = 0;
+#pragma unroll
+  for (int k = 0; k < NV; k++) {
+    const bool q = v[k] >= theta;
+    const uint64_t mask = __builtin_amdgcn_ballot_w64(q);
+    const int pos = base + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+    if (q && pos < 64) { cand_v[pos] = v[k]; cand_i[pos] = lane + 64 * k; }
+    base += __builtin_popcountll(mask);
+  }
+  if (base > 64) return select_blocks_regs<NV>(imp, t, nb_cap, p, lane);  // wave-uniform
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  float cv = lane < base ? cand_v[lane] : -3.f;
+  int ci = lane < base ? cand_i[lane] : 0x7fffffff;
+  for (int slot = forced; slot < nsel; slot++) {
+    const int w = wave_argmax_lowest(cv, ci, ci != 0x7fffffff);
+    if (lane == slot) result = w;
+    if (ci == w) ci = 0x7fffffff;
+  }
+  return result;
+}

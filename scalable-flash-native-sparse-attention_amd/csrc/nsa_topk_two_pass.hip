@@ -51,15 +51,21 @@ struct ScoreWs {
   int tok_lo, tok_hi, row_stride;
 };
 
+#ifndef NSA_TOPK_SCORE_WAVES
+#define NSA_TOPK_SCORE_WAVES 4
+#endif
 template <int D, int GP, bool PAGED>
-__global__ __launch_bounds__(256, 4) void topk_score_kernel(NsaTopkParams p, ScoreWs ws) {
+__global__ __launch_bounds__(256, NSA_TOPK_SCORE_WAVES) void topk_score_kernel(NsaTopkParams p, ScoreWs ws) {
   constexpr int TPW = 32 / GP;      // tokens per wave
   constexpr int TWG = 4 * TPW;      // tokens per workgroup
   constexpr int KP = D / 8;         // 16-byte chunks per key row
   constexpr int KJ = (KT * KP) / 256;
   constexpr int PLD = HALO + KT + 8;  // a fold may look up to 7 entries past its last key
   using SM = SlotMap<GP>;
-  __shared__ __attribute__((aligned(16))) bf16_t Ks2[2][KT * D];
+  // two separate arrays, addressed with compile-time buffer numbers: the compiler then knows that the LDS reads of
+  // the tile being computed do not alias the direct-to-LDS loads of the next tile, and does not wait for those
+  __shared__ __attribute__((aligned(16))) bf16_t Ks_a[KT * D];
+  __shared__ __attribute__((aligned(16))) bf16_t Ks_b[KT * D];
   __shared__ float pg_all[4 * TPW * PLD];
 
   const int tid = threadIdx.x;
@@ -131,8 +137,9 @@ __global__ __launch_bounds__(256, 4) void topk_score_kernel(NsaTopkParams p, Sco
     int cs = St - Kz;
 #pragma unroll
     for (int r = 0; r < 8; r++, cs += St) {
-      f_w[r] = (float)(min(cs + Kz, Bs) - max(cs, 0)) / (float)St;
-      asm volatile("" : "+v"(f_w[r]));  // keep the quotient in a register: the division must not sink into the loop
+      const float w = r < nloops ? (float)(min(cs + Kz, Bs) - max(cs, 0)) / (float)St : 0.f;
+      // wave-uniform: kept in a scalar register, so that the division does not sink into the loop
+      f_w[r] = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, w)));
     }
   }
 
@@ -144,7 +151,8 @@ __global__ __launch_bounds__(256, 4) void topk_score_kernel(NsaTopkParams p, Sco
     const int pc = tid + j * 256, row = pc / KP;
     goffk[j] = (int)((row * p.ck_sr + ((pc % KP) ^ swz<KP>(row)) * 8) * 2);
   }
-  auto stage = [&](int kt, int buf) {
+  auto stage = [&](int kt, auto buf_tag) {
+    bf16_t* Kdst = decltype(buf_tag)::value == 0 ? Ks_a : Ks_b;
     int64_t row0;
     if (PAGED) row0 = (int64_t)table[kt / p.page_size] * p.page_size + (kt % p.page_size);
     else row0 = (int64_t)kbase + kt;
@@ -153,15 +161,14 @@ __global__ __launch_bounds__(256, 4) void topk_score_kernel(NsaTopkParams p, Sco
     if (last >= KT - 1) {
 #pragma unroll
       for (int j = 0; j < KJ; j++)
-        __builtin_amdgcn_global_load_lds((nsa_gptr_t)(kb + goffk[j]), (nsa_lptr_t)&Ks2[buf][(j * 256 + wave * 64) * 8],
-                                         16, 0, 0);
+        __builtin_amdgcn_global_load_lds((nsa_gptr_t)(kb + goffk[j]), (nsa_lptr_t)&Kdst[(j * 256 + wave * 64) * 8], 16, 0, 0);
     } else {
 #pragma unroll
       for (int j = 0; j < KJ; j++) {
         const int pc = tid + j * 256;
         const int row = pc / KP, c = (pc % KP) ^ swz<KP>(row);
         __builtin_amdgcn_global_load_lds((nsa_gptr_t)(kb + ((int64_t)min(row, last) * p.ck_sr + c * 8) * 2),
-                                         (nsa_lptr_t)&Ks2[buf][(j * 256 + wave * 64) * 8], 16, 0, 0);
+                                         (nsa_lptr_t)&Kdst[(j * 256 + wave * 64) * 8], 16, 0, 0);
       }
     }
   };
@@ -171,15 +178,15 @@ __global__ __launch_bounds__(256, 4) void topk_score_kernel(NsaTopkParams p, Sco
     return *reinterpret_cast<const bf16x8*>(Ks + (row * KP + ((2 * kc + hl) ^ swz<KP>(row))) * 8);
   };
 
-  if (n_score > 0) stage(0, 0);
-  int buf = 0;
-  for (int tile = 0; tile < ntiles; tile++, buf ^= 1) {
+  if (n_score > 0) stage(0, std::integral_constant<int, 0>{});
+  auto do_tile = [&](int tile, auto buf_tag) {
+    constexpr int BUF = decltype(buf_tag)::value;
     const int kt = tile * KT;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's pieces of the tile have landed
     __syncthreads();  // the tile is visible; nobody reads the other buffer any more
-    if (tile + 1 < n_score) stage(kt + KT, buf ^ 1);
-    if (!wave_active) continue;
-    const bf16_t* Ks = Ks2[buf];
+    if (tile + 1 < n_score) stage(kt + KT, std::integral_constant<int, 1 - BUF>{});
+    if (!wave_active) return;
+    const bf16_t* Ks = BUF == 0 ? Ks_a : Ks_b;
 #pragma unroll
     for (int u = 0; u < 2; u++) {
       const int key0 = kt + u * 32;
@@ -192,8 +199,11 @@ __global__ __launch_bounds__(256, 4) void topk_score_kernel(NsaTopkParams p, Sco
         f32x16 sacc;
 #pragma unroll
         for (int i = 0; i < 16; i++) sacc[i] = 0.f;
+        bf16x8 kf[D / 16];  // all fragments of the unit in flight before the first product
 #pragma unroll
-        for (int kc = 0; kc < D / 16; kc++) sacc = mfma32(qf[kc], kfrag(Ks, u, kc), sacc);
+        for (int kc = 0; kc < D / 16; kc++) kf[kc] = kfrag(Ks, u, kc);
+#pragma unroll
+        for (int kc = 0; kc < D / 16; kc++) sacc = mfma32(qf[kc], kf[kc], sacc);
         const bool all_vis = rows_full && key0 + 32 <= nkeys && tw_lo >= St * (key0 + 31) + Kz - 1;
         if (all_vis) {
 #pragma unroll
@@ -222,19 +232,24 @@ __global__ __launch_bounds__(256, 4) void topk_score_kernel(NsaTopkParams p, Sco
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    // ---- fold: the blocks this tile completes, (token, block) pairs dealt to the lanes ----
-    for (int it = lane; it < TPW * BPT; it += 64) {
+    // ---- fold: the blocks this tile completes, (token, block) pairs dealt to the lanes.  All 8 weights are applied
+    // (those past the block's last key are 0 and meet finite entries of the strip), so the loop has no branches ----
+    auto fold_one = [&](int it) {
       const int tk = it / BPT, jj = it - tk * BPT;
       const int n = nw0 + tk;
       const int j = tile * BPT + jj;
       const float* src = pgw + tk * PLD + HALO + jj * bps - kps + 1;
       float acc = 0.f;
 #pragma unroll
-      for (int r = 0; r < 8; r++)
-        if (r < nloops) acc += src[r] * f_w[r];
+      for (int r = 0; r < 8; r++) acc += src[r] * f_w[r];
       const int64_t tok = (int64_t)x0 + n;
       if (n < xl && tok >= ws.tok_lo && tok < ws.tok_hi && j < ws.row_stride)
         ws.imp[((int64_t)kh * (ws.tok_hi - ws.tok_lo) + (tok - ws.tok_lo)) * ws.row_stride + j] = acc;
+    };
+    if (TPW * BPT <= 64) {
+      if (lane < TPW * BPT) fold_one(lane);
+    } else {
+      for (int it = lane; it < TPW * BPT; it += 64) fold_one(it);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -244,6 +259,10 @@ __global__ __launch_bounds__(256, 4) void topk_score_kernel(NsaTopkParams p, Sco
       const int tk = i / HALO, h = i - tk * HALO;
       pgw[tk * PLD + h] = pgw[tk * PLD + KT + h];
     }
+  };
+  for (int tile = 0; tile < ntiles; tile += 2) {
+    do_tile(tile, std::integral_constant<int, 0>{});
+    if (tile + 1 < ntiles) do_tile(tile + 1, std::integral_constant<int, 1>{});
   }
   // positions of the workgroup's tokens, for the pick kernel (kv head 0 writes them)
   if (kh == 0 && tid < TWG) {
@@ -281,10 +300,12 @@ __global__ __launch_bounds__(256) void topk_pick_kernel(PickParams p) {
   }
   // candidates per lane sized by the row's own number of visible blocks (wave-uniform)
   const int cap = min(p.nb_max, p.row_stride);
+  __shared__ float cand_v[4][64];
+  __shared__ int cand_i[4][64];
   int result;
-  if (jmax < 512) result = select_blocks_regs<8>(imp, t, min(cap, 512), p, lane);
-  else if (jmax < 1024) result = select_blocks_regs<16>(imp, t, min(cap, 1024), p, lane);
-  else result = select_blocks_regs<32>(imp, t, min(cap, 2048), p, lane);
+  if (jmax < 512) result = select_blocks_short_list<8>(imp, t, min(cap, 512), p, lane, cand_v[wave], cand_i[wave]);
+  else if (jmax < 1024) result = select_blocks_short_list<16>(imp, t, min(cap, 1024), p, lane, cand_v[wave], cand_i[wave]);
+  else result = select_blocks_short_list<32>(imp, t, min(cap, 2048), p, lane, cand_v[wave], cand_i[wave]);
   if (lane < p.top_n) p.topk[(int64_t)kh * p.tk_sh + tok * p.tk_st + lane] = result;
 }
 
