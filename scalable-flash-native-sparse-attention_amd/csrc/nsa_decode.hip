@@ -23,6 +23,7 @@ constexpr int DEC_WAVES = 8;
 // adds it to the dynamic size when it decides whether a launch fits the 160 KB of a CU
 constexpr size_t SLC_SWA_STATIC_LDS = (3 * 16 + 64 * 16) * sizeof(float);
 constexpr int UK = 32;  // keys per unit
+constexpr int SEL_INTS = 192;  // LDS words of a selecting wave: 64 selected blocks + candidate list (64 scores, 64 indices)
 
 // One wave's flash-attention state over units of 32 keys for the 16 heads of a kv group.
 // K and V rows of a unit are fetched as whole rows (16 lanes x 16 bytes per row: every cache line is requested once
@@ -407,10 +408,12 @@ NSA_DEVICE int select_blocks_lds(float* imp, int t, int nb_cap, const NsaDecodeP
   return result;
 }
 
-NSA_DEVICE int select_blocks_wave(float* imp, int t, int nb_cap, const NsaDecodeParams& p, int lane) {
-  if (nb_cap <= 512) return select_blocks_regs<8>(imp, t, nb_cap, p, lane);
-  if (nb_cap <= 1024) return select_blocks_regs<16>(imp, t, nb_cap, p, lane);
-  if (nb_cap <= 2048) return select_blocks_regs<32>(imp, t, nb_cap, p, lane);
+// cand_v / cand_i: 64 floats + 64 ints of LDS private to the selecting wave
+NSA_DEVICE int select_blocks_wave(float* imp, int t, int nb_cap, const NsaDecodeParams& p, int lane, float* cand_v,
+                                  int* cand_i) {
+  if (nb_cap <= 512) return select_blocks_short_list<8>(imp, t, nb_cap, p, lane, cand_v, cand_i);
+  if (nb_cap <= 1024) return select_blocks_short_list<16>(imp, t, nb_cap, p, lane, cand_v, cand_i);
+  if (nb_cap <= 2048) return select_blocks_short_list<32>(imp, t, nb_cap, p, lane, cand_v, cand_i);
   return select_blocks_lds(imp, t, nb_cap, p, lane);
 }
 
@@ -536,7 +539,8 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_cmp_topk_kernel(NsaDeco
   fold_block_scores(pg, imp, y, nb, p.nb_cap, p, tid, NW * 64);
   __syncthreads();
   if (wave != 0) return;
-  const int result = select_blocks_wave(imp, t, p.nb_cap, p, lane);
+  // the waves' partial statistics are consumed: their space is the selector's candidate list
+  const int result = select_blocks_wave(imp, t, p.nb_cap, p, lane, part_m, reinterpret_cast<int*>(part_l));
   if (lane < p.top_n) p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + lane] = result;
 }
 
@@ -754,7 +758,9 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecod
   float* part_m = reinterpret_cast<float*>(dyn_raw + (size_t)NW * SLOT * 2);
   float* part_l = part_m + NW * 16;
   int* blk_s = reinterpret_cast<int*>(part_l + NW * 16);
-  int* tab_s = blk_s + 64;  // the request's raw page table
+  float* cand_v = reinterpret_cast<float*>(blk_s + 64);  // the selector's candidate list (64 scores + 64 indices)
+  int* cand_i = blk_s + 128;
+  int* tab_s = blk_s + SEL_INTS;  // the request's raw page table
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -866,7 +872,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecod
   uf.init(p.q + (int64_t)b * p.q_st + (int64_t)head * p.q_sh, p.scale_log2, lane, Vs_all + wave * SLOT);
   const int w_first = select_here ? 1 : 0;
   if (wave < w_first) {
-    const int result = select_blocks_wave(imp, t, nb, p, lane);
+    const int result = select_blocks_wave(imp, t, nb, p, lane, cand_v, cand_i);
     blk_s[lane] = lane < nvalid ? max(result, 0) : 0;
     if (p.topk && lane < p.top_n) p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + lane] = result;
   } else {
@@ -957,7 +963,9 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_fused_kernel(NsaDecodeP
   float* lse_s = swa_l + NW * 16;
   float* imp = lse_s + 16;
   int* blk_s = reinterpret_cast<int*>(imp + ((p.nb_cap + 3) & ~3));
-  int* ctab_s = blk_s + 64;
+  float* cand_v = reinterpret_cast<float*>(blk_s + 64);  // the selector's candidate list (64 scores + 64 indices)
+  int* cand_i = blk_s + 128;
+  int* ctab_s = blk_s + SEL_INTS;
   const int ntab_c = (p.y_cap + p.page_size - 1) / p.page_size;
   int* tab_s = ctab_s + ((ntab_c + 3) & ~3);
   const int n_units_cap = (p.y_cap + UK - 1) / UK;
@@ -1114,7 +1122,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_fused_kernel(NsaDecodeP
   const int nvalid = t >= 0 ? min(p.top_n, t / Bs + 1) : 0;
   uf.reset();
   if (wave == 0) {
-    const int result = select_blocks_wave(imp, t, p.nb_cap, p, lane);
+    const int result = select_blocks_wave(imp, t, p.nb_cap, p, lane, cand_v, cand_i);
     blk_s[lane] = lane < nvalid ? max(result, 0) : 0;
     if (p.topk && lane < p.top_n) p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + lane] = result;
   } else {
@@ -1214,7 +1222,7 @@ int nsa_decode_cmp_topk_launch(const NsaDecodeParams& p, int B, int D, int VD, h
 int nsa_decode_slc_swa_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream) {
   if (B <= 0) return NSA_OK;
   dim3 grid(B, p.KH);
-  size_t extra = (size_t)(2 * DEC_WAVES * 16 + 64 + ((p.table_stride + 3) & ~3)) * sizeof(float);
+  size_t extra = (size_t)(2 * DEC_WAVES * 16 + SEL_INTS + ((p.table_stride + 3) & ~3)) * sizeof(float);
   if (p.pg != nullptr) extra += (size_t)((p.nb_cap + 3) & ~3) * sizeof(float);  // block scores
   if (D == 128 && VD == 128)
     return launch_dyn(decode_slc_swa_kernel<128, 128>, grid, slot_bytes<128, 128>() + extra, p, stream,
@@ -1257,7 +1265,7 @@ static size_t split_final_lds(const NsaDecodeParams& p) {
   const size_t slots = slot_bytes<D, VD>();
   if ((size_t)((p.y_cap + UK - 1) / UK) * UK * 4 > slots) return 0;  // head-summed probabilities overlay the slots
   const size_t nuc = (size_t)(p.y_cap + UK - 1) / UK;
-  const size_t total = slots + (size_t)(2 * DEC_WAVES * 16 + 64 + ((p.table_stride + 3) & ~3)) * 4 +
+  const size_t total = slots + (size_t)(2 * DEC_WAVES * 16 + SEL_INTS + ((p.table_stride + 3) & ~3)) * 4 +
                        (size_t)(((p.nb_cap + 3) & ~3) + (nuc * 16 > 2 * 64 * 16 ? nuc * 16 : 2 * 64 * 16)) * 4;  // factors, or the parts' (m, l)
   return total + SLC_SWA_STATIC_LDS <= 160 * 1024 ? total : 0;
 }
@@ -1306,7 +1314,7 @@ static size_t fused_lds(const NsaDecodeParams& p) {
   if (region < swa_part) region = swa_part;
   region = (region + 15) & ~(size_t)15;
   size_t n = slot_bytes<D, VD>() +
-             (size_t)(4 * DEC_WAVES * 16 + 16 + (((size_t)p.nb_cap + 3) & ~(size_t)3) + 64 + ((ntab_c + 3) & ~(size_t)3) +
+             (size_t)(4 * DEC_WAVES * 16 + 16 + (((size_t)p.nb_cap + 3) & ~(size_t)3) + SEL_INTS + ((ntab_c + 3) & ~(size_t)3) +
                       (((size_t)p.table_stride + 3) & ~(size_t)3) + units * 16) * sizeof(float) + region;
   if ((size_t)p.y_cap * sizeof(float) > slot_bytes<D, VD>()) return 0;
   return n <= 160 * 1024 ? n : 0;
