@@ -132,6 +132,22 @@ int nsa_cmp_attn_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void*
                           float* dcv, int64_t dcv_sr, int64_t dcv_sh, const int32_t* x_cu, const int32_t* y_cu,
                           int B, int x_maxlen, int y_maxlen, int QH, int KH, int D, int VD, int kernel_size,
                           int stride, int q_chunk_tokens, float sm_scale, void* stream);
+/* The same with a summation order that does not depend on the run (upstream's dkdv_repeat=True: per-head buffers and a
+ * final sum, flash_nsa/ops/compress_attn.py:594-598,691-693; here the q-heads of a group are summed inside the matrix
+ * accumulators and what remains to be ordered are the query chunks): every work item stores its fp32 partial result
+ * in its own slot of `workspace` (nsa_cmp_attn_bwd_dkdv_det_bytes(...) bytes, same sizes and q_chunk_tokens as the
+ * call), a second launch sums the slots of a key in ascending chunk order and stores dck / dcv (no zero-fill needed
+ * for the keys it writes; keys no query sees keep what the buffers held). */
+int64_t nsa_cmp_attn_bwd_dkdv_det_bytes(int B, int x_maxlen, int y_maxlen, int QH, int KH, int D, int VD,
+                                        int kernel_size, int stride, int q_chunk_tokens);
+int nsa_cmp_attn_bwd_dkdv_det(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr,
+                              int64_t ck_sh, const void* cv, int64_t cv_sr, int64_t cv_sh, const void* dO,
+                              int64_t do_st, int64_t do_sh, const float* lse, int64_t lse_st, int64_t lse_sh,
+                              const float* delta, int64_t delta_st, int64_t delta_sh, float* dck, int64_t dck_sr,
+                              int64_t dck_sh, float* dcv, int64_t dcv_sr, int64_t dcv_sh, const int32_t* x_cu,
+                              const int32_t* y_cu, int B, int x_maxlen, int y_maxlen, int QH, int KH, int D, int VD,
+                              int kernel_size, int stride, int q_chunk_tokens, float sm_scale, void* workspace,
+                              int64_t workspace_bytes, void* stream);
 /* flash_nsa/ops/sliding_window_attention.py:98-157 swa_bwd (FlashAttention varlen backward) */
 int nsa_swa_bwd_dq(const void* q, int64_t q_st, int64_t q_sh, const void* k, int64_t k_sr, int64_t k_sh,
                    const void* v, int64_t v_sr, int64_t v_sh, const void* dO, int64_t do_st, int64_t do_sh,
@@ -176,6 +192,20 @@ int nsa_slc_attn_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void*
                           const int32_t* blk_seq, const int32_t* csr_off, const int32_t* csr_tok,
                           const int32_t* item_off, int nblk_total, int chunk_tokens, int n_items_bound, int B,
                           int QH, int KH, int D, int VD, int block_size, float sm_scale, void* stream);
+/* The same with a run-independent summation order (upstream's dkdv_repeat=True, flash_nsa/ops/select_attn.py:528-531,
+ * 639-641): every work item (a chunk of a block's token list) stores its partial result in its own slot of
+ * `workspace` (nsa_slc_attn_bwd_dkdv_det_bytes(...) bytes), a second launch adds the slots of a block to dk / dv in
+ * ascending chunk order, one thread per element. */
+int64_t nsa_slc_attn_bwd_dkdv_det_bytes(int n_items_bound, int KH, int D, int VD, int block_size);
+int nsa_slc_attn_bwd_dkdv_det(const void* q, int64_t q_st, int64_t q_sh, const void* k, int64_t k_sr, int64_t k_sh,
+                              const void* v, int64_t v_sr, int64_t v_sh, const void* dO, int64_t do_st,
+                              int64_t do_sh, const float* lse, int64_t lse_st, int64_t lse_sh, const float* delta,
+                              int64_t delta_st, int64_t delta_sh, float* dk, int64_t dk_sr, int64_t dk_sh,
+                              float* dv, int64_t dv_sr, int64_t dv_sh, const int32_t* x_cu, const int32_t* kblk_cu,
+                              const int32_t* blk_seq, const int32_t* csr_off, const int32_t* csr_tok,
+                              const int32_t* item_off, int nblk_total, int chunk_tokens, int n_items_bound, int B,
+                              int QH, int KH, int D, int VD, int block_size, float sm_scale, void* workspace,
+                              int64_t workspace_bytes, void* stream);
 
 /* ---- paged KV (inference).  Caches are [num_pages, page_size, KH, D]; *_sr is the stride of a flat row
  * (page*page_size + offset), *_sh the head stride.  Request b's raw token n lives at flat row

@@ -289,17 +289,9 @@ int nsa_cmp_attn_bwd_dq_final(const void* q, int64_t q_st, int64_t q_sh, const v
                          x_maxlen, QH, KH, D, VD, kernel_size, stride, sm_scale, stream);
 }
 
-int nsa_cmp_attn_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr, int64_t ck_sh,
-                          const void* cv, int64_t cv_sr, int64_t cv_sh, const void* dO, int64_t do_st,
-                          int64_t do_sh, const float* lse, int64_t lse_st, int64_t lse_sh, const float* delta,
-                          int64_t delta_st, int64_t delta_sh, float* dck, int64_t dck_sr, int64_t dck_sh,
-                          float* dcv, int64_t dcv_sr, int64_t dcv_sh, const int32_t* x_cu, const int32_t* y_cu,
-                          int B, int x_maxlen, int y_maxlen, int QH, int KH, int D, int VD, int kernel_size,
-                          int stride, int q_chunk_tokens, float sm_scale, void* stream) {
-  int rc = check_heads("cmp_attn_bwd_dkdv", QH, KH, D, VD);
-  if (rc) return rc;
-  rc = check_nsa_sizes("cmp_attn_bwd_dkdv", kernel_size, stride, 0);
-  if (rc) return rc;
+// Query tokens per work item of the compressed dk/dv kernel when the caller leaves the choice to the library.
+static int cmp_dkdv_q_chunk(int q_chunk_tokens, int B, int x_maxlen, int y_maxlen, int QH, int KH, int D, int VD,
+                            int kernel_size, int stride) {
   if (q_chunk_tokens <= 0) {
     // The kernel keeps one workgroup per CU, so a launch takes about
     //   ceil(workgroups / CUs) * (fixed cost of a workgroup + its 64-row tiles * time per tile);
@@ -330,6 +322,22 @@ int nsa_cmp_attn_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void*
       if (q_chunk_tokens <= 0 || cost < best) { best = cost; q_chunk_tokens = chunk; }
     }
   }
+  return q_chunk_tokens;
+}
+
+static int cmp_attn_bwd_dkdv_impl(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr,
+                                  int64_t ck_sh, const void* cv, int64_t cv_sr, int64_t cv_sh, const void* dO,
+                                  int64_t do_st, int64_t do_sh, const float* lse, int64_t lse_st, int64_t lse_sh,
+                                  const float* delta, int64_t delta_st, int64_t delta_sh, float* dck, int64_t dck_sr,
+                                  int64_t dck_sh, float* dcv, int64_t dcv_sr, int64_t dcv_sh, const int32_t* x_cu,
+                                  const int32_t* y_cu, int B, int x_maxlen, int y_maxlen, int QH, int KH, int D,
+                                  int VD, int kernel_size, int stride, int q_chunk_tokens, float sm_scale,
+                                  bool deterministic, void* workspace, int64_t workspace_bytes, void* stream) {
+  int rc = check_heads("cmp_attn_bwd_dkdv", QH, KH, D, VD);
+  if (rc) return rc;
+  rc = check_nsa_sizes("cmp_attn_bwd_dkdv", kernel_size, stride, 0);
+  if (rc) return rc;
+  q_chunk_tokens = cmp_dkdv_q_chunk(q_chunk_tokens, B, x_maxlen, y_maxlen, QH, KH, D, VD, kernel_size, stride);
   BwdCommon c{q, q_st, q_sh, ck, ck_sr, ck_sh, cv, cv_sr, cv_sh, dO, do_st, do_sh, lse, lse_st, lse_sh, delta,
               delta_st, delta_sh};
   NsaBwdTileParams p = make_bwd(c, QH, KH, sm_scale);
@@ -339,8 +347,61 @@ int nsa_cmp_attn_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void*
   p.x_cu = x_cu; p.k_cu = y_cu;
   p.kernel_size = kernel_size; p.stride = stride;
   p.q_chunk_tokens = q_chunk_tokens;
-  return nsa_bwd_dkdv_launch(p, 0, B, x_maxlen, y_maxlen, D, VD, 0, (hipStream_t)stream);
+  if (!deterministic) return nsa_bwd_dkdv_launch(p, 0, B, x_maxlen, y_maxlen, D, VD, 0, (hipStream_t)stream);
+  if (B <= 0 || y_maxlen <= 0) return NSA_OK;
+  // every work item stores into its own slot, then one pass sums the slots of a key in ascending chunk order
+  const int64_t slots = nsa_bwd_dkdv_cmp_slots(B, KH, x_maxlen, y_maxlen, q_chunk_tokens, kernel_size, stride);
+  const int64_t kw = nsa_bwd_dkdv_slot_keys(0, 0);
+  const int64_t dk_bytes = (slots * kw * D * 4 + 255) & ~(int64_t)255;
+  const int64_t need = dk_bytes + slots * kw * VD * 4;
+  NSA_REQUIRE(workspace != nullptr && workspace_bytes >= need, NSA_ERR_WORKSPACE,
+              "cmp_attn_bwd_dkdv_det: workspace of %lld bytes, %lld needed", (long long)workspace_bytes,
+              (long long)need);
+  p.dkv_mode = 4;
+  p.part_dk = (float*)workspace;
+  p.part_dv = (float*)((char*)workspace + dk_bytes);
+  rc = nsa_bwd_dkdv_launch(p, 0, B, x_maxlen, y_maxlen, D, VD, 0, (hipStream_t)stream);
+  if (rc) return rc;
+  return nsa_dkdv_reduce_cmp_launch(p, B, x_maxlen, y_maxlen, D, VD, (hipStream_t)stream);
 }
+
+int nsa_cmp_attn_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr, int64_t ck_sh,
+                          const void* cv, int64_t cv_sr, int64_t cv_sh, const void* dO, int64_t do_st,
+                          int64_t do_sh, const float* lse, int64_t lse_st, int64_t lse_sh, const float* delta,
+                          int64_t delta_st, int64_t delta_sh, float* dck, int64_t dck_sr, int64_t dck_sh,
+                          float* dcv, int64_t dcv_sr, int64_t dcv_sh, const int32_t* x_cu, const int32_t* y_cu,
+                          int B, int x_maxlen, int y_maxlen, int QH, int KH, int D, int VD, int kernel_size,
+                          int stride, int q_chunk_tokens, float sm_scale, void* stream) {
+  return cmp_attn_bwd_dkdv_impl(q, q_st, q_sh, ck, ck_sr, ck_sh, cv, cv_sr, cv_sh, dO, do_st, do_sh, lse, lse_st,
+                                lse_sh, delta, delta_st, delta_sh, dck, dck_sr, dck_sh, dcv, dcv_sr, dcv_sh, x_cu,
+                                y_cu, B, x_maxlen, y_maxlen, QH, KH, D, VD, kernel_size, stride, q_chunk_tokens,
+                                sm_scale, false, nullptr, 0, stream);
+}
+
+int64_t nsa_cmp_attn_bwd_dkdv_det_bytes(int B, int x_maxlen, int y_maxlen, int QH, int KH, int D, int VD,
+                                        int kernel_size, int stride, int q_chunk_tokens) {
+  if (B <= 0 || x_maxlen <= 0 || y_maxlen <= 0 || KH <= 0 || QH <= 0 || stride <= 0) return 0;
+  q_chunk_tokens = cmp_dkdv_q_chunk(q_chunk_tokens, B, x_maxlen, y_maxlen, QH, KH, D, VD, kernel_size, stride);
+  const int64_t slots = nsa_bwd_dkdv_cmp_slots(B, KH, x_maxlen, y_maxlen, q_chunk_tokens, kernel_size, stride);
+  const int64_t kw = nsa_bwd_dkdv_slot_keys(0, 0);
+  return ((slots * kw * D * 4 + 255) & ~(int64_t)255) + slots * kw * VD * 4;
+}
+
+int nsa_cmp_attn_bwd_dkdv_det(const void* q, int64_t q_st, int64_t q_sh, const void* ck, int64_t ck_sr,
+                              int64_t ck_sh, const void* cv, int64_t cv_sr, int64_t cv_sh, const void* dO,
+                              int64_t do_st, int64_t do_sh, const float* lse, int64_t lse_st, int64_t lse_sh,
+                              const float* delta, int64_t delta_st, int64_t delta_sh, float* dck, int64_t dck_sr,
+                              int64_t dck_sh, float* dcv, int64_t dcv_sr, int64_t dcv_sh, const int32_t* x_cu,
+                              const int32_t* y_cu, int B, int x_maxlen, int y_maxlen, int QH, int KH, int D, int VD,
+                              int kernel_size, int stride, int q_chunk_tokens, float sm_scale, void* workspace,
+                              int64_t workspace_bytes, void* stream) {
+  return cmp_attn_bwd_dkdv_impl(q, q_st, q_sh, ck, ck_sr, ck_sh, cv, cv_sr, cv_sh, dO, do_st, do_sh, lse, lse_st,
+                                lse_sh, delta, delta_st, delta_sh, dck, dck_sr, dck_sh, dcv, dcv_sr, dcv_sh, x_cu,
+                                y_cu, B, x_maxlen, y_maxlen, QH, KH, D, VD, kernel_size, stride, q_chunk_tokens,
+                                sm_scale, true, workspace, workspace_bytes, stream);
+}
+
+
 
 int nsa_slc_bwd_chunk_tokens(int T, int KH, int top_n) {
   // list chunk (tokens per work item of the selected-attention dk/dv pass): 1024 for long batches, smaller when
@@ -415,14 +476,15 @@ int nsa_slc_attn_bwd_dq(const void* q, int64_t q_st, int64_t q_sh, const void* k
   return nsa_slc_bwd_dq_launch(p, B, x_maxlen, D, VD, (hipStream_t)stream);
 }
 
-int nsa_slc_attn_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void* k, int64_t k_sr, int64_t k_sh,
+static int slc_attn_bwd_dkdv_impl(const void* q, int64_t q_st, int64_t q_sh, const void* k, int64_t k_sr, int64_t k_sh,
                           const void* v, int64_t v_sr, int64_t v_sh, const void* dO, int64_t do_st,
                           int64_t do_sh, const float* lse, int64_t lse_st, int64_t lse_sh, const float* delta,
                           int64_t delta_st, int64_t delta_sh, float* dk, int64_t dk_sr, int64_t dk_sh, float* dv,
                           int64_t dv_sr, int64_t dv_sh, const int32_t* x_cu, const int32_t* kblk_cu,
                           const int32_t* blk_seq, const int32_t* csr_off, const int32_t* csr_tok,
                           const int32_t* item_off, int nblk_total, int chunk_tokens, int n_items_bound, int B,
-                          int QH, int KH, int D, int VD, int block_size, float sm_scale, void* stream) {
+                          int QH, int KH, int D, int VD, int block_size, float sm_scale, bool deterministic,
+                          void* workspace, int64_t workspace_bytes, void* stream) {
   int rc = check_heads("slc_attn_bwd_dkdv", QH, KH, D, VD);
   if (rc) return rc;
   NSA_REQUIRE(block_size % 32 == 0 && block_size > 0, NSA_ERR_UNSUPPORTED,
@@ -436,8 +498,60 @@ int nsa_slc_attn_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void*
   p.x_cu = x_cu; p.k_cu = x_cu;
   p.csr_off = csr_off; p.csr_tok = csr_tok; p.item_off = item_off; p.blk_seq = blk_seq; p.kblk_cu = kblk_cu;
   p.nblk_total = nblk_total; p.chunk_tokens = chunk_tokens; p.block_size = block_size;
-  return nsa_bwd_dkdv_launch(p, 2, B, 0, 0, D, VD, n_items_bound, (hipStream_t)stream);
+  if (!deterministic) return nsa_bwd_dkdv_launch(p, 2, B, 0, 0, D, VD, n_items_bound, (hipStream_t)stream);
+  if (n_items_bound <= 0) return NSA_OK;
+  const int64_t slots = nsa_bwd_dkdv_slc_slots(KH, n_items_bound, block_size);
+  const int64_t kw = nsa_bwd_dkdv_slot_keys(2, block_size);
+  const int64_t dk_bytes = (slots * kw * D * 4 + 255) & ~(int64_t)255;
+  const int64_t need = dk_bytes + slots * kw * VD * 4;
+  NSA_REQUIRE(workspace != nullptr && workspace_bytes >= need, NSA_ERR_WORKSPACE,
+              "slc_attn_bwd_dkdv_det: workspace of %lld bytes, %lld needed", (long long)workspace_bytes,
+              (long long)need);
+  p.dkv_mode = 4;
+  p.part_dk = (float*)workspace;
+  p.part_dv = (float*)((char*)workspace + dk_bytes);
+  rc = nsa_bwd_dkdv_launch(p, 2, B, 0, 0, D, VD, n_items_bound, (hipStream_t)stream);
+  if (rc) return rc;
+  return nsa_dkdv_reduce_slc_launch(p, n_items_bound, D, VD, (hipStream_t)stream);
 }
+
+int nsa_slc_attn_bwd_dkdv(const void* q, int64_t q_st, int64_t q_sh, const void* k, int64_t k_sr, int64_t k_sh,
+                          const void* v, int64_t v_sr, int64_t v_sh, const void* dO, int64_t do_st,
+                          int64_t do_sh, const float* lse, int64_t lse_st, int64_t lse_sh, const float* delta,
+                          int64_t delta_st, int64_t delta_sh, float* dk, int64_t dk_sr, int64_t dk_sh, float* dv,
+                          int64_t dv_sr, int64_t dv_sh, const int32_t* x_cu, const int32_t* kblk_cu,
+                          const int32_t* blk_seq, const int32_t* csr_off, const int32_t* csr_tok,
+                          const int32_t* item_off, int nblk_total, int chunk_tokens, int n_items_bound, int B,
+                          int QH, int KH, int D, int VD, int block_size, float sm_scale, void* stream) {
+  return slc_attn_bwd_dkdv_impl(q, q_st, q_sh, k, k_sr, k_sh, v, v_sr, v_sh, dO, do_st, do_sh, lse, lse_st, lse_sh,
+                                delta, delta_st, delta_sh, dk, dk_sr, dk_sh, dv, dv_sr, dv_sh, x_cu, kblk_cu, blk_seq,
+                                csr_off, csr_tok, item_off, nblk_total, chunk_tokens, n_items_bound, B, QH, KH, D, VD,
+                                block_size, sm_scale, false, nullptr, 0, stream);
+}
+
+int64_t nsa_slc_attn_bwd_dkdv_det_bytes(int n_items_bound, int KH, int D, int VD, int block_size) {
+  if (n_items_bound <= 0 || KH <= 0 || block_size <= 0) return 0;
+  const int64_t slots = nsa_bwd_dkdv_slc_slots(KH, n_items_bound, block_size);
+  const int64_t kw = nsa_bwd_dkdv_slot_keys(2, block_size);
+  return ((slots * kw * D * 4 + 255) & ~(int64_t)255) + slots * kw * VD * 4;
+}
+
+int nsa_slc_attn_bwd_dkdv_det(const void* q, int64_t q_st, int64_t q_sh, const void* k, int64_t k_sr, int64_t k_sh,
+                              const void* v, int64_t v_sr, int64_t v_sh, const void* dO, int64_t do_st,
+                              int64_t do_sh, const float* lse, int64_t lse_st, int64_t lse_sh, const float* delta,
+                              int64_t delta_st, int64_t delta_sh, float* dk, int64_t dk_sr, int64_t dk_sh,
+                              float* dv, int64_t dv_sr, int64_t dv_sh, const int32_t* x_cu, const int32_t* kblk_cu,
+                              const int32_t* blk_seq, const int32_t* csr_off, const int32_t* csr_tok,
+                              const int32_t* item_off, int nblk_total, int chunk_tokens, int n_items_bound, int B,
+                              int QH, int KH, int D, int VD, int block_size, float sm_scale, void* workspace,
+                              int64_t workspace_bytes, void* stream) {
+  return slc_attn_bwd_dkdv_impl(q, q_st, q_sh, k, k_sr, k_sh, v, v_sr, v_sh, dO, do_st, do_sh, lse, lse_st, lse_sh,
+                                delta, delta_st, delta_sh, dk, dk_sr, dk_sh, dv, dv_sr, dv_sh, x_cu, kblk_cu, blk_seq,
+                                csr_off, csr_tok, item_off, nblk_total, chunk_tokens, n_items_bound, B, QH, KH, D, VD,
+                                block_size, sm_scale, true, workspace, workspace_bytes, stream);
+}
+
+
 
 }  // extern "C"
 

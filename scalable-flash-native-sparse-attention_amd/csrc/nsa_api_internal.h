@@ -74,7 +74,9 @@ struct NsaBwdTileParams {
   const float* dq_partial; int64_t dqp_st, dqp_sh;
   void* dk; int64_t dk_sr, dk_sh;                   // dkdv kernels
   void* dv; int64_t dv_sr, dv_sh;
-  int dkv_mode;                                     // 0: store bf16, 1: store fp32, 3: atomic add into fp32
+  int dkv_mode;                                     // 0: store bf16, 1: store fp32, 3: atomic add into fp32,
+                                                    // 4: fp32 store into the workgroup's own slot of part_dk / part_dv
+  float* part_dk; float* part_dv;                   // dkv_mode 4: [slots][keys per workgroup][D | VD]
   const int32_t* x_cu;
   const int32_t* k_cu;
   // gathered (selected-attention) row lists: CSR over (kv head, global selection block)
@@ -95,6 +97,14 @@ int nsa_bwd_dq_tile_launch(const NsaBwdTileParams& p, int mode, int B, int max_q
                            hipStream_t stream);
 int nsa_bwd_dkdv_launch(const NsaBwdTileParams& p, int mode, int B, int max_q_len, int max_k_len, int D, int VD,
                         int n_items_bound, hipStream_t stream);
+// deterministic dk / dv (dkv_mode 4): slots a launch writes, and the ordered sums over them (nsa_dkdv_reduce.hip)
+int64_t nsa_bwd_dkdv_cmp_slots(int B, int KH, int max_q_len, int max_k_len, int q_chunk_tokens, int kernel_size,
+                               int stride);
+int64_t nsa_bwd_dkdv_slc_slots(int KH, int n_items_bound, int block_size);
+int nsa_bwd_dkdv_slot_keys(int mode, int block_size);
+int nsa_dkdv_reduce_cmp_launch(const NsaBwdTileParams& p, int B, int max_q_len, int max_k_len, int D, int VD,
+                               hipStream_t stream);
+int nsa_dkdv_reduce_slc_launch(const NsaBwdTileParams& p, int n_items_bound, int D, int VD, hipStream_t stream);
 
 struct NsaSlcBwdDqParams {
   const bf16_t* q; int64_t q_st, q_sh;

@@ -496,10 +496,14 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
   }
 
   const float osc = p.sm_scale;
+  // dkv_mode 4: the workgroup's own slot of the partial buffers (summed in a fixed order by a second kernel)
+  int64_t slot = 0;
+  if (MODE == MODE_CMP) slot = ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * p.KH + kh;
+  else if (MODE == MODE_SLC) slot = ((int64_t)kh * gridDim.x + blockIdx.x) * gridDim.y + blockIdx.y;
   auto emit = [&](void* base, int64_t off, f32x4 val) {
     if (p.dkv_mode == 0) {
       *reinterpret_cast<bf16x4*>((bf16_t*)base + off) = pack4(val[0], val[1], val[2], val[3]);
-    } else if (p.dkv_mode == 1) {
+    } else if (p.dkv_mode == 1 || p.dkv_mode == 4) {
       *reinterpret_cast<f32x4*>((float*)base + off) = val;
     } else {
       float* dst = (float*)base + off;
@@ -511,14 +515,22 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
   for (int kb = 0; kb < KB; kb++) {
     const int my_key = kw0 + kb * 32 + l32;
     if (my_key >= nkeys) continue;
-    const int64_t koff = ((int64_t)kbase + my_key) * p.dk_sr + (int64_t)kh * p.dk_sh;
-    const int64_t voff = ((int64_t)kbase + my_key) * p.dv_sr + (int64_t)kh * p.dv_sh;
+    int64_t koff = ((int64_t)kbase + my_key) * p.dk_sr + (int64_t)kh * p.dk_sh;
+    int64_t voff = ((int64_t)kbase + my_key) * p.dv_sr + (int64_t)kh * p.dv_sh;
+    void* dk_base = p.dk;
+    void* dv_base = p.dv;
+    if (p.dkv_mode == 4) {
+      koff = (slot * KW + (my_key - key0)) * D;
+      voff = (slot * KW + (my_key - key0)) * VD;
+      dk_base = p.part_dk;
+      dv_base = p.part_dv;
+    }
 #pragma unroll
     for (int dt = 0; dt < D / 32; dt++)
 #pragma unroll
       for (int i4 = 0; i4 < 4; i4++) {
         int d = dt * 32 + i4 * 8 + hl * 4;
-        emit(p.dk, koff + d, f32x4{dkacc[kb][dt][i4 * 4 + 0] * osc, dkacc[kb][dt][i4 * 4 + 1] * osc,
+        emit(dk_base, koff + d, f32x4{dkacc[kb][dt][i4 * 4 + 0] * osc, dkacc[kb][dt][i4 * 4 + 1] * osc,
                                    dkacc[kb][dt][i4 * 4 + 2] * osc, dkacc[kb][dt][i4 * 4 + 3] * osc});
       }
 #pragma unroll
@@ -526,7 +538,7 @@ __global__ __launch_bounds__(NW * 64) void bwd_dkdv_kernel(NsaBwdTileParams p) {
 #pragma unroll
       for (int i4 = 0; i4 < 4; i4++) {
         int d = dt * 32 + i4 * 8 + hl * 4;
-        emit(p.dv, voff + d, f32x4{dvacc[kb][dt][i4 * 4 + 0], dvacc[kb][dt][i4 * 4 + 1], dvacc[kb][dt][i4 * 4 + 2],
+        emit(dv_base, voff + d, f32x4{dvacc[kb][dt][i4 * 4 + 0], dvacc[kb][dt][i4 * 4 + 1], dvacc[kb][dt][i4 * 4 + 2],
                                    dvacc[kb][dt][i4 * 4 + 3]});
       }
   }
@@ -579,6 +591,27 @@ int launch(const NsaBwdTileParams& p0, int mode, int B, int max_q_len, int max_k
 }
 
 }  // namespace
+
+// workgroups (= slots of the partial buffers) of a compressed-branch launch: grid.x * B * KH, as launch() sizes it
+int64_t nsa_bwd_dkdv_cmp_slots(int B, int KH, int max_q_len, int max_k_len, int q_chunk_tokens, int kernel_size,
+                               int stride) {
+  const int KW = 4 * 32 * (nsa_tuning_knob("dkdv_key_blocks", 1) == 2 ? 2 : 1);
+  const int nch = cdiv_i(max_q_len, q_chunk_tokens);
+  int64_t total = 0;
+  for (int kt = 0; kt * KW < max_k_len; kt++) {
+    const int fc = (stride * kt * KW + kernel_size - 1) / q_chunk_tokens;
+    total += nch - (nch < fc ? nch : fc);
+  }
+  return total * B * KH;
+}
+int64_t nsa_bwd_dkdv_slc_slots(int KH, int n_items_bound, int block_size) {
+  return (int64_t)KH * n_items_bound * (block_size <= 64 ? 1 : cdiv_i(block_size, 128));
+}
+// keys of one slot
+int nsa_bwd_dkdv_slot_keys(int mode, int block_size) {
+  if (mode == MODE_SLC) return block_size <= 64 ? 64 : 128;
+  return 4 * 32 * (nsa_tuning_knob("dkdv_key_blocks", 1) == 2 ? 2 : 1);
+}
 
 int nsa_bwd_dkdv_launch(const NsaBwdTileParams& p, int mode, int B, int max_q_len, int max_k_len, int D, int VD,
                         int n_items_bound, hipStream_t stream) {

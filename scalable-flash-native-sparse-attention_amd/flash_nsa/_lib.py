@@ -9,9 +9,10 @@ import re
 
 _PKG_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB_PATH = os.path.join(_PKG_DIR, "lib", "libnsa_hip.so")
-# the build puts a copy of the header next to the library, so that an installed package needs no source tree
-_HEADER_CANDIDATES = (os.path.join(_PKG_DIR, "lib", "nsa_hip.h"),
-                      os.path.join(os.path.dirname(_PKG_DIR), "include", "nsa_hip.h"))
+# the header of the source tree when there is one; else the copy that the build puts next to the library, so that an
+# installed package needs no source tree
+_HEADER_CANDIDATES = (os.path.join(os.path.dirname(_PKG_DIR), "include", "nsa_hip.h"),
+                      os.path.join(_PKG_DIR, "lib", "nsa_hip.h"))
 HEADER_PATH = next((p for p in _HEADER_CANDIDATES if os.path.exists(p)), _HEADER_CANDIDATES[-1])
 
 _CTYPE = {

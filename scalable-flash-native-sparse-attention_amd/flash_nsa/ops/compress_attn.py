@@ -30,9 +30,11 @@ def cmp_attn_bwd(q, k, v, o, lse, do, dq=None, dkdv_repeat=False, sm_scale=None,
     dq: fresh bf16 tensor, or the caller's fp32 buffer, which is added into; with finalize_dq the fp32 buffer is
     only read and the returned dq is a fresh tensor in q's dtype holding buffer + this branch.
     parts = "dq" / "dkdv" launches only that kernel (the other results are None).
-    dk, dv: fp32 [y_len,KH,*] accumulated with atomics over the q-heads of a group and over query chunks
-    (non-deterministic summation order, as upstream's dkdv_repeat=False path); `dkdv_repeat` is accepted for call
-    compatibility and ignored.  delta may be passed when already known (delta[T,QH] fp32 = rowsum(o*do)).
+    dk, dv: fp32 [y_len,KH,*].  dkdv_repeat=False (default, as upstream): the work items (query chunks) add their
+    partial results with fp32 atomics, so the summation order changes from run to run; dkdv_repeat=True (or
+    NSAHelper.set_deterministic(True)): every work item stores into its own slot of a scratch buffer and a second
+    launch sums the slots in a fixed order -- bit-identical results across runs.
+    delta may be passed when already known (delta[T,QH] fp32 = rowsum(o*do)).
     q_chunk_tokens: queries per work item of the dk/dv kernel (0: chosen by the library from the sizes)."""
     check_thd(do, "do")
     T, QH, D = q.shape
@@ -61,10 +63,16 @@ def cmp_attn_bwd(q, k, v, o, lse, do, dq=None, dkdv_repeat=False, sm_scale=None,
     if parts in ("both", "dkdv"):
         dk = torch.zeros(Y, KH, D, device=q.device, dtype=torch.float32)
         dv = torch.zeros(Y, KH, VD, device=q.device, dtype=torch.float32)
-        _lib.call("nsa_cmp_attn_bwd_dkdv", *common, dk.data_ptr(), dk.stride(0), dk.stride(1), dv.data_ptr(),
-                  dv.stride(0), dv.stride(1), helper.x_cu_seqlens.data_ptr(), helper.y_cu_seqlens.data_ptr(),
-                  helper.batch, helper.x_maxlen, helper.y_maxlen, QH, KH, D, VD, helper.kernel_size, helper.stride,
-                  q_chunk_tokens, sm_scale, _lib.stream_ptr())
+        sizes = (helper.batch, helper.x_maxlen, helper.y_maxlen, QH, KH, D, VD, helper.kernel_size, helper.stride,
+                 q_chunk_tokens)
+        args = (*common, dk.data_ptr(), dk.stride(0), dk.stride(1), dv.data_ptr(), dv.stride(0), dv.stride(1),
+                helper.x_cu_seqlens.data_ptr(), helper.y_cu_seqlens.data_ptr(), *sizes, sm_scale)
+        if dkdv_repeat or getattr(helper, "deterministic", False):
+            ws = torch.empty(max(_lib.value("nsa_cmp_attn_bwd_dkdv_det_bytes", *sizes), 1), dtype=torch.uint8,
+                             device=q.device)
+            _lib.call("nsa_cmp_attn_bwd_dkdv_det", *args, ws.data_ptr(), ws.numel(), _lib.stream_ptr())
+        else:
+            _lib.call("nsa_cmp_attn_bwd_dkdv", *args, _lib.stream_ptr())
     return dq_buf, dk, dv
 
 

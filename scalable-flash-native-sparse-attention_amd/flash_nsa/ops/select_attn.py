@@ -25,11 +25,13 @@ def slc_attn_fwd(q, k, v, topk, sm_scale=None, helper=NSAHelper):
 
 
 def slc_attn_bwd(q, k, v, topk, o, lse, do, dq=None, dk=None, dv=None, sm_scale=None, helper=NSAHelper, delta=None,
-                 bind=None, parts="both"):
+                 bind=None, parts="both", dkdv_repeat=False):
     """Backward of selected attention.  Returns (dq, dk, dv).
     dq: fresh bf16 tensor, or the caller's fp32 buffer (added into).  dk/dv: fp32 [T,KH,*]; the caller's buffers
-    are added into with atomics (summation order is not deterministic, as upstream), otherwise zero-filled ones are
-    created.  `bind` is the inverse index from get_bind_from_find (built here when absent).
+    are added into, otherwise zero-filled ones are created.  dkdv_repeat=False (default): with fp32 atomics, so the
+    summation order changes from run to run (as upstream's dkdv_repeat=False); dkdv_repeat=True (or
+    NSAHelper.set_deterministic(True)): the work items store into slots of a scratch buffer that a second launch adds
+    in a fixed order -- bit-identical results across runs.  `bind` is the inverse index from get_bind_from_find (built here when absent).
     parts = "dq" / "dkdv" launches only that kernel (the other results are None)."""
     from .topk import get_bind_from_find
     check_thd(do, "do")
@@ -56,11 +58,16 @@ def slc_attn_bwd(q, k, v, topk, o, lse, do, dq=None, dk=None, dv=None, sm_scale=
     assert dk.dtype == torch.float32 and dv.dtype == torch.float32
     if bind is None:
         bind = get_bind_from_find(topk, helper)
-    _lib.call("nsa_slc_attn_bwd_dkdv", *common, dk.data_ptr(), dk.stride(0), dk.stride(1), dv.data_ptr(),
-              dv.stride(0), dv.stride(1), helper.x_cu_seqlens.data_ptr(), helper.k_cu_seqlens.data_ptr(),
-              helper.blk_seq.data_ptr(), bind["csr_off"].data_ptr(), bind["csr_tok"].data_ptr(),
-              bind["item_off"].data_ptr(), bind["nblk"], bind["chunk_tokens"], bind["n_items_bound"], helper.batch,
-              QH, KH, D, VD, helper.block_size, sm_scale, _lib.stream_ptr())
+    args = (*common, dk.data_ptr(), dk.stride(0), dk.stride(1), dv.data_ptr(), dv.stride(0), dv.stride(1),
+            helper.x_cu_seqlens.data_ptr(), helper.k_cu_seqlens.data_ptr(), helper.blk_seq.data_ptr(),
+            bind["csr_off"].data_ptr(), bind["csr_tok"].data_ptr(), bind["item_off"].data_ptr(), bind["nblk"],
+            bind["chunk_tokens"], bind["n_items_bound"], helper.batch, QH, KH, D, VD, helper.block_size, sm_scale)
+    if dkdv_repeat or getattr(helper, "deterministic", False):
+        nbytes = _lib.value("nsa_slc_attn_bwd_dkdv_det_bytes", bind["n_items_bound"], KH, D, VD, helper.block_size)
+        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=q.device)
+        _lib.call("nsa_slc_attn_bwd_dkdv_det", *args, ws.data_ptr(), ws.numel(), _lib.stream_ptr())
+    else:
+        _lib.call("nsa_slc_attn_bwd_dkdv", *args, _lib.stream_ptr())
     return dq_buf, dk, dv
 
 

@@ -56,6 +56,7 @@ class NSAHelper:
     k_len = 0
     blk_seq = None  # [k_len] sequence id of every selection block (used by the inverse index)
     batch = 0
+    deterministic = False       # dk / dv summed in a fixed order instead of with atomics (set_deterministic)
     _registered = None          # the cu_seqlens tensor object of the registered batch and its version counter
     _registered_version = -1
     _host_cu = None
@@ -82,6 +83,13 @@ class NSAHelper:
         cls.recompute_slc_o = recompute_slc_o
         cls.recompute_cmp_kv = recompute_cmp_kv
         cls.recompute_cmp_o = recompute_cmp_o
+
+    @classmethod
+    def set_deterministic(cls, deterministic=True):
+        """dK / dV of the compressed and the selected branch summed in a run-independent order (what upstream's
+        dkdv_repeat=True buys): the backward kernels store per-work-item partial results that a second launch adds in
+        a fixed order, instead of fp32 atomic additions.  Costs scratch memory and a few per cent of the backward."""
+        cls.deterministic = bool(deterministic)
 
     @classmethod
     def set_pipeline_parallel_world_size(cls, pp_size):
@@ -171,7 +179,8 @@ class BwdNSAHelper:
     between a forward and its backward (upstream flash_nsa/utils.py:465-482)."""
     _FIELDS = ("kernel_size", "stride", "block_size", "window_size", "top_n", "num_init_blocks", "num_local_blocks",
                "x_cu_seqlens", "x_seqlens", "x_maxlen", "y_cu_seqlens", "y_seqlens", "y_maxlen", "y_len",
-               "k_cu_seqlens", "k_seqlens", "k_maxlen", "k_len", "blk_seq", "batch", "cmp_k_method", "cmp_v_method")
+               "k_cu_seqlens", "k_seqlens", "k_maxlen", "k_len", "blk_seq", "batch", "cmp_k_method", "cmp_v_method",
+               "deterministic")
 
     def __init__(self):
         for f in self._FIELDS:

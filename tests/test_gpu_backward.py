@@ -414,3 +414,65 @@ def test_weight_gradient_accumulates_into_main_grad(device):
     assert mixed.cmp_k_weight.grad is None
     assert mixed.cmp_v_weight.grad_added_to_main_grad is True
     assert mixed.cmp_v_weight.grad is not None and mixed.cmp_v_weight.grad.shape == mixed.cmp_v_weight.shape
+
+
+@pytest.mark.parametrize("block_size,lens,QH,KH", [(64, [5000, 700, 333, 64, 0, 1500], 32, 2),
+                                                   (128, [3000, 129], 16, 2), (32, [2500, 77], 8, 4)])
+def test_deterministic_dk_dv(device, block_size, lens, QH, KH):
+    """dkdv_repeat=True / NSAHelper.set_deterministic: the work items of the dk/dv kernels store into their own slots
+    and a second launch sums them in a fixed order.  Two runs are bit-identical in every gradient, and the results
+    agree with the default (atomic) mode to the order of fp32 summation.  The sequences are long enough for several
+    query chunks per key tile and several list chunks per selection block (forced small chunk sizes)."""
+    from flash_nsa import NSAConfig, NSACore, NSAHelper
+    from flash_nsa.ops.compress_kv import mean_pooling_fwd
+    from flash_nsa.ops.compress_attn import cmp_attn_fwd, cmp_attn_bwd
+    from flash_nsa.ops.select_attn import slc_attn_fwd, slc_attn_bwd
+    from flash_nsa.ops.topk import slc_topk_indices, get_bind_from_find
+    D = 128
+    cu = make_cu(lens)
+    T = int(cu[-1])
+    q, k, v, w = [t.to(device) for t in make_qkvw(T, QH, KH, D, seed=120)]
+    do = randn_bf16(T, QH, D, seed=125).to(device)
+    # the operators, with chunk sizes that give every key several work items
+    H = setup_helper(cu.to(device), block_size=block_size, top_n=6)
+    ck, cv = mean_pooling_fwd(k), mean_pooling_fwd(v)
+    o, lse = cmp_attn_fwd(q, ck, cv)
+    runs = [cmp_attn_bwd(q, ck, cv, o, lse, do, dkdv_repeat=True, q_chunk_tokens=256, parts="dkdv")[1:] for _ in range(3)]
+    for r in runs[1:]:
+        assert torch.equal(r[0], runs[0][0]) and torch.equal(r[1], runs[0][1]), "compressed dk/dv differ between runs"
+    _, dk_a, dv_a = cmp_attn_bwd(q, ck, cv, o, lse, do, q_chunk_tokens=256, parts="dkdv")
+    assert_close(runs[0][0], dk_a, "compressed dk: ordered sum vs atomics", atol=1e-3, rtol=1e-4)
+    assert_close(runs[0][1], dv_a, "compressed dv: ordered sum vs atomics", atol=1e-3, rtol=1e-4)
+    topk, _ = slc_topk_indices(q, ck, lse)
+    so, slse = slc_attn_fwd(q, k, v, topk)
+    bind = get_bind_from_find(topk, chunk_tokens=64)
+    base = torch.full((T, KH, D), 0.5, device=device, dtype=torch.float32)   # dk / dv are added into
+    sruns = []
+    for _ in range(3):
+        dk, dv = base.clone(), base.clone()
+        slc_attn_bwd(q, k, v, topk, so, slse, do, None, dk, dv, bind=bind, parts="dkdv", dkdv_repeat=True)
+        sruns.append((dk, dv))
+    for r in sruns[1:]:
+        assert torch.equal(r[0], sruns[0][0]) and torch.equal(r[1], sruns[0][1]), "selected dk/dv differ between runs"
+    dk, dv = base.clone(), base.clone()
+    slc_attn_bwd(q, k, v, topk, so, slse, do, None, dk, dv, bind=bind, parts="dkdv")
+    assert_close(sruns[0][0], dk, "selected dk: ordered sum vs atomics", atol=1e-3, rtol=1e-4)
+    assert_close(sruns[0][1], dv, "selected dv: ordered sum vs atomics", atol=1e-3, rtol=1e-4)
+    # the fused core: every gradient bit-identical across runs, and equal to the default mode up to summation order
+    core = NSACore(NSAConfig(head_dim=D, num_heads=QH, num_kv_heads=KH, block_size=block_size, top_n=6))
+
+    def run():
+        ts = [t.clone().requires_grad_() for t in (q, k, v, w)]
+        core(*ts, cu.to(device)).backward(do)
+        return [t.grad for t in ts]
+
+    try:
+        NSAHelper.set_deterministic(True)
+        a, b = run(), run()
+    finally:
+        NSAHelper.set_deterministic(False)
+    for name, x, y in zip(("dq", "dk", "dv", "dw"), a, b):
+        assert torch.equal(x, y), f"{name} differs between two deterministic runs"
+    c = run()
+    for name, x, y in zip(("dq", "dk", "dv", "dw"), a, c):
+        assert_close(x, y.float(), f"{name}: deterministic vs default mode", atol=2e-3, rtol=8e-3, row_scale=True)
