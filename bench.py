@@ -320,6 +320,10 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain 1 GiB device-to-device copy kernel, so that a counter run of this "
                          "command holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE with")
+    ap.add_argument("--decode-leg", type=str, default="all", choices=["all", "hot", "cold", "unstaggered", "cache-write"],
+                    help="run only this leg of the decode benchmark (for kernel traces that should reproduce one "
+                         "reported figure)")
+    ap.add_argument("--decode-only", action="store_true", help="skip the training step (with --decode-leg)")
     ap.add_argument("--sweep", type=str, default=None,
                     help="comma-separated sequence lengths: print forward / backward times per length and exit")
     args = ap.parse_args()
@@ -339,6 +343,10 @@ def main():
         length_sweep([int(x) for x in args.sweep.split(",")])
         return
     dev = torch.device("cuda:0")
+    if args.decode_only:
+        from bench_decode import decode_bench
+        print(json.dumps({"decode": decode_bench(dev, leg=args.decode_leg)}))
+        return
     T, QH, KH, D = args.seq_len, 64, 4, 128
     g = torch.Generator(device=dev).manual_seed(0)
     rnd = lambda *s: torch.randn(*s, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
@@ -412,9 +420,27 @@ def main():
         "algorithmic_tflop": {"fwd": fl["fwd_total"] / 1e12, "bwd": fl["bwd_total"] / 1e12},
         "stage_ms": {k_: round(v_, 4) for k_, v_ in stages.items()},
         "stage_tflops": {s: round(fl[s] / (stages[s] * 1e-3) / 1e12, 1) for s in mfma_stages},
+        # fraction of the bf16 MFMA peak of every matrix-bound stage kernel (the worst kernel, not only the longest)
+        "stage_frac": {s: round(fl[s] / (stages[s] * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4) for s in mfma_stages},
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": achieved, "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS, "traffic": traffic},
+                     "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS, "traffic": traffic,
+                     # the whole step against the same peak
+                     "step_frac": total_flops / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+                     "fwd_frac": fl["fwd_total"] / (fwd_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS},
     }
+    # the same step with dK / dV summed in a run-independent order (NSAHelper.set_deterministic)
+    from flash_nsa import NSAHelper
+    NSAHelper.set_deterministic(True)
+    try:
+        step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        result["ms_per_step_deterministic"] = (time.perf_counter() - t0) * 1e3 / args.steps
+    finally:
+        NSAHelper.set_deterministic(False)
     if traffic is not None:
         # the selected-block kernels re-read K/V blocks that fall out of the 4 MB L2 slices: their launch time is
         # set by this memory-side rate rather than by the MFMA work
@@ -422,7 +448,7 @@ def main():
         result["roofline"]["memory_side_frac_of_hbm_peak"] = result["roofline"]["memory_side_gbs"] / PEAK_HBM_GBS
     if not args.no_decode:
         from bench_decode import decode_bench, cache_writer_bench
-        result["decode"] = decode_bench(dev)
+        result["decode"] = decode_bench(dev, leg=args.decode_leg)
         result["cache_writer"] = cache_writer_bench(dev)
         result["layer"] = layer_bench(dev, T, QH, KH, D)
     if not args.no_cpu:

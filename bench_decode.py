@@ -107,8 +107,10 @@ def _time_replays(graphs, reps, warmup):
     return s.elapsed_time(e) * 1e3 / reps
 
 
-def decode_bench(dev, reps=500, warmup=100, cold_copies=6):
-    """Hot: one graph replayed over one batch (its 342 MB of K/V can stay partly in the 256 MB memory-side cache between
+def decode_bench(dev, reps=500, warmup=100, cold_copies=6, leg="all"):
+    """leg: "all", or one of "hot", "cold", "unstaggered", "cache-write" to run that leg alone (a kernel trace of the
+    command then holds the launches of one reported figure only).
+    Hot: one graph replayed over one batch (its 342 MB of K/V can stay partly in the 256 MB memory-side cache between
     replays).  Cold: `cold_copies` copies of the batch in disjoint memory, one graph each, replayed round-robin, so
     that (cold_copies - 1) x 342 MB of other K/V pass through the caches before a copy is read again: every replay
     streams its K/V from HBM."""
@@ -125,6 +127,17 @@ def decode_bench(dev, reps=500, warmup=100, cold_copies=6):
     eager = nsa_decode(*args, **kw)
     torch.cuda.synchronize()
     graph, out = _capture(lambda: nsa_decode(*args, **kw))
+    want = lambda name: leg in ("all", name)
+    if not want("hot"):
+        res = {"workload": "paged NSA decode, batch 64, ctx uniform [4096,32768] (seed 3), page 256, leg " + leg,
+               "algorithmic_bytes": algorithmic_bytes(c["lens"])}
+        if want("cold"):
+            _decode_cold_leg(res, c, graph, out, eager, args_of, kw, reps, cold_copies)
+        if want("unstaggered"):
+            _decode_unstaggered_leg(res, dev, eager, args_of, kw, reps, warmup)
+        if want("cache-write"):
+            _decode_cache_write_leg(res, c, dev, args, eager, kw, reps, warmup)
+        return res
     us = _time_replays([graph], reps, warmup)
     same = bool(torch.equal(out, eager))
     # eager (no graph) for comparison
@@ -143,7 +156,18 @@ def decode_bench(dev, reps=500, warmup=100, cold_copies=6):
            "graph_equals_eager": same, "algorithmic_bytes": nbytes,
            "roofline": {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                         "frac": gbs / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_DEFAULT_CASE}}
-    # cold: copies of the pool, tables and inputs at other addresses
+    if leg == "hot":
+        return res
+    _decode_cold_leg(res, c, graph, out, eager, args_of, kw, reps, cold_copies)
+    _decode_unstaggered_leg(res, dev, eager, args_of, kw, reps, warmup)
+    _decode_cache_write_leg(res, c, dev, args, eager, kw, reps, warmup)
+    return res
+
+
+def _decode_cold_leg(res, c, graph, out, eager, args_of, kw, reps, cold_copies):
+    """copies of the pool, tables and inputs at other addresses, one graph each, replayed in turn"""
+    from flash_nsa import nsa_decode
+    nbytes = res["algorithmic_bytes"]
     copies = [c] + [dict(c, **{n: c[n].clone() for n in ("q", "k", "v", "w", "ctx", "bt", "slots", "cbt")})
                     for _ in range(cold_copies - 1)]
     graphs, outs = [graph], [out]
@@ -159,9 +183,13 @@ def decode_bench(dev, reps=500, warmup=100, cold_copies=6):
     res["cold_equals_hot"] = all(bool(torch.equal(o, eager)) for o in outs)
     res["roofline_cold"] = {"bound": "hbm", "achieved": cold_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                             "frac": cold_gbs / PEAK_HBM_GBS, "traffic": None}
-    del copies, graphs, outs
-    # the same batch in pools whose K and V bases coincide modulo 1 KB (one pool allocated right behind the other, as
-    # upstream's engine does): both streams of a workgroup then share a quarter of the memory channels
+
+
+def _decode_unstaggered_leg(res, dev, eager, args_of, kw, reps, warmup):
+    """the same batch in pools whose K and V bases coincide modulo 1 KB (one pool allocated right behind the other, as
+    upstream's engine does): both streams of a workgroup then share a quarter of the memory channels"""
+    from flash_nsa import nsa_decode
+    from synthetic_decode import build_decode_case, pool_all_rows
     ca = build_decode_case(dev, staggered_pools=False)
     pool_all_rows(ca, dev)
     aa = args_of(ca)
@@ -169,8 +197,11 @@ def decode_bench(dev, reps=500, warmup=100, cold_copies=6):
     ga, oa = _capture(lambda: nsa_decode(*aa, **kw))
     res["us_per_step_unstaggered_pools"] = _time_replays([ga], reps, warmup)
     res["unstaggered_equals_staggered"] = bool(torch.equal(oa, eager))
-    del ca, aa, ga, oa
-    # the same step with the cache write of the newest token's K/V inside the launch (KV-cache writer fused)
+
+
+def _decode_cache_write_leg(res, c, dev, args, eager, kw, reps, warmup):
+    """the same step with the cache write of the newest token's K/V inside the launch (KV-cache writer fused)"""
+    from flash_nsa import nsa_decode
     page = c["page"]
     KH, D = c["k"].size(2), c["k"].size(3)
     newest = [int(c["bt"][b, (L - 1) // page]) * page + (L - 1) % page for b, L in enumerate(c["lens"])]
@@ -183,7 +214,6 @@ def decode_bench(dev, reps=500, warmup=100, cold_copies=6):
     graph2, out2 = _capture(lambda: nsa_decode(*args, **kw2))
     res["us_per_step_with_cache_write"] = _time_replays([graph2], reps, warmup)
     res["cache_write_equals_plain"] = bool(torch.equal(out2, eager))
-    return res
 
 
 def cache_writer_bench(dev, reps=50):
