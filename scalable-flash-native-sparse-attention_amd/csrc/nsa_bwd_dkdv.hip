@@ -548,7 +548,9 @@ template <int D, int VD>
 int launch(const NsaBwdTileParams& p0, int mode, int B, int max_q_len, int max_k_len, int n_items_bound,
            hipStream_t stream) {
   NsaBwdTileParams p = p0;
-  const int kb_cmp = nsa_tuning_knob("dkdv_key_blocks", 1);  // 32-key blocks per wave of the cmp / swa kernels
+  // the variant with two 32-key blocks per wave exists for the head dims it was measured on
+  constexpr bool KB2_BUILT = D >= 64 && D <= 192;
+  const int kb_cmp = KB2_BUILT ? nsa_tuning_knob("dkdv_key_blocks", 1) : 1;  // 32-key blocks per wave (cmp / swa)
   if (mode == MODE_CMP) {
     if (B <= 0 || max_k_len <= 0) return NSA_OK;
     const int KW = 4 * 32 * (kb_cmp == 2 ? 2 : 1);
@@ -560,17 +562,23 @@ int launch(const NsaBwdTileParams& p0, int mode, int B, int max_q_len, int max_k
     }
     if (total <= 0) return NSA_OK;
     dim3 grid(total, B, p.KH);
-    if (kb_cmp == 2) bwd_dkdv_kernel<D, VD, MODE_CMP, 4, 2><<<grid, 256, 0, stream>>>(p);
-    else bwd_dkdv_kernel<D, VD, MODE_CMP, 4, 1><<<grid, 256, 0, stream>>>(p);
+    if constexpr (KB2_BUILT) {
+      if (kb_cmp == 2) bwd_dkdv_kernel<D, VD, MODE_CMP, 4, 2><<<grid, 256, 0, stream>>>(p);
+      else bwd_dkdv_kernel<D, VD, MODE_CMP, 4, 1><<<grid, 256, 0, stream>>>(p);
+    } else {
+      bwd_dkdv_kernel<D, VD, MODE_CMP, 4, 1><<<grid, 256, 0, stream>>>(p);
+    }
   } else if (mode == MODE_SWA) {
     if (B <= 0 || max_k_len <= 0) return NSA_OK;
-    if (kb_cmp == 2) {
-      dim3 grid(cdiv_i(max_k_len, 256), B, p.KH);
-      bwd_dkdv_kernel<D, VD, MODE_SWA, 4, 2><<<grid, 256, 0, stream>>>(p);
-    } else {
-      dim3 grid(cdiv_i(max_k_len, 128), B, p.KH);
-      bwd_dkdv_kernel<D, VD, MODE_SWA, 4, 1><<<grid, 256, 0, stream>>>(p);
+    if constexpr (KB2_BUILT) {
+      if (kb_cmp == 2) {
+        dim3 grid(cdiv_i(max_k_len, 256), B, p.KH);
+        bwd_dkdv_kernel<D, VD, MODE_SWA, 4, 2><<<grid, 256, 0, stream>>>(p);
+        return nsa_check_launch("bwd_dkdv_kernel");
+      }
     }
+    dim3 grid(cdiv_i(max_k_len, 128), B, p.KH);
+    bwd_dkdv_kernel<D, VD, MODE_SWA, 4, 1><<<grid, 256, 0, stream>>>(p);
   } else {
     if (n_items_bound <= 0) return NSA_OK;
     if (p.block_size <= 0 || p.block_size % 32 != 0) {
@@ -595,7 +603,7 @@ int launch(const NsaBwdTileParams& p0, int mode, int B, int max_q_len, int max_k
 // workgroups (= slots of the partial buffers) of a compressed-branch launch: grid.x * B * KH, as launch() sizes it
 int64_t nsa_bwd_dkdv_cmp_slots(int B, int KH, int max_q_len, int max_k_len, int q_chunk_tokens, int kernel_size,
                                int stride) {
-  const int KW = 4 * 32 * (nsa_tuning_knob("dkdv_key_blocks", 1) == 2 ? 2 : 1);
+  const int KW = nsa_bwd_dkdv_slot_keys(0, 0);
   const int nch = cdiv_i(max_q_len, q_chunk_tokens);
   int64_t total = 0;
   for (int kt = 0; kt * KW < max_k_len; kt++) {
@@ -618,6 +626,8 @@ int nsa_bwd_dkdv_launch(const NsaBwdTileParams& p, int mode, int B, int max_q_le
   if (D == 128 && VD == 128) return launch<128, 128>(p, mode, B, max_q_len, max_k_len, n_items_bound, stream);
   if (D == 64 && VD == 64) return launch<64, 64>(p, mode, B, max_q_len, max_k_len, n_items_bound, stream);
   if (D == 192 && VD == 128) return launch<192, 128>(p, mode, B, max_q_len, max_k_len, n_items_bound, stream);
+  if (D == 256 && VD == 256) return launch<256, 256>(p, mode, B, max_q_len, max_k_len, n_items_bound, stream);
+  if (D == 32 && VD == 32) return launch<32, 32>(p, mode, B, max_q_len, max_k_len, n_items_bound, stream);
   nsa_set_error("attention dk/dv: unsupported head dims D=%d VD=%d", D, VD);
   return NSA_ERR_UNSUPPORTED;
 }

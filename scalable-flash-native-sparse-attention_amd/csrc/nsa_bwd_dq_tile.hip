@@ -235,6 +235,8 @@ int dispatch(const NsaBwdTileParams& p, int B, int max_q_len, int D, int VD, hip
     else bwd_dq_tile_kernel<128, 128, MODE, 1, false><<<grid, 256, 0, stream>>>(p);
   } else if (D == 64 && VD == 64) bwd_dq_tile_kernel<64, 64, MODE, 2, false><<<grid, 256, 0, stream>>>(p);
   else if (D == 192 && VD == 128) bwd_dq_tile_kernel<192, 128, MODE, 1, false><<<grid, 256, 0, stream>>>(p);
+  else if (D == 256 && VD == 256) bwd_dq_tile_kernel<256, 256, MODE, 1, false><<<grid, 256, 0, stream>>>(p);
+  else if (D == 32 && VD == 32) bwd_dq_tile_kernel<32, 32, MODE, 2, false><<<grid, 256, 0, stream>>>(p);
   else {
     nsa_set_error("attention dq: unsupported head dims D=%d VD=%d", D, VD);
     return NSA_ERR_UNSUPPORTED;

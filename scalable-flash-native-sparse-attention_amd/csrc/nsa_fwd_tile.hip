@@ -396,7 +396,12 @@ int launch_fwd_tile(const NsaFwdTileParams& p, int B, int max_q_len, hipStream_t
   const int variant = nsa_tuning_knob("fwd_variant", 0);
   constexpr bool pow2 = (D == 64 || D == 128) && (VD == 64 || VD == 128);
   const bool async = variant == 4 || (variant == 0 && MODE == MODE_CMP && pow2);
-  if (variant == 2) {
+  if constexpr (D > 192 || VD > 128) {
+    // head dims of 256: the output accumulators alone take 128 registers, one workgroup per CU
+    dim3 grid(cdiv_i(max_q_len * p.G, 128), B, p.KH);
+    fwd_tile_kernel<D, VD, MODE, PAGED, 1, 1, false><<<grid, 256, 0, stream>>>(p);
+    return nsa_check_launch("fwd_tile_kernel");
+  } else if (variant == 2) {
     dim3 grid(cdiv_i(max_q_len * p.G, 256), B, p.KH);
     fwd_tile_kernel<D, VD, MODE, PAGED, 2, 1, false><<<grid, 256, 0, stream>>>(p);
   } else if (variant == 3) {
@@ -417,7 +422,9 @@ int dispatch_fwd_tile(const NsaFwdTileParams& p, int B, int max_q_len, int D, in
   if (D == 128 && VD == 128) return launch_fwd_tile<128, 128, MODE, PAGED>(p, B, max_q_len, stream);
   if (D == 64 && VD == 64) return launch_fwd_tile<64, 64, MODE, PAGED>(p, B, max_q_len, stream);
   if (D == 192 && VD == 128) return launch_fwd_tile<192, 128, MODE, PAGED>(p, B, max_q_len, stream);
-  nsa_set_error("attention forward: unsupported head dims D=%d VD=%d (built: 128/128, 64/64, 192/128)", D, VD);
+  if (D == 256 && VD == 256) return launch_fwd_tile<256, 256, MODE, PAGED>(p, B, max_q_len, stream);
+  if (D == 32 && VD == 32) return launch_fwd_tile<32, 32, MODE, PAGED>(p, B, max_q_len, stream);
+  nsa_set_error("attention forward: unsupported head dims D=%d VD=%d (built: 128/128, 64/64, 192/128, 256/256, 32/32)", D, VD);
   return NSA_ERR_UNSUPPORTED;
 }
 

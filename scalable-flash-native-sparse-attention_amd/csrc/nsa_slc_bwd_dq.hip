@@ -190,6 +190,8 @@ int nsa_slc_bwd_dq_launch(const NsaSlcBwdDqParams& p, int B, int max_q_len, int 
   if (D == 128 && VD == 128) slc_dq_kernel<128, 128><<<grid, 256, 0, stream>>>(p);
   else if (D == 64 && VD == 64) slc_dq_kernel<64, 64><<<grid, 256, 0, stream>>>(p);
   else if (D == 192 && VD == 128) slc_dq_kernel<192, 128><<<grid, 256, 0, stream>>>(p);
+  else if (D == 256 && VD == 256) slc_dq_kernel<256, 256><<<grid, 256, 0, stream>>>(p);
+  else if (D == 32 && VD == 32) slc_dq_kernel<32, 32><<<grid, 256, 0, stream>>>(p);
   else {
     nsa_set_error("selected attention dq: unsupported head dims D=%d VD=%d", D, VD);
     return NSA_ERR_UNSUPPORTED;

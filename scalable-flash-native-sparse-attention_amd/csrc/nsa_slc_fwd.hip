@@ -234,6 +234,8 @@ int dispatch_slc(const NsaSlcParams& p, int B, int max_q_len, int D, int VD, hip
   if (D == 128 && VD == 128) return launch_slc<128, 128, PAGED>(p, B, max_q_len, stream);
   if (D == 64 && VD == 64) return launch_slc<64, 64, PAGED>(p, B, max_q_len, stream);
   if (D == 192 && VD == 128) return launch_slc<192, 128, PAGED>(p, B, max_q_len, stream);
+  if (D == 256 && VD == 256) return launch_slc<256, 256, PAGED>(p, B, max_q_len, stream);
+  if (D == 32 && VD == 32) return launch_slc<32, 32, PAGED>(p, B, max_q_len, stream);
   nsa_set_error("selected attention forward: unsupported head dims D=%d VD=%d", D, VD);
   return NSA_ERR_UNSUPPORTED;
 }

@@ -537,6 +537,8 @@ int nsa_topk_launch(const NsaTopkParams& p, bool paged, int B, int max_q_len, in
   if (D == 128) return paged ? dispatch_gp<128, true>(p, B, max_q_len, stream) : dispatch_gp<128, false>(p, B, max_q_len, stream);
   if (D == 64) return paged ? dispatch_gp<64, true>(p, B, max_q_len, stream) : dispatch_gp<64, false>(p, B, max_q_len, stream);
   if (D == 192) return paged ? dispatch_gp<192, true>(p, B, max_q_len, stream) : dispatch_gp<192, false>(p, B, max_q_len, stream);
+  if (D == 256) return paged ? dispatch_gp<256, true>(p, B, max_q_len, stream) : dispatch_gp<256, false>(p, B, max_q_len, stream);
+  if (D == 32) return paged ? dispatch_gp<32, true>(p, B, max_q_len, stream) : dispatch_gp<32, false>(p, B, max_q_len, stream);
   nsa_set_error("top-k: unsupported head dim D=%d", D);
   return NSA_ERR_UNSUPPORTED;
 }

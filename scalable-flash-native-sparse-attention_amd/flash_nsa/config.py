@@ -9,7 +9,7 @@ def _is_pow2(n: int) -> bool:
 
 
 # (qk head dim, v head dim) pairs the kernels are built for
-SUPPORTED_HEAD_DIMS = ((128, 128), (64, 64), (192, 128))
+SUPPORTED_HEAD_DIMS = ((128, 128), (64, 64), (192, 128), (32, 32), (256, 256))
 
 
 def check_supported(qk_head_dim, v_head_dim, kernel_size, stride, block_size):

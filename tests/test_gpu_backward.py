@@ -235,6 +235,10 @@ def test_nsa_core_fwd_bwd(device, core, lens, QH, KH, D, methods):
     dict(kernel_size=32, stride=16, block_size=96, top_n=5, window_size=64),
     dict(kernel_size=64, stride=16, block_size=256, top_n=3, window_size=128),
     dict(kernel_size=32, stride=32, block_size=160, top_n=4, num_local_blocks=1, window_size=32),
+    # head dims other than 128 (upstream accepts every power of two, flash_nsa/ops/compress_attn.py:542)
+    dict(head_dim=32, top_n=6, window_size=100),
+    dict(head_dim=256, top_n=6, window_size=100),
+    dict(head_dim=64, top_n=6, window_size=100),
 ])
 def test_nsa_core_other_hyperparameters(device, hp):
     """Compression window / stride, selection block, top-n, forced blocks and window other than the defaults
@@ -244,7 +248,8 @@ def test_nsa_core_other_hyperparameters(device, hp):
     from flash_nsa.ops.compress_attn import cmp_attn_fwd
     from flash_nsa.ops.topk import slc_topk_indices
     from flash_nsa.modules.megatron_level_nsa import compress_kv_fwd
-    lens, QH, KH, D = [1500, 700, 90], 8, 2, 128
+    hp = dict(hp)
+    lens, QH, KH, D = [1500, 700, 90], 8, 2, hp.pop("head_dim", 128)
     cu = make_cu(lens)
     T = int(cu[-1])
     q, k, v, w = make_qkvw(T, QH, KH, D, seed=71)

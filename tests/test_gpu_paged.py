@@ -635,12 +635,13 @@ def test_split_decode_pools_the_new_row_itself(device, nsplit):
     assert torch.equal(o1, o3)
 
 
-def test_decode_qk192_v128_equals_training_last_row(device):
-    """Dqk = 192, Dv = 128, 2 kv heads (the head shape of upstream's inference notebook, cell 43): nsa_decode takes
-    the stage-by-stage kernels here; its output equals the last row of the training forward on the gathered
-    contiguous sequence."""
+@pytest.mark.parametrize("D,VD", [(192, 128), (32, 32), (256, 256)])
+def test_decode_qk192_v128_equals_training_last_row(device, D, VD):
+    """Dqk = 192, Dv = 128, 2 kv heads (the head shape of upstream's inference notebook, cell 43), and head dims of 32
+    and 256: nsa_decode takes the stage-by-stage kernels here; its output equals the last row of the training forward
+    on the gathered contiguous sequence."""
     from flash_nsa import nsa_decode, NSAConfig, NSACore
-    QH, KH, D, VD = 16, 2, 192, 128
+    QH, KH = 16, 2
     ctx = [1000, 333, 64, 2049]
     case = build_pool(ctx, KH, D, VD, page=128, seed=51)
     prepool(case, [L - 1 for L in ctx])

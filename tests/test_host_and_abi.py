@@ -149,10 +149,12 @@ def test_unsupported_shapes_are_rejected_where_the_model_is_configured():
     NSAConfig(qk_head_dim=192, v_head_dim=128)
     with pytest.raises(AssertionError, match="multiples of 32"):
         NSAConfig(block_size=48)
+    NSAConfig(head_dim=256)
+    NSAConfig(head_dim=32)
     with pytest.raises(AssertionError, match="not built"):
-        NSAConfig(head_dim=256)
+        NSAConfig(head_dim=512)
     with pytest.raises(AssertionError, match="not built"):
-        NSAConfig(head_dim=32)
+        NSAConfig(qk_head_dim=256, v_head_dim=128)
     loose = SimpleNamespace(head_dim=128, qk_head_dim=None, v_head_dim=None, num_heads=16, num_kv_heads=1,
                             kernel_size=32, stride=16, block_size=80, cmp_k_method="mean", cmp_v_method="mean")
     for core in (NSACore, HFNSACore):
