@@ -24,8 +24,8 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 # what the same counter reads for a 1 GiB copy: x2.000 and x1.000), measured on the T=65536 workload of this file;
 # reported as roofline.traffic for that workload only.
 MEASURED_TRAFFIC_T64K = {
-    "cmp_dkdv": 34.10e9, "slc_dq": 75.52e9, "slc_fwd": 73.08e9, "slc_dkdv": 36.58e9, "cmp_dq": 7.04e9,
-    "topk": 1.26e9, "cmp_fwd": 2.25e9, "swa_dkdv": 11.38e9, "swa_dq": 6.32e9, "swa_fwd": 3.24e9,
+    "cmp_dkdv": 34.40e9, "slc_dq": 75.55e9, "slc_fwd": 73.02e9, "slc_dkdv": 36.38e9, "cmp_dq": 7.21e9,
+    "topk": 2.30e9, "cmp_fwd": 2.25e9, "swa_dkdv": 11.39e9, "swa_dq": 6.54e9, "swa_fwd": 3.24e9,
 }
 PEAK_HBM_GBS = 8000.0
 
