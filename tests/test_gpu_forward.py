@@ -118,10 +118,12 @@ def test_topk_and_slc_fwd(device, lens, QH, KH, D):
 @pytest.mark.parametrize("lens,QH,KH,D", [([9000, 2500, 700], 32, 2, 128), ([6000, 100], 4, 4, 64),
                                           ([5000, 3000], 4, 2, 128), ([4500], 64, 1, 64)])
 def test_topk_segmented_selection_equals_one_pass(device, lens, QH, KH, D):
-    """Long contexts keep the block scores of one segment of blocks in LDS and merge every finished segment into a
-    running list of winners.  The segment length (a tuning value set through nsa_set_tuning) must not change
-    the result: indices and returned scores are bit-identical to the one-pass selector, and match the oracle."""
+    """Three forms of the block selector must return bit-identical indices and scores: the one-launch kernel with the
+    scores of all blocks in LDS, the same kernel working segment by segment (long contexts; the segment length is a
+    tuning value), and the two-launch form with the scores in a workspace -- in one pass over all tokens and in chunks
+    of as many tokens as a small workspace holds.  All of them match the oracle."""
     from flash_nsa import _lib
+    from flash_nsa.ops import topk as topk_mod
     from flash_nsa.ops.compress_kv import mean_pooling_fwd
     from flash_nsa.ops.compress_attn import cmp_attn_fwd
     from flash_nsa.ops.topk import slc_topk_indices
@@ -135,6 +137,7 @@ def test_topk_segmented_selection_equals_one_pass(device, lens, QH, KH, D):
     G = QH // KH
     results = {}
     try:
+        _lib.call("nsa_set_tuning", b"topk_two_pass", 0)
         for seg in (0, 32, 64, 96):
             if seg == 0 and G <= 2:
                 continue  # the score rows of 64 / 32 tokens per workgroup do not fit in one pass at this length
@@ -143,6 +146,13 @@ def test_topk_segmented_selection_equals_one_pass(device, lens, QH, KH, D):
     finally:
         _lib.call("nsa_reset_tuning")
     results["auto"] = slc_topk_indices(qd, ck, lse, return_slc_prob=True)
+    limit = topk_mod.TOPK_WORKSPACE_LIMIT
+    try:
+        for small in (1 << 20, 300 << 10):   # a few hundred tokens per chunk, chunk edges inside sequences
+            topk_mod.TOPK_WORKSPACE_LIMIT = small
+            results[f"workspace {small}"] = slc_topk_indices(qd, ck, lse, return_slc_prob=True)
+    finally:
+        topk_mod.TOPK_WORKSPACE_LIMIT = limit
     keys = list(results)
     for key in keys[1:]:
         assert torch.equal(results[key][0], results[keys[0]][0]), f"indices differ: segment {key} vs {keys[0]}"
