@@ -333,6 +333,26 @@ int nsa_decode_split(const void* q, int64_t q_st, int64_t q_sh, const void* k_ca
                      int cmp_table_stride, int page_size, int B, int QH, int KH, int D, int VD, int fixed_y_maxlen,
                      int fixed_num_slc_blocks, int kernel_size, int stride, int block_size, int top_n, int num_init,
                      int num_local, int ignore_index, int window, float sm_scale, void* stream);
+/* nsa_decode_split with launch (2) cut as well: upstream's slc_num_splits (flash_nsa/inference/__init__.py:195-196,
+ * inference/select_attn.py:329-331,492-498 -- the selected blocks of one token dealt over several programs, merged
+ * through fp32 partials).  Here slc_nsplit workgroups per (request, kv head) share the window units and the selected
+ * blocks (every one of them repeats the merge of the compressed parts and the selection), and a third launch merges
+ * their partial results and applies the gates.  Worth it only when B x KH workgroups leave most of the GPU idle.
+ * slc_nsplit in [1,16]; 1 = nsa_decode_split.  Extra scratch (caller-allocated, contents undefined):
+ *   sp2_ml [B,KH,slc_nsplit,2,2,16] fp32, sp2_o [B,KH,slc_nsplit,2,16,VD] fp32, cmp_tmp [B,QH,VD] bf16 addressed with
+ *   co_st / co_sh. */
+int nsa_decode_split_parts(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr,
+                           int64_t k_sh, const void* v_cache, int64_t v_sr, int64_t v_sh, const void* w, int64_t w_st,
+                           int64_t w_sh, void* out, int64_t o_st, int64_t o_sh, void* cmp_o, void* slc_o, void* swa_o,
+                           int64_t co_st, int64_t co_sh, float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk,
+                           int64_t tk_sh, int64_t tk_st, float* sp_m, float* sp_l, float* sp_o, void* sp_keep_p,
+                           float* sp_keep_m, int nsplit, const int32_t* cmp_slot_mapping,
+                           const int32_t* context_lens, const int32_t* block_tables, int table_stride,
+                           const int32_t* cmp_block_tables, int cmp_table_stride, int page_size, int B, int QH,
+                           int KH, int D, int VD, int fixed_y_maxlen, int fixed_num_slc_blocks, int kernel_size,
+                           int stride, int block_size, int top_n, int num_init, int num_local, int ignore_index,
+                           int window, float sm_scale, int slc_nsplit, float* sp2_ml, float* sp2_o, void* cmp_tmp,
+                           void* stream);
 /* nsa_decode_split without any allocation.  No counterpart upstream: it is for callers that cannot allocate device
  * memory around the call (code under graph capture, tight serving loops, harnesses that forbid hipMalloc).  The
  * arguments are those of nsa_decode_split minus the five scratch buffers, which are carved out of one file-scope

@@ -796,7 +796,7 @@ int nsa_decode_split_lds_total(int D, int VD, int fixed_y_maxlen, int fixed_num_
   return dyn > 0 ? dyn + nsa_decode_split_static_lds_bytes() : 0;
 }
 
-int nsa_decode_split(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr, int64_t k_sh,
+static int decode_split_impl(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr, int64_t k_sh,
                      const void* v_cache, int64_t v_sr, int64_t v_sh, const void* w, int64_t w_st, int64_t w_sh,
                      void* out, int64_t o_st, int64_t o_sh, void* cmp_o, void* slc_o, void* swa_o, int64_t co_st,
                      int64_t co_sh, float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk, int64_t tk_sh,
@@ -805,7 +805,8 @@ int nsa_decode_split(const void* q, int64_t q_st, int64_t q_sh, const void* k_ca
                      const int32_t* block_tables, int table_stride, const int32_t* cmp_block_tables,
                      int cmp_table_stride, int page_size, int B, int QH, int KH, int D, int VD, int fixed_y_maxlen,
                      int fixed_num_slc_blocks, int kernel_size, int stride, int block_size, int top_n, int num_init,
-                     int num_local, int ignore_index, int window, float sm_scale, void* stream) {
+                     int num_local, int ignore_index, int window, float sm_scale, int slc_nsplit, float* sp2_ml,
+                     float* sp2_o, void* cmp_tmp, void* stream) {
   int rc = check_heads("decode_split", QH, KH, D, VD);
   if (rc) return rc;
   rc = check_nsa_sizes("decode_split", kernel_size, stride, block_size);
@@ -823,7 +824,12 @@ int nsa_decode_split(const void* q, int64_t q_st, int64_t q_sh, const void* k_ca
               fixed_num_slc_blocks);
   NSA_REQUIRE(out && w && sp_m && sp_l && sp_o && sp_keep_p && sp_keep_m, NSA_ERR_BAD_ARG,
               "decode_split: out, w and the five scratch buffers are required");
+  NSA_REQUIRE(slc_nsplit >= 1 && slc_nsplit <= 16, NSA_ERR_BAD_ARG, "decode_split: slc_nsplit %d must be in [1,16]",
+              slc_nsplit);
+  NSA_REQUIRE(slc_nsplit == 1 || (sp2_ml && sp2_o && cmp_tmp), NSA_ERR_BAD_ARG,
+              "decode_split: slc_nsplit > 1 needs the three buffers of the window / selected parts");
   NsaDecodeParams p{};
+  p.slc_nsplit = slc_nsplit; p.sp2_ml = sp2_ml; p.sp2_o = sp2_o; p.cmp_tmp = (bf16_t*)cmp_tmp;
   p.q = (const bf16_t*)q; p.q_st = q_st; p.q_sh = q_sh;
   p.k = (const bf16_t*)k_cache; p.k_sr = k_sr; p.k_sh = k_sh;
   p.v = (const bf16_t*)v_cache; p.v_sr = v_sr; p.v_sh = v_sh;
@@ -844,6 +850,43 @@ int nsa_decode_split(const void* q, int64_t q_st, int64_t q_sh, const void* k_ca
   p.num_init = num_init; p.num_local = num_local; p.ignore_index = ignore_index;
   fill_decode_split(p, fixed_y_maxlen, fixed_num_slc_blocks, table_stride);
   return nsa_decode_split_launch(p, B, D, VD, (hipStream_t)stream);
+}
+
+int nsa_decode_split(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr, int64_t k_sh,
+                     const void* v_cache, int64_t v_sr, int64_t v_sh, const void* w, int64_t w_st, int64_t w_sh,
+                     void* out, int64_t o_st, int64_t o_sh, void* cmp_o, void* slc_o, void* swa_o, int64_t co_st,
+                     int64_t co_sh, float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk, int64_t tk_sh,
+                     int64_t tk_st, float* sp_m, float* sp_l, float* sp_o, void* sp_keep_p, float* sp_keep_m,
+                     int nsplit, const int32_t* cmp_slot_mapping, const int32_t* context_lens,
+                     const int32_t* block_tables, int table_stride, const int32_t* cmp_block_tables,
+                     int cmp_table_stride, int page_size, int B, int QH, int KH, int D, int VD, int fixed_y_maxlen,
+                     int fixed_num_slc_blocks, int kernel_size, int stride, int block_size, int top_n, int num_init,
+                     int num_local, int ignore_index, int window, float sm_scale, void* stream) {
+  return decode_split_impl(q, q_st, q_sh, k_cache, k_sr, k_sh, v_cache, v_sr, v_sh, w, w_st, w_sh, out, o_st, o_sh, cmp_o, slc_o,
+                           swa_o, co_st, co_sh, lse, lse_st, lse_sh, topk, tk_sh, tk_st, sp_m, sp_l, sp_o, sp_keep_p,
+                           sp_keep_m, nsplit, cmp_slot_mapping, context_lens, block_tables, table_stride,
+                           cmp_block_tables, cmp_table_stride, page_size, B, QH, KH, D, VD, fixed_y_maxlen,
+                           fixed_num_slc_blocks, kernel_size, stride, block_size, top_n, num_init, num_local,
+                           ignore_index, window, sm_scale, 1, nullptr, nullptr, nullptr, stream);
+}
+
+int nsa_decode_split_parts(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr, int64_t k_sh,
+                     const void* v_cache, int64_t v_sr, int64_t v_sh, const void* w, int64_t w_st, int64_t w_sh,
+                     void* out, int64_t o_st, int64_t o_sh, void* cmp_o, void* slc_o, void* swa_o, int64_t co_st,
+                     int64_t co_sh, float* lse, int64_t lse_st, int64_t lse_sh, int32_t* topk, int64_t tk_sh,
+                     int64_t tk_st, float* sp_m, float* sp_l, float* sp_o, void* sp_keep_p, float* sp_keep_m,
+                     int nsplit, const int32_t* cmp_slot_mapping, const int32_t* context_lens,
+                     const int32_t* block_tables, int table_stride, const int32_t* cmp_block_tables,
+                     int cmp_table_stride, int page_size, int B, int QH, int KH, int D, int VD, int fixed_y_maxlen,
+                     int fixed_num_slc_blocks, int kernel_size, int stride, int block_size, int top_n, int num_init,
+                     int num_local, int ignore_index, int window, float sm_scale, int slc_nsplit, float* sp2_ml,
+                     float* sp2_o, void* cmp_tmp, void* stream) {
+  return decode_split_impl(q, q_st, q_sh, k_cache, k_sr, k_sh, v_cache, v_sr, v_sh, w, w_st, w_sh, out, o_st, o_sh, cmp_o, slc_o,
+                           swa_o, co_st, co_sh, lse, lse_st, lse_sh, topk, tk_sh, tk_st, sp_m, sp_l, sp_o, sp_keep_p,
+                           sp_keep_m, nsplit, cmp_slot_mapping, context_lens, block_tables, table_stride,
+                           cmp_block_tables, cmp_table_stride, page_size, B, QH, KH, D, VD, fixed_y_maxlen,
+                           fixed_num_slc_blocks, kernel_size, stride, block_size, top_n, num_init, num_local,
+                           ignore_index, window, sm_scale, slc_nsplit, sp2_ml, sp2_o, cmp_tmp, stream);
 }
 
 int nsa_decode_slc_swa_combine(const void* q, int64_t q_st, int64_t q_sh, const void* k_cache, int64_t k_sr,

@@ -149,6 +149,11 @@ struct NsaDecodeParams {
   // probabilities [16][ceil32(y_cap)] and the maxima they refer to [ceil32(y_cap)/32][16]; the final kernel merges
   // the nsplit parts, folds the probabilities into block scores and selects
   _Float16* sp_keep_p; float* sp_keep_m; int nsplit;
+  // two-launch split path with the window and selected branches cut as well (slc_nsplit > 1 parts per request and kv
+  // head): every part writes its un-normalised (m, l, o) of both branches, part 0 the merged compressed-branch
+  // output, and a third launch merges and combines.  sp2_ml [B,KH,slc_nsplit,2 branches,2 (m,l),16],
+  // sp2_o [B,KH,slc_nsplit,2,16,VD] fp32, cmp_tmp [B,QH,VD] bf16
+  int slc_nsplit; float* sp2_ml; float* sp2_o; bf16_t* cmp_tmp;
 };
 int nsa_decode_cmp_topk_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream);
 int nsa_decode_slc_swa_launch(const NsaDecodeParams& p, int B, int D, int VD, hipStream_t stream);

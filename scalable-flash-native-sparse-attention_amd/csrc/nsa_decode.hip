@@ -766,6 +766,9 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecod
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int b = blockIdx.x, kh = blockIdx.y;
+  // the window and selected units of a (request, kv head) may be cut into gridDim.z parts (every part repeats the
+  // prologue and the selection, which all of them need, and writes partial results for a merging launch)
+  const int part = blockIdx.z, nparts = gridDim.z;
   const int G = p.G;
   const int L = p.ctx_lens[b];
   const int t = L - 1;
@@ -874,19 +877,63 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecod
   if (wave < w_first) {
     const int result = select_blocks_wave(imp, t, nb, p, lane, cand_v, cand_i);
     blk_s[lane] = lane < nvalid ? max(result, 0) : 0;
-    if (p.topk && lane < p.top_n) p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + lane] = result;
+    if (p.topk && part == 0 && lane < p.top_n) p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + lane] = result;
   } else {
     if (t >= 0) {
       const int klo = max(0, t - p.window);
       const int k0 = (klo / UK) * UK;
       const int nu = (t - k0) / UK + 1;
-      uf.run(wave - w_first, NW - w_first, nu, klo, t, [&](int u) { return k0 + u * UK; }, tab_s, page, kbase, p.k_sr,
-             vbase, p.v_sr);
+      uf.run(part * (NW - w_first) + wave - w_first, nparts * (NW - w_first), nu, klo, t,
+             [&](int u) { return k0 + u * UK; }, tab_s, page, kbase, p.k_sr, vbase, p.v_sr);
     }
     uf.publish(part_m + wave * 16, part_l + wave * 16, reinterpret_cast<float*>(Vs_all + wave * SLOT));
   }
   __syncthreads();
   const float* part_o = reinterpret_cast<const float*>(Vs_all);
+  // parts: the un-normalised (m, l, o) of this part's waves, one thread per output value (same arithmetic as the
+  // partial kernel of the compressed branch)
+  auto spill_part = [&](int branch, int w0, int nw) {
+    const int64_t base = ((((int64_t)b * p.KH + kh) * nparts + part) * 2 + branch);
+    for (int idx = tid; idx < 16 * VD; idx += NT) {
+      const int h = idx / VD, d = idx - h * VD;
+      float m = NSA_NEG_INF;
+      for (int w = w0; w < w0 + nw; w++) m = fmaxf(m, part_m[w * 16 + h]);
+      float l = 0.f, o = 0.f;
+      if (m != NSA_NEG_INF) {
+        for (int w = w0; w < w0 + nw; w++) {
+          const float mw = part_m[w * 16 + h];
+          const float a = (mw == NSA_NEG_INF) ? 0.f : fast_exp2((mw - m) * p.scale_log2);
+          l += a * part_l[w * 16 + h];
+          o += a * part_o[w * (SLOT / 2) + h * UF::OLD + d];
+        }
+      }
+      p.sp2_o[(base * 16 + h) * VD + d] = o;
+      if (d == 0) { p.sp2_ml[(base * 2 + 0) * 16 + h] = m; p.sp2_ml[(base * 2 + 1) * 16 + h] = l; }
+    }
+  };
+  if (nparts > 1) {
+    spill_part(1, w_first, NW - w_first);
+    __syncthreads();  // the slots are staging space again
+    uf.reset();
+    if (t >= 0) {
+      const int upb = Bs / UK;
+      uf.run(part * NW + wave, nparts * NW, nvalid * upb, 0, t,
+             [&](int u) { int slot = u / upb; return blk_s[slot] * Bs + (u - slot * upb) * UK; }, tab_s, page, kbase,
+             p.k_sr, vbase, p.v_sr);
+    }
+    uf.publish(part_m + wave * 16, part_l + wave * 16, reinterpret_cast<float*>(Vs_all + wave * SLOT));
+    __syncthreads();
+    spill_part(0, 0, NW);
+    if (part == 0 && p.sp_keep_p != nullptr) {  // the compressed branch's output, merged in the prologue
+#pragma unroll
+      for (int r = 0; r < OPT; r++) {
+        const int idx = tid + r * NT;
+        const int h = idx / VD, d = idx - h * VD;
+        if (h < G) p.cmp_tmp[(int64_t)b * p.co_st + (int64_t)(kh * G + h) * p.co_sh + d] = (bf16_t)ocmp_pre[r];
+      }
+    }
+    return;
+  }
   if (tid < 16) merge_weights(part_m + w_first * 16, part_l + w_first * 16, NW - w_first, 16, tid, p.scale_log2);
   __syncthreads();
   float o_swa_pre[OPT];
@@ -937,6 +984,52 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_slc_swa_kernel(NsaDecod
       }
       p.out[(int64_t)b * p.o_st + (int64_t)hq * p.o_sh + d] = (bf16_t)(o_cmp * s0 + o_slc * s1 + o_swa * s2);
     }
+  }
+}
+
+// grid (B, KH): merges the parts written by decode_slc_swa_kernel when it ran with several parts per (request, kv
+// head) and applies the gates -> final output (and the branch outputs on request)
+template <int VD>
+__global__ __launch_bounds__(256) void decode_split_final_kernel(NsaDecodeParams p) {
+  const int b = blockIdx.x, kh = blockIdx.y, tid = threadIdx.x;
+  const int G = p.G, S = p.slc_nsplit;
+  for (int idx = tid; idx < G * (VD / 4); idx += 256) {
+    const int h = idx / (VD / 4), d = (idx - h * (VD / 4)) * 4;
+    const int hq = kh * G + h;
+    f32x4 res[2];
+#pragma unroll
+    for (int br = 0; br < 2; br++) {
+      const int64_t base0 = (((int64_t)b * p.KH + kh) * S) * 2 + br;
+      float m = NSA_NEG_INF;
+      for (int s2 = 0; s2 < S; s2++) m = fmaxf(m, p.sp2_ml[((base0 + s2 * 2) * 2 + 0) * 16 + h]);
+      float l = 0.f;
+      f32x4 o = {0.f, 0.f, 0.f, 0.f};
+      if (m != NSA_NEG_INF) {
+        for (int s2 = 0; s2 < S; s2++) {
+          const int64_t base = base0 + s2 * 2;
+          const float ms = p.sp2_ml[(base * 2 + 0) * 16 + h];
+          const float a = (ms == NSA_NEG_INF) ? 0.f : fast_exp2((ms - m) * p.scale_log2);
+          l += a * p.sp2_ml[(base * 2 + 1) * 16 + h];
+          const f32x4 x = *reinterpret_cast<const f32x4*>(p.sp2_o + (base * 16 + h) * VD + d);
+          o[0] += a * x[0]; o[1] += a * x[1]; o[2] += a * x[2]; o[3] += a * x[3];
+        }
+      }
+      const float inv = l > 0.f ? 1.f / l : 0.f;
+      // branch outputs are rounded to bf16 before the gated sum, as the other decode paths store them
+      res[br] = round_bf16x4(f32x4{o[0] * inv, o[1] * inv, o[2] * inv, o[3] * inv});
+    }
+    const int64_t co = (int64_t)b * p.co_st + (int64_t)hq * p.co_sh + d;
+    if (p.slc_o) *reinterpret_cast<bf16x4*>(p.slc_o + co) = pack4(res[0][0], res[0][1], res[0][2], res[0][3]);
+    if (p.swa_o) *reinterpret_cast<bf16x4*>(p.swa_o + co) = pack4(res[1][0], res[1][1], res[1][2], res[1][3]);
+    const bf16x4 c4 = *reinterpret_cast<const bf16x4*>(p.cmp_tmp + co);
+    if (p.cmp_o) *reinterpret_cast<bf16x4*>(p.cmp_o + co) = c4;
+    const bf16_t* wp = p.w + (int64_t)b * p.w_st + (int64_t)hq * p.w_sh;
+    const float s0 = 1.f / (1.f + __expf(-(float)wp[0]));
+    const float s1 = 1.f / (1.f + __expf(-(float)wp[1]));
+    const float s2g = 1.f / (1.f + __expf(-(float)wp[2]));
+    *reinterpret_cast<bf16x4*>(p.out + (int64_t)b * p.o_st + (int64_t)hq * p.o_sh + d) =
+        pack4((float)c4[0] * s0 + res[0][0] * s1 + res[1][0] * s2g, (float)c4[1] * s0 + res[0][1] * s1 + res[1][1] * s2g,
+              (float)c4[2] * s0 + res[0][2] * s1 + res[1][2] * s2g, (float)c4[3] * s0 + res[0][3] * s1 + res[1][3] * s2g);
   }
 }
 
@@ -1124,7 +1217,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_fused_kernel(NsaDecodeP
   if (wave == 0) {
     const int result = select_blocks_wave(imp, t, p.nb_cap, p, lane, cand_v, cand_i);
     blk_s[lane] = lane < nvalid ? max(result, 0) : 0;
-    if (p.topk && lane < p.top_n) p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + lane] = result;
+    if (p.topk && part == 0 && lane < p.top_n) p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + lane] = result;
   } else {
     if (t >= 0)
       uf.template run<PREFETCH_SWA>(wave - 1, NW - 1, swa_nu, swa_klo, t, swa_key, tab_s, page, kbase, p.k_sr, vbase,
@@ -1286,7 +1379,8 @@ int nsa_decode_split_launch(const NsaDecodeParams& p, int B, int D, int VD, hipS
                   "not fit the final kernel's LDS", D, VD, p.y_cap, p.nb_cap, p.table_stride);
     return NSA_ERR_UNSUPPORTED;
   }
-  dim3 grid1(B, p.KH, p.nsplit), grid2(B, p.KH);
+  const int S = p.slc_nsplit > 1 ? p.slc_nsplit : 1;
+  dim3 grid1(B, p.KH, p.nsplit), grid2(B, p.KH, S);
   const int ntab = (p.y_cap + p.page_size - 1) / p.page_size;
   const size_t dyn1 = (size_t)SPLIT_WAVES * (D == 128 ? UnitFlash<128, 128>::SLOT : UnitFlash<64, 64>::SLOT) * 2 +
                       (size_t)(2 * SPLIT_WAVES * 16 + ntab) * 4;
@@ -1294,14 +1388,20 @@ int nsa_decode_split_launch(const NsaDecodeParams& p, int B, int D, int VD, hipS
     decode_cmp_partial_kernel<128, 128><<<grid1, SPLIT_WAVES * 64, dyn1, stream>>>(p);
     int rc = nsa_check_launch("decode_cmp_partial_kernel");
     if (rc) return rc;
-    return launch_dyn(decode_slc_swa_kernel<128, 128>, grid2, (size_t)lds2, p, stream, "decode_slc_swa_kernel",
-                      SLC_SWA_STATIC_LDS);
+    rc = launch_dyn(decode_slc_swa_kernel<128, 128>, grid2, (size_t)lds2, p, stream, "decode_slc_swa_kernel",
+                    SLC_SWA_STATIC_LDS);
+    if (rc || S == 1) return rc;
+    decode_split_final_kernel<128><<<dim3(B, p.KH), 256, 0, stream>>>(p);
+    return nsa_check_launch("decode_split_final_kernel");
   }
   decode_cmp_partial_kernel<64, 64><<<grid1, SPLIT_WAVES * 64, dyn1, stream>>>(p);
   int rc = nsa_check_launch("decode_cmp_partial_kernel");
   if (rc) return rc;
-  return launch_dyn(decode_slc_swa_kernel<64, 64>, grid2, (size_t)lds2, p, stream, "decode_slc_swa_kernel",
-                    SLC_SWA_STATIC_LDS);
+  rc = launch_dyn(decode_slc_swa_kernel<64, 64>, grid2, (size_t)lds2, p, stream, "decode_slc_swa_kernel",
+                  SLC_SWA_STATIC_LDS);
+  if (rc || S == 1) return rc;
+  decode_split_final_kernel<64><<<dim3(B, p.KH), 256, 0, stream>>>(p);
+  return nsa_check_launch("decode_split_final_kernel");
 }
 
 // LDS of the one-launch decode kernel; 0 when it does not fit (the caller then takes the two-launch path)

@@ -57,7 +57,9 @@ def auto_cmp_splits(batch, num_kv_heads, fixed_y_maxlen, num_cus=256, one_launch
       38 / 39 / 40 / 39, 8 x 32K 54 / 59 / 58 / 55, 16 x 32K 61 / 62 / 62 / 65 -- parts pay for up to 16 (request,
       kv head) pairs and then only with 8 of them; short contexts in a large capacity lose 1-2 us to them;
       capacity 8192 rows (two launches without parts): 8 x 64K 105 / 72 / 68 / 64, 16 x 64K 114 / 80 / 77 / 80,
-      16 x 128K 192 / 127 / 114 / 114, 32 x 64K 140 / 111 / 119 / 126, 32 x 128K 240 / 185 / 188 / 191."""
+      16 x 128K 192 / 127 / 114 / 114, 32 x 64K 140 / 111 / 119 / 126, 32 x 128K 240 / 185 / 188 / 191;
+      8 / 16 / 32 / 64 parts: 1 x 128K 61.3 / 58.8 / 61.1 / 69.1, 2 x 128K 64.8 / 62.7 / 65.9 / 76.8, 4 x 128K
+      67.9 / 68.3 / 76.7 / 89.6 -- 16 parts pay for up to 8 pairs."""
     pairs = batch * num_kv_heads
     if fixed_y_maxlen < 1024:
         return 1
@@ -66,6 +68,8 @@ def auto_cmp_splits(batch, num_kv_heads, fixed_y_maxlen, num_cus=256, one_launch
     scale = num_cus / 256.0
     if one_launch_fits:
         return 8 if pairs <= 16 * scale else 1
+    if pairs <= 8 * scale and fixed_y_maxlen >= 8192:
+        return 16
     if pairs <= 32 * scale:
         return 8
     if pairs <= 64 * scale:
@@ -122,7 +126,8 @@ def nsa_decode(q, k, v, w, context_lens, block_tables, cmp_slot_mapping, cmp_blo
                             fixed_y_maxlen=fixed_y_maxlen, fixed_num_slc_blocks=fixed_num_slc_blocks,
                             kernel_size=kernel_size, stride=stride, block_size=block_size, top_n=top_n,
                             num_inital=num_init_blocks, num_local=num_local_blocks, window_size=window_size,
-                            sm_scale=sm_scale, cmp_slot_mapping=cmp_slot_mapping if fuse_pool else None)
+                            sm_scale=sm_scale, cmp_slot_mapping=cmp_slot_mapping if fuse_pool else None,
+                            slc_nsplit=max(1, min(int(slc_num_splits), 16)))
     kv_mean_pooling_decode(k, v, block_table=block_tables, slot_mapping=cmp_slot_mapping, context_lens=context_lens,
                            kernel_size=kernel_size, stride=stride)
     if fused_decode_supported(q, k, v):

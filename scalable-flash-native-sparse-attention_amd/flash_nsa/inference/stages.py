@@ -335,7 +335,7 @@ def decode_split_fits(q, k, v, block_tables, fixed_y_maxlen, fixed_num_slc_block
 def decode_split(q, k, v, w, block_tables, cmp_block_tables, context_lens, nsplit=4, fixed_y_maxlen=8192,
                  fixed_num_slc_blocks=2048, kernel_size=32, stride=16, block_size=64, top_n=16, num_inital=1,
                  num_local=2, window_size=512, sm_scale=None, return_parts=False, cmp_slot_mapping=None,
-                 static_scratch=False):
+                 static_scratch=False, slc_nsplit=1):
     """The decode step in two launches, for small batches of long contexts: the compressed branch cut into `nsplit`
     parts per (request, kv head) so that it fills the GPU, then one workgroup per pair for the merge, the block
     selection, selected + window attention and the gated combine.  -> o [B,QH,VD]
@@ -343,7 +343,10 @@ def decode_split(q, k, v, w, block_tables, cmp_block_tables, context_lens, nspli
     cmp_slot_mapping [B] (-1: none): the first launch also pools the compressed row that the newest token completes;
     None: that row is in the pool already.
     static_scratch: the library's own static device buffer holds the parts' partial results (entry point
-    nsa_decode_split_static, which allocates nothing); sizes beyond that buffer raise."""
+    nsa_decode_split_static, which allocates nothing); sizes beyond that buffer raise.
+    slc_nsplit > 1: the second launch runs with that many workgroups per (request, kv head), which share the window
+    and the selected blocks, and a third launch merges them (upstream's slc_num_splits,
+    flash_nsa/inference/__init__.py:195-196)."""
     check_bf16(q)
     page, KH, D, ksr, ksh = _pool_args(k)
     _, _, VD, vsr, vsh = _pool_args(v)
@@ -374,16 +377,25 @@ def decode_split(q, k, v, w, block_tables, cmp_block_tables, context_lens, nspli
     sp_o = torch.empty(B, KH, nsplit, 16, VD, device=dev, dtype=torch.float32)
     keep_p = torch.empty(B, KH, 16, ycap32, device=dev, dtype=torch.float16)
     keep_m = torch.empty(B, KH, ycap32 // 32, 16, device=dev, dtype=torch.float32)
-    _lib.call("nsa_decode_split", q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), ksr, ksh, v.data_ptr(), vsr,
-              vsh, w.data_ptr(), w.stride(0), w.stride(1), out.data_ptr(), out.stride(0), out.stride(1),
-              _lib.ptr(parts[0]), _lib.ptr(parts[1]), _lib.ptr(parts[2]), out.stride(0), out.stride(1),
-              _lib.ptr(lse), lse.stride(0) if return_parts else 0, lse.stride(1) if return_parts else 0,
-              _lib.ptr(topk), topk.stride(0) if return_parts else 0, topk.stride(1) if return_parts else 0,
-              sp_ml[0].data_ptr(), sp_ml[1].data_ptr(), sp_o.data_ptr(), keep_p.data_ptr(), keep_m.data_ptr(), nsplit,
-              _lib.ptr(None if cmp_slot_mapping is None else _i32(cmp_slot_mapping)), _i32(context_lens).data_ptr(), _i32(block_tables).data_ptr(), block_tables.stride(0),
-              _i32(cmp_block_tables).data_ptr(), cmp_block_tables.stride(0), page, B, QH, KH, D, VD,
-              int(fixed_y_maxlen), int(fixed_num_slc_blocks), kernel_size, stride, block_size, top_n, num_inital,
-              num_local, -1, window_size, sm_scale, _lib.stream_ptr())
+    args = (q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), ksr, ksh, v.data_ptr(), vsr,
+            vsh, w.data_ptr(), w.stride(0), w.stride(1), out.data_ptr(), out.stride(0), out.stride(1),
+            _lib.ptr(parts[0]), _lib.ptr(parts[1]), _lib.ptr(parts[2]), out.stride(0), out.stride(1),
+            _lib.ptr(lse), lse.stride(0) if return_parts else 0, lse.stride(1) if return_parts else 0,
+            _lib.ptr(topk), topk.stride(0) if return_parts else 0, topk.stride(1) if return_parts else 0,
+            sp_ml[0].data_ptr(), sp_ml[1].data_ptr(), sp_o.data_ptr(), keep_p.data_ptr(), keep_m.data_ptr(), nsplit,
+            _lib.ptr(None if cmp_slot_mapping is None else _i32(cmp_slot_mapping)), _i32(context_lens).data_ptr(),
+            _i32(block_tables).data_ptr(), block_tables.stride(0),
+            _i32(cmp_block_tables).data_ptr(), cmp_block_tables.stride(0), page, B, QH, KH, D, VD,
+            int(fixed_y_maxlen), int(fixed_num_slc_blocks), kernel_size, stride, block_size, top_n, num_inital,
+            num_local, -1, window_size, sm_scale)
+    if slc_nsplit > 1:
+        sp2_ml = torch.empty(B, KH, slc_nsplit, 2, 2, 16, device=dev, dtype=torch.float32)
+        sp2_o = torch.empty(B, KH, slc_nsplit, 2, 16, VD, device=dev, dtype=torch.float32)
+        cmp_tmp = torch.empty_like(out)
+        _lib.call("nsa_decode_split_parts", *args, int(slc_nsplit), sp2_ml.data_ptr(), sp2_o.data_ptr(),
+                  cmp_tmp.data_ptr(), _lib.stream_ptr())
+    else:
+        _lib.call("nsa_decode_split", *args, _lib.stream_ptr())
     if return_parts:
         return out, parts[0], parts[1], parts[2], topk, lse
     return out

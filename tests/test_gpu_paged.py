@@ -538,6 +538,37 @@ def test_split_decode_matches_one_launch(device, QH, KH, D, nsplit):
     assert torch.equal(out, out2), "optional outputs must not change the result"
 
 
+@pytest.mark.parametrize("QH,KH,D", [(64, 4, 128), (12, 2, 64)])
+@pytest.mark.parametrize("slc_nsplit", [2, 3, 4])
+def test_split_decode_with_window_and_selected_blocks_in_parts(device, QH, KH, D, slc_nsplit):
+    """slc_nsplit workgroups per (request, kv head) share the window units and the selected blocks and a third
+    launch merges them: the selection and lse are those of the uncut second launch bit for bit (the prologue is the
+    same code on the same data), the branch outputs and the output agree to bf16 rounding (the merge sums the same
+    partial results in another order)."""
+    from flash_nsa.inference import decode_split
+    ctx = [4096, 333, 48, 31, 1, 777, 2999, 640, 1024, 65, 0, 513, 514]
+    case = build_pool([max(c, 1) for c in ctx], KH, D, D, page=128, seed=61)
+    prepool(case, [max(c, 1) for c in ctx])
+    B = len(ctx)
+    d = to_dev(case, device)
+    q = randn_bf16(B, QH, D, seed=62).to(device)
+    w = randn_bf16(B, QH, 3, seed=63).to(device)
+    ctx_t = torch.tensor(ctx, dtype=torch.int32, device=device)
+    kw = dict(nsplit=3, fixed_y_maxlen=512, fixed_num_slc_blocks=64, top_n=8, window_size=200)
+    ref = decode_split(q, d["k"], d["v"], w, d["bt"], d["cbt"], ctx_t, return_parts=True, **kw)
+    got = decode_split(q, d["k"], d["v"], w, d["bt"], d["cbt"], ctx_t, return_parts=True, slc_nsplit=slc_nsplit, **kw)
+    live = ctx_t > 0
+    assert torch.equal(got[4][:, live], ref[4][:, live]), "selection"
+    assert torch.equal(got[5][live], ref[5][live]), "lse"
+    assert torch.equal(got[1][live], ref[1][live]), "cmp_o"
+    assert_close(got[2][live], ref[2][live], "slc_o", atol=4e-3, rtol=1e-2)
+    assert_close(got[3][live], ref[3][live], "swa_o", atol=4e-3, rtol=1e-2)
+    assert_close(got[0][live], ref[0][live], "o", atol=8e-3, rtol=1e-2)
+    assert float(got[0][~live].abs().max()) == 0.0, "a padded request (context 0) must give zeros"
+    out2 = decode_split(q, d["k"], d["v"], w, d["bt"], d["cbt"], ctx_t, slc_nsplit=slc_nsplit, **kw)
+    assert torch.equal(got[0], out2), "optional outputs must not change the result"
+
+
 def test_one_launch_decode_pools_the_new_row_itself(device):
     """nsa_decode's one-launch kernel with a slot mapping == pooling kernel followed by the same kernel without:
     the pools end bit-identical and so do the outputs."""

@@ -127,7 +127,9 @@ def test_decode_picks_parts_only_for_small_batches_of_long_contexts():
     assert auto_cmp_splits(32, 4, 4096) == 2
     assert auto_cmp_splits(16, 4, 8192) == 4
     assert auto_cmp_splits(8, 4, 8192) == 8
-    assert auto_cmp_splits(1, 1, 8192) == 8           # never more than 8
+    assert auto_cmp_splits(1, 1, 8192) == 16          # 16 only for a handful of pairs at a large capacity
+    assert auto_cmp_splits(2, 4, 8192) == 16 and auto_cmp_splits(3, 4, 8192) == 8
+    assert auto_cmp_splits(1, 4, 4096) == 8
     assert auto_cmp_splits(1, 1, 2048) == 8           # 32K tokens of capacity: worth the second launch
     assert auto_cmp_splits(4, 4, 2048) == 8 and auto_cmp_splits(5, 4, 2048) == 1   # ... for up to 16 pairs
     assert auto_cmp_splits(8, 4, 2048) == 1 and auto_cmp_splits(8, 4, 2048, one_launch_fits=False) == 8
