@@ -1217,7 +1217,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_fused_kernel(NsaDecodeP
   if (wave == 0) {
     const int result = select_blocks_wave(imp, t, p.nb_cap, p, lane, cand_v, cand_i);
     blk_s[lane] = lane < nvalid ? max(result, 0) : 0;
-    if (p.topk && part == 0 && lane < p.top_n) p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + lane] = result;
+    if (p.topk && lane < p.top_n) p.topk[(int64_t)kh * p.tk_sh + (int64_t)b * p.tk_st + lane] = result;
   } else {
     if (t >= 0)
       uf.template run<PREFETCH_SWA>(wave - 1, NW - 1, swa_nu, swa_klo, t, swa_key, tab_s, page, kbase, p.k_sr, vbase,
