@@ -13,6 +13,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 typedef __bf16 bf16_t;
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -91,6 +92,18 @@ NSA_DEVICE float xhalf_max(float v) {
 NSA_DEVICE float xhalf_sum(float v) {
   uint32_t b = __builtin_bit_cast(uint32_t, v);
   auto r = __builtin_amdgcn_permlane32_swap(b, b, false, false);
+  return __builtin_bit_cast(float, (uint32_t)r[0]) + __builtin_bit_cast(float, (uint32_t)r[1]);
+}
+
+// exchange between neighbouring 16-lane rows (lane l <-> lane l ^ 16) on the VALU (v_permlane16_swap)
+NSA_DEVICE float xrow_max(float v) {
+  uint32_t b = __builtin_bit_cast(uint32_t, v);
+  auto r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+  return fmaxf(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1]));
+}
+NSA_DEVICE float xrow_sum(float v) {
+  uint32_t b = __builtin_bit_cast(uint32_t, v);
+  auto r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
   return __builtin_bit_cast(float, (uint32_t)r[0]) + __builtin_bit_cast(float, (uint32_t)r[1]);
 }
 

@@ -158,7 +158,7 @@ struct UnitFlash {
     }
     float tmax = fmaxf(fmaxf(fmaxf(sacc[0][0], sacc[0][1]), fmaxf(sacc[0][2], sacc[0][3])),
                        fmaxf(fmaxf(sacc[1][0], sacc[1][1]), fmaxf(sacc[1][2], sacc[1][3])));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = xrow_max(tmax);
     tmax = xhalf_max(tmax);
     const float m_old = m_run;
     const float m_new = fmaxf(m_old, tmax);
@@ -251,7 +251,7 @@ struct UnitFlash {
   }
   // wave partial -> LDS slot: m (raw units), l, o[16 heads][VD]
   NSA_DEVICE void publish(float* pm, float* pl, float* po) {
-    float l_tot = l_run + __shfl_xor(l_run, 16, 64);
+    float l_tot = xrow_sum(l_run);
     l_tot = xhalf_sum(l_tot);
     if (kq == 0) { pm[l16] = m_run; pl[l16] = l_tot; }
 #pragma unroll

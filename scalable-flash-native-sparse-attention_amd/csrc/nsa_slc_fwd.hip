@@ -153,8 +153,8 @@ __global__ __launch_bounds__(256, 2) void slc_fwd_kernel(NsaSlcParams p) {
     }
     float tmax = fmaxf(fmaxf(fmaxf(sacc[0][0], sacc[0][1]), fmaxf(sacc[0][2], sacc[0][3])),
                        fmaxf(fmaxf(sacc[1][0], sacc[1][1]), fmaxf(sacc[1][2], sacc[1][3])));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    tmax = xrow_max(tmax);
+    tmax = xhalf_max(tmax);
     const float m_old = m_run;
     const float m_new = fmaxf(m_old, tmax);
     const float m_safe = (m_new == NSA_NEG_INF) ? 0.f : m_new;
@@ -206,8 +206,8 @@ __global__ __launch_bounds__(256, 2) void slc_fwd_kernel(NsaSlcParams p) {
     }
   }
 
-  float l_tot = l_run + __shfl_xor(l_run, 16, 64);
-  l_tot += __shfl_xor(l_tot, 32, 64);
+  float l_tot = xrow_sum(l_run);
+  l_tot = xhalf_sum(l_tot);
   if (!head_ok) return;
   float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   bf16_t* op = p.o + tok * p.o_st + (int64_t)head * p.o_sh + kq * 4;
