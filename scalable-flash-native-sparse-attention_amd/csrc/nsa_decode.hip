@@ -528,8 +528,8 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void decode_cmp_topk_kernel(NsaDeco
 #pragma unroll
         for (int i = 0; i < 4; i++)
           if (kq * 4 + i < G) acc += fast_exp2(__builtin_fmaf(s[i], p.scale_log2, -lse4[i]));
-        acc += __shfl_xor(acc, 16, 64);
-        acc += __shfl_xor(acc, 32, 64);
+        acc = xrow_sum(acc);
+        acc = xhalf_sum(acc);
         int key = key0 + jt * 16 + l16;
         if (kq == 0 && key < y) pg[key] = acc;
       }
@@ -727,8 +727,8 @@ __global__ __launch_bounds__(SPLIT_WAVES * 64) void decode_importance_kernel(Nsa
 #pragma unroll
       for (int i = 0; i < 4; i++)
         if (kq * 4 + i < G) acc += fast_exp2(__builtin_fmaf(sv[i], p.scale_log2, -lse4[i]));
-      acc += __shfl_xor(acc, 16, 64);
-      acc += __shfl_xor(acc, 32, 64);
+      acc = xrow_sum(acc);
+      acc = xhalf_sum(acc);
       int key = u * UK + jt * 16 + l16;
       if (kq == 0 && key < y) pg[key] = acc;
     }

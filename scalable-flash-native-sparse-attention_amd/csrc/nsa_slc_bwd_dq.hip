@@ -66,7 +66,7 @@ __global__ __launch_bounds__(256, 2) void slc_dq_kernel(NsaSlcBwdDqParams p) {
 
   auto unit_key0 = [&](int u) {  // wave-uniform; -1: nothing to attend in this unit
     int slot = u / upb;
-    int blk = __builtin_amdgcn_readfirstlane(__shfl(my_blk, slot, 64));
+    int blk = __builtin_amdgcn_readlane(my_blk, slot);
     int key0 = blk * Bs + (u - slot * upb) * UK;
     return (blk < 0 || key0 > key_last) ? -1 : key0;
   };

@@ -73,7 +73,7 @@ __global__ __launch_bounds__(256, 2) void slc_fwd_kernel(NsaSlcParams p) {
   // block) and ignore values (negative ids) are reported as -1 and skipped.
   auto unit_key0 = [&](int u) {
     int slot = u / upb;
-    int blk = __builtin_amdgcn_readfirstlane(__shfl(my_blk, slot, 64));
+    int blk = __builtin_amdgcn_readlane(my_blk, slot);
     int key0 = blk * Bs + (u - slot * upb) * UK;
     return (blk < 0 || key0 > key_last) ? -1 : key0;
   };
