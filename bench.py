@@ -160,6 +160,42 @@ def staged_step(timer, q, k, v, w, wv, do, sm_scale):
     R("cmp_v_bwd", cmp_v_bwd)
 
 
+def selected_attention_floor(q, k, v, do, KH, reps=3):
+    """Extra, not part of `value`: the selected-attention forward and dQ kernels on two synthetic selection patterns
+    of the benchmark shape -- `random` (3 forced blocks + 13 uniformly random earlier blocks per token and kv head:
+    what random q / k select, bound by the L2-miss path) and `clustered` (the 13 free blocks drawn from the 64
+    nearest: K/V stay in cache, which shows the kernels' own floor).  Milliseconds per launch."""
+    import torch
+    from flash_nsa.ops.select_attn import slc_attn_fwd, slc_attn_bwd
+    T, QH, D = q.shape
+    dev = q.device
+    g = torch.Generator(device=dev).manual_seed(7)
+    cur = torch.arange(T, device=dev) // 64
+    forced = torch.stack([torch.zeros_like(cur), cur, cur - 1], -1)[None].expand(KH, T, 3)
+
+    def timed(fn):
+        fn()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(reps):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        return s.elapsed_time(e) / reps
+
+    out = {}
+    for name in ("random", "clustered"):
+        u = torch.rand(KH, T, 13, generator=g, device=dev)
+        free = (u * (cur + 1)[None, :, None]).long() if name == "random" else cur[None, :, None] - (u * 64).long()
+        topk = torch.cat([forced, free], -1).clamp_(min=0).to(torch.int32).contiguous()
+        o, lse = slc_attn_fwd(q, k, v, topk)
+        dq = torch.zeros(T, QH, D, device=dev, dtype=torch.float32)
+        out[name] = {"slc_fwd_ms": round(timed(lambda: slc_attn_fwd(q, k, v, topk)), 3),
+                     "slc_dq_ms": round(timed(lambda: slc_attn_bwd(q, k, v, topk, o, lse, do, dq=dq, parts="dq")), 3)}
+    return out
+
+
 def layer_bench(dev, T, QH, KH, D, reps=20):
     """The step either side of the core: the fused rotary embedding of q and k at the headline shape (an HBM-bound
     kernel: q and k read and written once, the fp32 tables read once), and, for scale, forward+backward of the whole
@@ -441,6 +477,9 @@ def main():
         result["ms_per_step_deterministic"] = (time.perf_counter() - t0) * 1e3 / args.steps
     finally:
         NSAHelper.set_deterministic(False)
+    with torch.no_grad():
+        result["selected_attention_by_selection_pattern"] = selected_attention_floor(q.detach(), k.detach(),
+                                                                                     v.detach(), do, KH)
     if traffic is not None:
         # the selected-block kernels re-read K/V blocks that fall out of the 4 MB L2 slices: their launch time is
         # set by this memory-side rate rather than by the MFMA work
