@@ -24,7 +24,7 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 # what the same counter reads for a 1 GiB copy: x2.000 and x1.000), measured on the T=65536 workload of this file;
 # reported as roofline.traffic for that workload only.
 MEASURED_TRAFFIC_T64K = {
-    "cmp_dkdv": 34.40e9, "slc_dq": 75.55e9, "slc_fwd": 73.02e9, "slc_dkdv": 36.38e9, "cmp_dq": 7.21e9,
+    "cmp_dkdv": 34.26e9, "slc_dq": 75.58e9, "slc_fwd": 73.54e9, "slc_dkdv": 36.38e9, "cmp_dq": 7.21e9,
     "topk": 2.30e9, "cmp_fwd": 2.25e9, "swa_dkdv": 11.39e9, "swa_dq": 6.54e9, "swa_fwd": 3.24e9,
 }
 PEAK_HBM_GBS = 8000.0
@@ -360,6 +360,9 @@ def main():
                     help="run only this leg of the decode benchmark (for kernel traces that should reproduce one "
                          "reported figure)")
     ap.add_argument("--decode-only", action="store_true", help="skip the training step (with --decode-leg)")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the labelled extras that launch the step's kernels on other inputs (for kernel traces "
+                         "and counter runs, whose per-kernel averages should cover the benchmark step only)")
     ap.add_argument("--sweep", type=str, default=None,
                     help="comma-separated sequence lengths: print forward / backward times per length and exit")
     args = ap.parse_args()
@@ -477,9 +480,10 @@ def main():
         result["ms_per_step_deterministic"] = (time.perf_counter() - t0) * 1e3 / args.steps
     finally:
         NSAHelper.set_deterministic(False)
-    with torch.no_grad():
-        result["selected_attention_by_selection_pattern"] = selected_attention_floor(q.detach(), k.detach(),
-                                                                                     v.detach(), do, KH)
+    if not args.no_extras:
+        with torch.no_grad():
+            result["selected_attention_by_selection_pattern"] = selected_attention_floor(q.detach(), k.detach(),
+                                                                                         v.detach(), do, KH)
     if traffic is not None:
         # the selected-block kernels re-read K/V blocks that fall out of the 4 MB L2 slices: their launch time is
         # set by this memory-side rate rather than by the MFMA work
