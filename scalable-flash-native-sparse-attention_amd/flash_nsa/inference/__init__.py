@@ -86,6 +86,10 @@ def nsa_decode(q, k, v, w, context_lens, block_tables, cmp_slot_mapping, cmp_blo
     """One query token per request.  q [B,QH,D]; w [B,QH,3]; cmp_slot_mapping [B] (-1: no compressed row completes
     at this step).  Rows with context_lens == 0 (graph padding) produce zeros.  Returns o [B,QH,VD].
     cmp_num_splits: 0 = chosen from the batch size and fixed_y_maxlen (auto_cmp_splits), 1 = never split.
+    slc_num_splits (upstream flash_nsa/inference/__init__.py:195-196): > 1 cuts the window and selected blocks of a
+    request over that many workgroups; honoured where the compressed branch is cut as well (the two-launch path for
+    small batches of long contexts, plus a merging launch), ignored by the one-launch kernel, whose batches fill the
+    GPU without it.  Measured, it does not pay on MI355X (one request of 128K tokens: 61.5 us with or without).
     As upstream, the newest token's K/V are expected in the pools already; alternatively pass them as new_k / new_v
     [B,KH,*] with their flat pool rows slot_mapping [B] (-1: padding) and the cache write happens here (inside the
     single decode launch when that path is taken)."""
