@@ -358,6 +358,9 @@ def decode_split(q, k, v, w, block_tables, cmp_block_tables, context_lens, nspli
     topk = torch.empty(KH, B, top_n, device=dev, dtype=torch.int32) if return_parts else None
     lse = torch.empty(B, QH, device=dev, dtype=torch.float32) if return_parts else None
     if static_scratch:
+        if slc_nsplit > 1:
+            raise ValueError("decode_split: the static-scratch entry point has no parts of the window / selected "
+                             "branches (slc_nsplit must be 1)")
         _lib.call("nsa_decode_split_static", q.data_ptr(), q.stride(0), q.stride(1), k.data_ptr(), ksr, ksh,
                   v.data_ptr(), vsr, vsh, w.data_ptr(), w.stride(0), w.stride(1), out.data_ptr(), out.stride(0),
                   out.stride(1), _lib.ptr(parts[0]), _lib.ptr(parts[1]), _lib.ptr(parts[2]), out.stride(0),
