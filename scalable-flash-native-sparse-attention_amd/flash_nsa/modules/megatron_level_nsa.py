@@ -147,8 +147,9 @@ class NSAFunction(torch.autograd.Function):
                                         finalize_dq=True, parts="dq", **kw)
                 dq.record_stream(main)
             # dk/dv kernels on the caller's stream.  The compressed branch (matrix bound) goes first, next to the
-            # selected dq kernel (bound by the gather path) on the other stream: 67.2 -> 65.5 ms per step at T = 64K
-            # against the order window, selected, compressed, which ran the two selected kernels side by side.  The
+            # selected dq kernel (bound by the gather path) on the other stream: 0.7-1.7 ms per step less at T = 64K
+            # (67.7 -> 67.0 and 67.2 -> 65.5 ms on two GPUs) than the order window, selected, compressed, which ran the
+            # two selected kernels side by side.  The
             # window branch writes every element of dk / dv, the selected branch then adds to them.
             _, dcmp_k, dcmp_v = cmp_attn_bwd(q, cmp_k, cmp_v, cmp_o, cmp_lse, dcmp_o, delta=delta[0], parts="dkdv",
                                              **kw)
